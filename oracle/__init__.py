@@ -1,0 +1,327 @@
+"""ctypes front-end of the CPU oracle (``monarch_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py``.  The product package never imports this module.
+All arrays are numpy arrays on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from typing import List, Sequence, Tuple
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libmonarch_oracle.so")
+
+ERR_NAMES = {
+    0: "Ok",
+    1: "InvalidDims",
+    2: "NonrectangularShape",
+    3: "NonuniqueStrides",
+    4: "StrideTooSmall",
+    5: "IndexOutOfRange",
+    6: "ValueNotInSlice",
+    7: "IncompatibleView",
+    8: "NonContiguous",
+    9: "EmptyRange",
+    10: "DimensionOutOfRange",
+}
+
+
+def build(force: bool = False) -> str:
+    src = os.path.join(_HERE, "monarch_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "libmonarch_oracle.so"],
+                              stdout=subprocess.DEVNULL)
+    return _SO
+
+
+class OracleError(Exception):
+    def __init__(self, code: int):
+        super().__init__(ERR_NAMES.get(code, str(code)))
+        self.code = code
+        self.name = ERR_NAMES.get(code, str(code))
+
+
+class _CSlice(C.Structure):
+    _fields_ = [("offset", C.c_uint64), ("ndim", C.c_uint32),
+                ("sizes", C.POINTER(C.c_uint64)), ("strides", C.POINTER(C.c_uint64))]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_SO)
+        _lib.o_slice_len.restype = C.c_uint64
+        _lib.o_slice_iter.restype = C.c_uint64
+        _lib.o_mesh_ranks_for_dims.restype = C.c_int64
+        _lib.o_e4m3fn_encode.restype = C.c_uint8
+        _lib.o_e4m3fn_encode.argtypes = [C.c_float, C.c_int]
+        _lib.o_e4m3fn_decode.restype = C.c_float
+        _lib.o_e4m3fn_decode.argtypes = [C.c_uint8]
+    return _lib
+
+
+def _u64(xs: Sequence[int]):
+    return (C.c_uint64 * max(1, len(xs)))(*xs)
+
+
+class OSlice:
+    """Restatement of ``ndslice::Slice``; ``OSlice(...)`` validates like ``Slice::new``,
+    ``OSlice.unchecked(...)`` constructs like ``new_row_major``/``subview`` do."""
+
+    def __init__(self, offset: int, sizes: Sequence[int], strides: Sequence[int], _validate=True):
+        self.offset, self.sizes, self.strides = int(offset), list(sizes), list(strides)
+        if _validate:
+            rc = lib().o_slice_new(C.c_uint64(self.offset), _u64(self.sizes), C.c_uint32(len(self.sizes)),
+                                   _u64(self.strides), C.c_uint32(len(self.strides)))
+            if rc:
+                raise OracleError(rc)
+        self._keep = (_u64(self.sizes), _u64(self.strides))
+        self.c = _CSlice(self.offset, len(self.sizes), self._keep[0], self._keep[1])
+
+    @classmethod
+    def unchecked(cls, offset, sizes, strides):
+        return cls(offset, sizes, strides, _validate=False)
+
+    @classmethod
+    def row_major(cls, sizes):
+        strides, acc = [], 1
+        for n in reversed(list(sizes)):
+            strides.append(acc)
+            acc *= n
+        return cls.unchecked(0, sizes, list(reversed(strides)))
+
+    def __repr__(self):
+        return f"OSlice(offset={self.offset}, sizes={self.sizes}, strides={self.strides})"
+
+    @property
+    def ndim(self):
+        return len(self.sizes)
+
+    def __len__(self):
+        return int(lib().o_slice_len(C.byref(self.c)))
+
+    def is_contiguous(self) -> bool:
+        return bool(lib().o_slice_is_contiguous(C.byref(self.c)))
+
+    def get(self, i: int) -> int:
+        out = C.c_uint64()
+        rc = lib().o_slice_get(C.byref(self.c), C.c_uint64(i), C.byref(out))
+        if rc:
+            raise OracleError(rc)
+        return out.value
+
+    def location(self, coord: Sequence[int]) -> int:
+        out = C.c_uint64()
+        rc = lib().o_slice_location(C.byref(self.c), _u64(coord), C.c_uint32(len(coord)), C.byref(out))
+        if rc:
+            raise OracleError(rc)
+        return out.value
+
+    def iter(self) -> np.ndarray:
+        n = len(self)
+        out = np.empty(max(n, 1), dtype=np.uint64)
+        lib().o_slice_iter(C.byref(self.c), out.ctypes.data_as(C.c_void_p), C.c_uint64(n))
+        return out[:n]
+
+    def coordinates(self, value: int) -> List[int]:
+        out = _u64([0] * self.ndim)
+        rc = lib().o_slice_coordinates(C.byref(self.c), C.c_uint64(value), out)
+        if rc:
+            raise OracleError(rc)
+        return list(out)[: self.ndim]
+
+    def index(self, value: int) -> int:
+        out = C.c_uint64()
+        rc = lib().o_slice_index(C.byref(self.c), C.c_uint64(value), C.byref(out))
+        if rc:
+            raise OracleError(rc)
+        return out.value
+
+    def contains(self, value: int) -> bool:
+        try:
+            self.coordinates(value)
+            return True
+        except OracleError:
+            return False
+
+    def select(self, dim, begin, end, step) -> "OSlice":
+        off = C.c_uint64()
+        sz, st = _u64([0] * self.ndim), _u64([0] * self.ndim)
+        rc = lib().o_slice_select(C.byref(self.c), C.c_uint32(dim), C.c_uint64(begin), C.c_uint64(end),
+                                  C.c_uint64(step), C.byref(off), sz, st)
+        if rc:
+            raise OracleError(rc)
+        return OSlice.unchecked(off.value, list(sz)[: self.ndim], list(st)[: self.ndim])
+
+    def at(self, dim, index) -> "OSlice":
+        off = C.c_uint64()
+        sz, st = _u64([0] * self.ndim), _u64([0] * self.ndim)
+        rc = lib().o_slice_at(C.byref(self.c), C.c_uint32(dim), C.c_uint64(index), C.byref(off), sz, st)
+        if rc:
+            raise OracleError(rc)
+        return OSlice.unchecked(off.value, list(sz)[: self.ndim - 1], list(st)[: self.ndim - 1])
+
+    def subview(self, starts, lens) -> "OSlice":
+        off = C.c_uint64()
+        rc = lib().o_slice_subview(C.byref(self.c), _u64(starts), C.c_uint32(len(starts)), _u64(lens),
+                                   C.c_uint32(len(lens)), C.byref(off))
+        if rc:
+            raise OracleError(rc)
+        return OSlice.unchecked(off.value, list(lens), list(self.strides))
+
+    def view(self, new_sizes) -> "OSlice":
+        st = _u64([0] * len(new_sizes))
+        rc = lib().o_slice_view(C.byref(self.c), _u64(new_sizes), C.c_uint32(len(new_sizes)), st)
+        if rc:
+            raise OracleError(rc)
+        return OSlice.unchecked(0, list(new_sizes), list(st)[: len(new_sizes)])
+
+    def enforce_embedding(self, other: "OSlice") -> "OSlice":
+        rc = lib().o_slice_enforce_embedding(C.byref(self.c), C.byref(other.c))
+        if rc:
+            raise OracleError(rc)
+        return self
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def pack(src_base: np.ndarray, s: OSlice, runs: bool = False) -> np.ndarray:
+    """dst[i] = src_base.flat[s.get(i)]; ``src_base`` is the flat storage."""
+    src_base = np.ascontiguousarray(src_base).reshape(-1)
+    dst = np.empty(len(s), dtype=src_base.dtype)
+    fn = lib().o_pack_runs if runs else lib().o_slice_pack
+    fn(_ptr(dst), _ptr(src_base), C.byref(s.c), C.c_uint32(src_base.itemsize))
+    return dst
+
+
+def unpack(dst_base: np.ndarray, src: np.ndarray, s: OSlice) -> None:
+    """dst_base.flat[s.get(i)] = src[i], in place on the flat storage ``dst_base``."""
+    assert dst_base.flags.c_contiguous and src.flags.c_contiguous and dst_base.dtype == src.dtype
+    lib().o_slice_unpack(_ptr(dst_base), _ptr(src), C.byref(s.c), C.c_uint32(src.itemsize))
+
+
+_REDUCE = {"float32": "o_reduce_f32", "float64": "o_reduce_f64", "uint16": "o_reduce_bf16",
+           "uint8": "o_reduce_u8", "int32": "o_reduce_i32", "int64": "o_reduce_i64"}
+
+SUM, AVG = 0, 4
+
+
+def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = None) -> np.ndarray:
+    """Elementwise Sum/Avg over ``ins``.  bf16 data is passed as uint16 bit patterns."""
+    ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
+    dt = ins[0].dtype
+    if out is None:
+        out = np.empty_like(ins[0])
+    ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+    name = _REDUCE[dt.name]
+    args = [_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint64(ins[0].size)]
+    if dt.name in ("float32", "float64", "uint16"):
+        args.append(C.c_int(op))
+    else:
+        assert op == SUM
+    getattr(lib(), name)(*args)
+    return out
+
+
+def reduce_scatter(ins: Sequence[np.ndarray], in_view: OSlice, out_views: Sequence[OSlice],
+                   op: int = SUM) -> List[np.ndarray]:
+    ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
+    dt = ins[0].dtype
+    outs = [np.empty(len(v), dtype=dt) for v in out_views]
+    views = (_CSlice * len(out_views))(*[v.c for v in out_views])
+    inp = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+    outp = (C.c_void_p * len(outs))(*[x.ctypes.data for x in outs])
+    fn = {"float32": lib().o_reduce_scatter_f32, "uint16": lib().o_reduce_scatter_bf16}[dt.name]
+    fn(outp, views, C.c_uint32(len(outs)), inp, C.byref(in_view.c), C.c_uint32(len(ins)), C.c_int(op))
+    return outs
+
+
+def bf16_to_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().o_bf16_to_f32(_ptr(out), _ptr(x), C.c_uint64(x.size))
+    return out
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().o_f32_to_bf16(_ptr(out), _ptr(x), C.c_uint64(x.size))
+    return out
+
+
+def mesh_dim_members(ranks: OSlice, rank: int, dim: int) -> Tuple[List[int], int]:
+    out = _u64([0] * ranks.sizes[dim])
+    dr = C.c_uint64()
+    rc = lib().o_mesh_dim_members(C.byref(ranks.c), C.c_uint64(rank), C.c_uint32(dim), out, C.byref(dr))
+    if rc:
+        raise OracleError(rc)
+    return list(out)[: ranks.sizes[dim]], dr.value
+
+
+def mesh_ranks_for_dims(ranks: OSlice, rank: int, dims: Sequence[int]) -> List[int]:
+    total = 1
+    for d in dims:
+        total *= ranks.sizes[d]
+    out = _u64([0] * total)
+    n = lib().o_mesh_ranks_for_dims(C.byref(ranks.c), C.c_uint64(rank), (C.c_uint32 * max(1, len(dims)))(*dims),
+                                    C.c_uint32(len(dims)), out)
+    if n < 0:
+        raise OracleError(6)
+    return list(out)[:n]
+
+
+def e4m3fn_encode(f: float, saturate: bool = False) -> int:
+    return int(lib().o_e4m3fn_encode(C.c_float(f), C.c_int(int(saturate))))
+
+
+def e4m3fn_decode(c: int) -> float:
+    return float(lib().o_e4m3fn_decode(C.c_uint8(c)))
+
+
+def fp8_quantize(x_bf16: np.ndarray, block: int = 1024) -> Tuple[np.ndarray, np.ndarray]:
+    x = np.ascontiguousarray(x_bf16, dtype=np.uint16).reshape(-1)
+    nb = (x.size + block - 1) // block
+    q = np.empty(x.size, dtype=np.uint8)
+    scales = np.empty(nb, dtype=np.float32)
+    lib().o_fp8_quantize(_ptr(q), _ptr(scales), _ptr(x), C.c_uint64(x.size), C.c_uint32(block))
+    return q, scales
+
+
+def fp8_dequant_accumulate(acc: np.ndarray, q: np.ndarray, scales: np.ndarray, block: int = 1024) -> None:
+    assert acc.dtype == np.float32 and q.dtype == np.uint8 and scales.dtype == np.float32
+    assert acc.flags.c_contiguous and q.flags.c_contiguous and scales.flags.c_contiguous
+    lib().o_fp8_dequant_accumulate(_ptr(acc), _ptr(q), _ptr(scales), C.c_uint64(q.size), C.c_uint32(block))
+
+
+def fp8_dequantize(q: np.ndarray, scales: np.ndarray, block: int = 1024) -> np.ndarray:
+    out = np.empty(q.size, dtype=np.float32)
+    lib().o_fp8_dequantize(_ptr(out), _ptr(q), _ptr(scales), C.c_uint64(q.size), C.c_uint32(block))
+    return out
+
+
+def flat_pack(tensors: Sequence[np.ndarray], offsets: Sequence[int]) -> np.ndarray:
+    tensors = [np.ascontiguousarray(t).reshape(-1) for t in tensors]
+    dt = tensors[0].dtype
+    flat = np.zeros(offsets[-1], dtype=dt)
+    ptrs = (C.c_void_p * len(tensors))(*[t.ctypes.data for t in tensors])
+    lib().o_flat_pack(_ptr(flat), ptrs, _u64(offsets), C.c_uint32(len(tensors)), C.c_uint32(dt.itemsize))
+    return flat
+
+
+def flat_unpack(flat: np.ndarray, offsets: Sequence[int]) -> List[np.ndarray]:
+    outs = [np.empty(offsets[i + 1] - offsets[i], dtype=flat.dtype) for i in range(len(offsets) - 1)]
+    ptrs = (C.c_void_p * len(outs))(*[t.ctypes.data for t in outs])
+    lib().o_flat_unpack(ptrs, _ptr(flat), _u64(offsets), C.c_uint32(len(outs)), C.c_uint32(flat.itemsize))
+    return outs
