@@ -1,0 +1,366 @@
+#!/usr/bin/env python3
+"""Benchmark of the mesh data-movement / reduce hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one pass of the hot path over one batch of synthetic, seeded input that is
+already resident in HBM.  The default workload is the bf16 gradient-bucket reduce
+(8 x 25,165,824 bf16 -> fp32 sum -> /8 -> bf16).  Prints ONE JSON line; ``value`` is
+algorithmic GB/s (every input element read once, every output element written once)
+over wall-clock time; ``roofline.achieved`` is the same bytes over the average kernel
+duration measured with HIP events on the launch stream.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path"
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
+# None until a counter run exists for the workload.
+MEASURED_TRAFFIC = {}
+
+
+def _load():
+    import torch
+    import monarch_amd
+    from monarch_amd import _lib
+
+    lib = monarch_amd.lib()  # raises if the HIP library was not built: no fallback
+    return torch, lib, _lib
+
+
+def STREAM() -> int:
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def prepared(symbol, *args):
+    """A launch with its ctypes arguments built once: the timed loop then costs one foreign call per step."""
+    import monarch_amd
+    fn = getattr(monarch_amd.lib(), symbol)
+    keep = args  # keeps pointer tables and Slice structs alive
+
+    def call(_i=0):
+        return fn(*keep)
+
+    return call
+
+
+class Events:
+    """HIP event pair on an explicit stream, through the C ABI."""
+
+    def __init__(self, lib, stream):
+        self.lib, self.stream = lib, stream
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        assert lib.mhip_event_create(C.byref(self.a)) == 0 and lib.mhip_event_create(C.byref(self.b)) == 0
+
+    def start(self):
+        assert self.lib.mhip_event_record(self.a, self.stream) == 0
+
+    def stop_ms(self) -> float:
+        assert self.lib.mhip_event_record(self.b, self.stream) == 0
+        assert self.lib.mhip_event_synchronize(self.b) == 0
+        ms = C.c_float()
+        assert self.lib.mhip_event_elapsed_ms(C.byref(ms), self.a, self.b) == 0
+        return ms.value
+
+
+# ---------------------------------------------------------------------------
+# workloads: each returns (name, algorithmic_bytes_per_step, launch(i), cpu_baseline(), kernel_name)
+# ---------------------------------------------------------------------------
+
+def wl_c2(torch, in_place=False, sets=3):
+    from monarch_amd import _lib
+    from monarch_amd import reduce as R
+    from monarch_amd._lib import ptr_array
+    n, numel = 8, 25_165_824
+    g = torch.Generator(device="cuda:0").manual_seed(2000)
+    bufs = []
+    for _ in range(sets):  # rotate buffer sets so that no pass is served from the 256 MB Infinity Cache
+        ins = [(torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16() for _ in range(n)]
+        out = ins[0] if in_place else torch.empty_like(ins[0])
+        bufs.append((ins, out))
+    nbytes = (n + 1) * numel * 2
+
+    for ins, out in bufs:  # one checked call through the host API, then raw prepared calls in the timed loop
+        R.all_reduce(out, ins, R.ReduceOp.Avg)
+    calls = [prepared("mhip_reduce", out.data_ptr(), ptr_array([t.data_ptr() for t in ins]), n, numel,
+                      _lib.DTYPE_BF16, _lib.OP_AVG, STREAM()) for ins, out in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import numpy as np
+        import oracle
+        g2 = torch.Generator(device="cuda:0").manual_seed(2000)
+        hosts = [(torch.randn(numel, generator=g2, device="cuda:0") * 0.02).bfloat16().cpu().view(torch.uint16).numpy()
+                 for _ in range(n)]
+        out = np.empty_like(hosts[0])
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or time.perf_counter() - t0 < 5.0:
+            oracle.reduce(hosts, oracle.AVG, out=out)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"full workload, {reps} passes of the oracle's scalar fp32-accumulate loop"}
+
+    name = "c2_bf16_bucket_reduce_avg8_inplace" if in_place else "c2_bf16_bucket_reduce_avg8"
+    return name, nbytes, launch, cpu, "reduce_kernel<bf16,8,avg>", "bf16"
+
+
+def wl_c2p(torch, unpack=False, sets=6):
+    from monarch_amd import Slice, staging
+    numel = 25_165_824
+    g = torch.Generator(device="cuda:0").manual_seed(2001)
+    s = Slice.new_row_major([numel])
+    bufs = [((torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16(),
+             torch.empty(numel, dtype=torch.bfloat16, device="cuda:0")) for _ in range(sets)]
+    nbytes = 2 * numel * 2
+
+    for x, st in bufs:
+        staging.pack(x, s, out=st)
+    if unpack:
+        calls = [prepared("mhip_slice_unpack", x.data_ptr(), st.data_ptr(), C.byref(s.c), 2, STREAM()) for x, st in bufs]
+    else:
+        calls = [prepared("mhip_slice_pack", st.data_ptr(), x.data_ptr(), C.byref(s.c), 2, STREAM()) for x, st in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import numpy as np
+        import oracle
+        h = bufs[0][0].cpu().view(torch.uint16).numpy()
+        os_ = oracle.OSlice(0, [numel], [1])
+        t0 = time.perf_counter()
+        oracle.pack(h, os_)
+        dt = time.perf_counter() - t0
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "full workload, 1 pass of the per-element Slice::get walk"}
+
+    return ("c2p_contiguous_unpack" if unpack else "c2p_contiguous_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
+
+
+def wl_c3(torch, unpack=False, sets=3):
+    from monarch_amd import Slice, staging
+    from monarch_amd._lib import ptr_array
+    from monarch_amd.ndslice import slice_array
+    g = torch.Generator(device="cuda:0").manual_seed(3000)
+    views = [Slice(offset=k * 1792, sizes=[4096, 1792], strides=[14336, 1]) for k in range(8)]
+    bufs = []
+    for _ in range(sets):
+        w = (torch.randn(4096, 14336, generator=g, device="cuda:0") * 0.02).bfloat16()
+        outs = [torch.empty(4096 * 1792, dtype=torch.bfloat16, device="cuda:0") for _ in range(8)]
+        staging.pack_many(w, views, outs)
+        bufs.append((w, outs))
+    nbytes = 2 * 4096 * 14336 * 2
+
+    arr = slice_array(views)
+    if unpack:
+        calls = [prepared("mhip_slice_unpack_many", w.data_ptr(), ptr_array([o.data_ptr() for o in outs]), arr, 8, 2,
+                          STREAM()) for w, outs in bufs]
+    else:
+        calls = [prepared("mhip_slice_pack_many", ptr_array([o.data_ptr() for o in outs]), w.data_ptr(), arr, 8, 2,
+                          STREAM()) for w, outs in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import oracle
+        h = bufs[0][0].cpu().view(torch.uint16).numpy().reshape(-1)
+        ov = [oracle.OSlice(v.offset, v.sizes, v.strides) for v in views]
+        t0 = time.perf_counter()
+        for v in ov[:2]:
+            oracle.pack(h, v)
+        dt = (time.perf_counter() - t0) * 4
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "2 of the 8 column blocks through the per-element Slice::get walk, scaled x4"}
+
+    return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
+
+
+def wl_c4(torch, sets=2):
+    from monarch_amd import Slice, _lib
+    from monarch_amd._lib import ptr_array
+    from monarch_amd.ndslice import slice_array
+    H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
+    g = torch.Generator(device="cuda:0").manual_seed(4000)
+    slab, w = Rr * Cc, Cc // K
+    in_view = Slice(offset=0, sizes=[H, Rr, Cc], strides=[G * slab, Cc, 1])
+    out_views = [Slice(offset=k * w, sizes=[H, Rr, w], strides=[Rr * Cc, Cc, 1]) for k in range(K)]
+    bufs = []
+    for _ in range(sets):
+        x = torch.rand(H, G, Rr, Cc, generator=g, device="cuda:0") * 2 - 1
+        group = [x.view(-1)[gi * slab:] for gi in range(G)]
+        outs = [torch.empty(H * Rr * w, device="cuda:0") for _ in range(K)]
+        bufs.append((x, group, outs))
+    nbytes = H * G * slab * 4 + H * slab * 4
+
+    arr = slice_array(out_views)
+    calls = [prepared("mhip_reduce_scatter", ptr_array([o.data_ptr() for o in outs]), arr, K,
+                      ptr_array([t.data_ptr() for t in group]), C.byref(in_view.c), 0, G, _lib.DTYPE_F32, _lib.OP_SUM,
+                      STREAM()) for _, group, outs in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import oracle
+        hx = bufs[0][0].cpu().numpy().reshape(-1)
+        ov = oracle.OSlice(in_view.offset, in_view.sizes, in_view.strides)
+        o0 = oracle.OSlice(out_views[0].offset, out_views[0].sizes, out_views[0].strides)
+        t0 = time.perf_counter()
+        oracle.reduce_scatter([hx[gi * slab:] for gi in range(G)], ov, [o0], oracle.SUM)
+        dt = (time.perf_counter() - t0) * K
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "1 of the 8 scatter outputs through the oracle, scaled x8"}
+
+    return "c4_mesh_dim_reduce_scatter_f32", nbytes, launch, cpu, "reduce_scatter_kernel<f32,vec>", "f32"
+
+
+def _c5_setup(torch):
+    import numpy as np
+    from monarch_amd import fp8
+    rng = np.random.default_rng(5000)
+    sizes = np.round(np.exp(rng.uniform(np.log(2**10), np.log(2**22), size=1500))).astype(np.int64).tolist()
+    total = sum(sizes)
+    g = torch.Generator(device="cuda:0").manual_seed(5001)
+    x = torch.randn(total, generator=g, device="cuda:0")
+    x = torch.where(torch.rand(total, generator=g, device="cuda:0") < 1e-3, x * 50, x).bfloat16()
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    tensors = [x[offs[i]: offs[i + 1]].clone() for i in range(1500)]
+    del x
+    bucket = fp8.FlatBucket(tensors)
+    return fp8, bucket, tensors, sizes, total
+
+
+def wl_c5(torch, stage="quantize"):
+    fp8, bucket, tensors, sizes, total = _c5_setup(torch)
+    nblk = (total + 1023) // 1024
+    flat = bucket.pack()
+    q, s = fp8.quantize(flat)
+    acc = torch.zeros(total, device="cuda:0")
+    outs = [torch.empty(n, device="cuda:0") for n in sizes] if stage == "flat_unpack" else None
+    if stage == "flat_pack":
+        nbytes, kern = 4 * total, "flat_copy_kernel<pack>"
+        launch = prepared("mhip_flat_pack", flat.data_ptr(), bucket.d_ptrs.data_ptr(), bucket.d_offsets.data_ptr(),
+                          len(sizes), total, 2, STREAM())
+    elif stage == "quantize":
+        nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_kernel"
+        launch = prepared("mhip_fp8_quantize", q.data_ptr(), s.data_ptr(), flat.data_ptr(), total, 1024, STREAM())
+    elif stage == "dequant_accumulate":
+        nbytes, kern = 9 * total + 4 * nblk, "fp8_dequant_accumulate_kernel"
+        launch = prepared("mhip_fp8_dequant_accumulate", acc.data_ptr(), q.data_ptr(), s.data_ptr(), total, 1024,
+                          STREAM())
+    else:
+        nbytes, kern = 8 * total, "flat_copy_kernel<unpack>"
+        ptrs = bucket.pointer_table(outs)
+
+        launch = prepared("mhip_flat_unpack", ptrs.data_ptr(), acc.data_ptr(), bucket.d_offsets.data_ptr(), len(sizes),
+                          total, 4, STREAM())
+
+    def cpu():
+        import numpy as np
+        import oracle
+        sample = min(total, 64 * 1024 * 1024)
+        h = flat[:sample].cpu().view(torch.uint16).numpy()
+        t0 = time.perf_counter()
+        if stage == "quantize":
+            oracle.fp8_quantize(h, 1024)
+        elif stage == "dequant_accumulate":
+            hq, hs = q[:sample].cpu().numpy(), s[: (sample + 1023) // 1024].cpu().numpy()
+            ha = np.zeros(sample, dtype=np.float32)
+            t0 = time.perf_counter()
+            oracle.fp8_dequant_accumulate(ha, hq, hs, 1024)
+        else:
+            np.copyto(np.empty_like(h), h)
+        dt = (time.perf_counter() - t0) * (total / sample)
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"first {sample} elements of the flat buffer through the oracle, scaled to {total}"}
+
+    return f"c5_fp8_{stage}", nbytes, launch, cpu, kern, "bf16->f8e4m3fn"
+
+
+WORKLOADS = {
+    "c2": lambda t: wl_c2(t, False),
+    "c2_inplace": lambda t: wl_c2(t, True),
+    "c2p_pack": lambda t: wl_c2p(t, False),
+    "c2p_unpack": lambda t: wl_c2p(t, True),
+    "c3_pack": lambda t: wl_c3(t, False),
+    "c3_unpack": lambda t: wl_c3(t, True),
+    "c4": wl_c4,
+    "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
+    "c5_quantize": lambda t: wl_c5(t, "quantize"),
+    "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
+    "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
+}
+
+
+def run(workload: str, steps: int, warmup: int, cpu_baseline: bool):
+    torch, lib, _ = _load()
+    torch.cuda.set_device(0)
+    name, nbytes, launch, cpu, kernel, dtype = WORKLOADS[workload](torch)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = 0
+    for i in range(warmup):
+        rc |= launch(i)
+    torch.cuda.synchronize()
+    ev = Events(lib, stream)
+    t0 = time.perf_counter()
+    ev.start()
+    for i in range(steps):
+        rc |= launch(i)
+    kernel_ms = ev.stop_ms() / steps
+    if rc != 0:
+        sys.exit(f"a launch returned status {rc}")
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    rec = {
+        "metric": METRIC, "value": nbytes / (wall_ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": wall_ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": name, "algorithmic_bytes_per_step": nbytes, "kernel": kernel},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(workload)},
+    }
+    if cpu_baseline:
+        rec["cpu_baseline"] = cpu()
+        rec["cpu_baseline"]["host_cpus"] = os.cpu_count()
+    return rec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=60)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also run every other workload; their lines go to stderr")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.all:
+        for w in sorted(WORKLOADS):
+            if w != args.workload:
+                rec = run(w, args.steps, args.warmup, not args.no_cpu_baseline)
+                print(json.dumps(rec), file=sys.stderr, flush=True)
+    print(json.dumps(run(args.workload, args.steps, args.warmup, not args.no_cpu_baseline)), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,258 @@
+/*
+ * monarch_hip.h - C ABI of libmonarch_hip.so: the MI355X (gfx950) data plane for
+ * Monarch's mesh data-movement / reduce path.
+ *
+ * This is the contract a `hip-sys` crate binds (the sibling of the reference's
+ * cuda-sys/ and nccl-sys/ crates).  Plain pointers and sizes only; every entry
+ * point returns an int status (0 = success, 1..9999 = hipError_t passed through,
+ * >= 10000 = the library's own classes below).  Device entry points enqueue on the
+ * caller's stream and never synchronise; completion is observed the way the
+ * reference does it, by recording an event on that stream afterwards
+ * (monarch_tensor_worker/src/comm.rs:156).  All device pointers are caller-owned;
+ * the library allocates nothing.  Entry points may be called from any thread; the
+ * device is taken from the stream (or is the current device for the NULL stream).
+ *
+ * Units: a Slice counts ELEMENTS (ndslice/src/slice.rs:85-90); pack/unpack take the
+ * element size in bytes; RdmaBuffer-style staging memory is addressed in bytes
+ * (monarch_rdma/src/rdma_components.rs:94-102).
+ */
+#ifndef MONARCH_HIP_H
+#define MONARCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* hipStream_t / hipEvent_t, kept opaque so that binding this header needs no HIP headers.
+ * Replaces cudaStream_t / CUstream_st of nccl-sys/build.rs:93-148 and
+ * torch-sys-cuda/src/cuda.rs:15-17 on this path. */
+typedef void* mhip_stream_t;
+typedef void* mhip_event_t;
+
+/* ---- status codes ---- */
+enum {
+    MHIP_SUCCESS = 0,
+    /* SliceError, ndslice/src/slice.rs:15-51 */
+    MHIP_ERR_INVALID_DIMS = 10001,
+    MHIP_ERR_NONRECTANGULAR_SHAPE = 10002,
+    MHIP_ERR_NONUNIQUE_STRIDES = 10003,
+    MHIP_ERR_STRIDE_TOO_SMALL = 10004,
+    MHIP_ERR_INDEX_OUT_OF_RANGE = 10005,
+    MHIP_ERR_VALUE_NOT_IN_SLICE = 10006,
+    MHIP_ERR_INCOMPATIBLE_VIEW = 10007,
+    MHIP_ERR_NONCONTIGUOUS = 10008,
+    MHIP_ERR_EMPTY_RANGE = 10009,
+    MHIP_ERR_DIMENSION_OUT_OF_RANGE = 10010,
+    /* NcclError argument checks, torch-sys-cuda/src/nccl.rs:56-93 */
+    MHIP_ERR_INVALID_DATA_TYPE = 10101,
+    MHIP_ERR_NONCONTIGUOUS_TENSOR = 10102,
+    MHIP_ERR_INVALID_DEVICE = 10103,
+    MHIP_ERR_FLOAT8_REDUCTION = 10104,
+    MHIP_ERR_TYPE_MISMATCH = 10105,
+    MHIP_ERR_OUTPUT_SIZE_MISMATCH = 10106,
+    MHIP_ERR_INPUT_SIZE_MISMATCH = 10107,
+    MHIP_ERR_UNDEFINED_TENSOR = 10108,
+    /* library-specific */
+    MHIP_ERR_INVALID_ARGUMENT = 10201,
+    MHIP_ERR_UNSUPPORTED_OP = 10202,
+    MHIP_ERR_TOO_MANY_INPUTS = 10203,
+    MHIP_ERR_UNSUPPORTED_BLOCK = 10204
+};
+
+/* Text for any status this library returns (hipGetErrorString for HIP codes);
+ * the counterpart of cuGetErrorString in monarch_rdma/src/macros.rs:9-24. */
+const char* mhip_error_string(int status);
+/* Library version, major*10000 + minor*100 + patch. */
+int mhip_version(void);
+
+/* ---- element types: c10::ScalarType numbering, as carried by
+ * monarch_messages Factory.dtype (monarch_messages/src/worker.rs:434-447) ---- */
+enum {
+    MHIP_DTYPE_U8 = 0,
+    MHIP_DTYPE_I8 = 1,
+    MHIP_DTYPE_I32 = 3,
+    MHIP_DTYPE_I64 = 4,
+    MHIP_DTYPE_F16 = 5,
+    MHIP_DTYPE_F32 = 6,
+    MHIP_DTYPE_F64 = 7,
+    MHIP_DTYPE_BF16 = 15,
+    MHIP_DTYPE_F8E5M2 = 23,
+    MHIP_DTYPE_F8E4M3FN = 24,
+    MHIP_DTYPE_F8E5M2FNUZ = 25,
+    MHIP_DTYPE_F8E4M3FNUZ = 26
+};
+/* Size in bytes of a dtype, 0 if unknown. */
+uint32_t mhip_dtype_size(int dtype);
+
+/* ncclRedOp_t numbering, torch-sys-cuda/src/nccl.rs:285-292. */
+enum { MHIP_OP_SUM = 0, MHIP_OP_PROD = 1, MHIP_OP_MAX = 2, MHIP_OP_MIN = 3, MHIP_OP_AVG = 4 };
+
+/* ====================================================================== */
+/* Slice: host-side index algebra (no GPU needed)                         */
+/* ====================================================================== */
+
+/* ndslice::Slice {offset, sizes, strides}, ndslice/src/slice.rs:85-90.  sizes and
+ * strides each hold ndim entries and stay owned by the caller. */
+typedef struct {
+    uint64_t offset;
+    uint32_t ndim;
+    const uint64_t* sizes;
+    const uint64_t* strides;
+} mhip_slice_t;
+
+#define MHIP_MAX_DIMS 32
+
+/* Slice::new validation (slice.rs:99-139): same rules, same error classes, same order. */
+int mhip_slice_validate(uint64_t offset, const uint64_t* sizes, uint32_t nsizes,
+                        const uint64_t* strides, uint32_t nstrides);
+/* Slice::len (slice.rs:382-384). */
+int mhip_slice_len(const mhip_slice_t* s, uint64_t* len);
+/* Slice::is_contiguous (slice.rs:198-207). */
+int mhip_slice_is_contiguous(const mhip_slice_t* s, int* result);
+/* Slice::get (slice.rs:523-537). */
+int mhip_slice_get(const mhip_slice_t* s, uint64_t index, uint64_t* loc);
+/* Slice::location (slice.rs:330-343). */
+int mhip_slice_location(const mhip_slice_t* s, const uint64_t* coord, uint32_t ncoord, uint64_t* loc);
+/* Slice::coordinates (slice.rs:347-374); coords holds ndim entries. */
+int mhip_slice_coordinates(const mhip_slice_t* s, uint64_t value, uint64_t* coords);
+/* Slice::index (slice.rs:460-471). */
+int mhip_slice_index(const mhip_slice_t* s, uint64_t value, uint64_t* index);
+/* Slice::iter (slice.rs:391-396, 704-781): locations of items [start, start+count) of the
+ * row-major enumeration, clipped to len; *written receives how many were produced. */
+int mhip_slice_iter(const mhip_slice_t* s, uint64_t start, uint64_t count, uint64_t* locs,
+                    uint64_t* written);
+/* Slice::select (slice.rs:291-327); out arrays hold ndim entries. */
+int mhip_slice_select(const mhip_slice_t* s, uint32_t dim, uint64_t begin, uint64_t end,
+                      uint64_t step, uint64_t* out_offset, uint64_t* out_sizes,
+                      uint64_t* out_strides);
+/* Slice::at (slice.rs:243-264); out arrays hold ndim-1 entries. */
+int mhip_slice_at(const mhip_slice_t* s, uint32_t dim, uint64_t index, uint64_t* out_offset,
+                  uint64_t* out_sizes, uint64_t* out_strides);
+/* Slice::subview (slice.rs:638-661): result is {*out_offset, lens, s->strides}. */
+int mhip_slice_subview(const mhip_slice_t* s, const uint64_t* starts, uint32_t nstarts,
+                       const uint64_t* lens, uint32_t nlens, uint64_t* out_offset);
+/* Slice::view (slice.rs:579-635): result is {0, new_sizes, out_strides}. */
+int mhip_slice_view(const mhip_slice_t* s, const uint64_t* new_sizes, uint32_t nnew,
+                    uint64_t* out_strides);
+/* Slice::enforce_embedding (slice.rs:683-687). */
+int mhip_slice_enforce_embedding(const mhip_slice_t* s, const mhip_slice_t* other);
+/* Smallest and largest location the slice touches (for sizing/guarding the base
+ * allocation); MHIP_ERR_INVALID_ARGUMENT for an empty slice.  No reference counterpart. */
+int mhip_slice_bounds(const mhip_slice_t* s, uint64_t* min_loc, uint64_t* max_loc);
+
+/* DeviceMesh::new, one dimension (monarch_tensor_worker/src/device_mesh.rs:71-102):
+ * members[0..sizes[dim]) and the owning rank's position among them. */
+int mhip_mesh_dim_members(const mhip_slice_t* ranks, uint64_t rank, uint32_t dim,
+                          uint64_t* members, uint64_t* dim_rank);
+/* DeviceMesh::get_ranks_for_dim_slice (device_mesh.rs:120-177): the reduce group of the
+ * named dims (given as dim indices, in the caller's order); *count receives the group
+ * size N that Avg divides by and scatter splits into (monarch_tensor_worker/src/lib.rs:899,911). */
+int mhip_mesh_ranks_for_dims(const mhip_slice_t* ranks, uint64_t rank, const uint32_t* dims,
+                             uint32_t ndims, uint64_t* out, uint64_t cap, uint64_t* count);
+
+/* ====================================================================== */
+/* pack / unpack: Slice view <-> contiguous staging memory                 */
+/* ====================================================================== */
+
+/* dst[i] = src_base[s.get(i)] for i in [0, len): gathers the view, in Slice::iter order
+ * (slice.rs:391-396), into contiguous staging memory - the bytes an RdmaBuffer
+ * {addr = dst, size = len*elem_size} then moves with read_into
+ * (monarch_rdma/src/rdma_components.rs:117-137).  The slice must pass mhip_slice_validate.
+ * dst must not overlap the view. */
+int mhip_slice_pack(void* dst, const void* src_base, const mhip_slice_t* s, uint32_t elem_size,
+                    mhip_stream_t stream);
+/* dst_base[s.get(i)] = src[i]: scatters staging memory that write_from filled
+ * (rdma_components.rs:152-171) back into the view; elements outside the view are untouched. */
+int mhip_slice_unpack(void* dst_base, const void* src, const mhip_slice_t* s, uint32_t elem_size,
+                      mhip_stream_t stream);
+/* nviews packs / unpacks of views of ONE base tensor in a single launch (a reshard's
+ * column blocks): dsts[k][i] = src_base[views[k].get(i)], resp. the inverse. */
+int mhip_slice_pack_many(void* const* dsts, const void* src_base, const mhip_slice_t* views,
+                         uint32_t nviews, uint32_t elem_size, mhip_stream_t stream);
+int mhip_slice_unpack_many(void* dst_base, const void* const* srcs, const mhip_slice_t* views,
+                           uint32_t nviews, uint32_t elem_size, mhip_stream_t stream);
+
+/* Flat bucket with an offsets table (torch.cat / split of a gradient bucket,
+ * python/tests/simulator/test_simulator.py:190-203, for ragged tensors):
+ * flat[offsets[t] + j] = tensors[t][j].  d_tensors (ntensors pointers) and d_offsets
+ * (ntensors+1 element offsets, offsets[0] == 0) live in DEVICE memory; total ==
+ * offsets[ntensors] is passed by value so that the call needs no device read-back. */
+int mhip_flat_pack(void* flat, const void* const* d_tensors, const uint64_t* d_offsets,
+                   uint32_t ntensors, uint64_t total, uint32_t elem_size, mhip_stream_t stream);
+int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d_offsets,
+                     uint32_t ntensors, uint64_t total, uint32_t elem_size, mhip_stream_t stream);
+
+/* ====================================================================== */
+/* Reduce: the chunks one GPU owns                                         */
+/* ====================================================================== */
+
+/* out[i] = op_r in[r][i], r in [0, n): the local combine of Communicator::all_reduce
+ * (torch-sys-cuda/src/nccl.rs:464-489) as StreamActor::reduce uses it
+ * (monarch_tensor_worker/src/stream.rs:1437-1462).  out may alias in[0] (the in-place
+ * form); any other overlap is undefined.  Floating types accumulate in fp32 (f64 in f64)
+ * in rank order and round once; Avg divides the sum by n.  Integer Sum wraps.
+ * Argument checks follow nccl.rs:300-316,474-476: null pointer -> UNDEFINED_TENSOR,
+ * unknown dtype -> INVALID_DATA_TYPE, fp8 dtype -> FLOAT8_REDUCTION; ops other than
+ * Sum/Avg -> UNSUPPORTED_OP; n > 64 -> TOO_MANY_INPUTS. */
+int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, int dtype, int op,
+                mhip_stream_t stream);
+
+/* reduced[i] = op_g in[g][in_view.get(i)] over in_view's index space;
+ * outs[k][j] = reduced[out_views[k].get(j)]: the local combine of
+ * Communicator::reduce_scatter_tensor (nccl.rs:661-703; stream.rs:1422-1436) with the
+ * scatter expressed as Slice views of the reduced tensor.  in_view == NULL means the
+ * n_in inputs are contiguous with len == in_numel.  ncclReduceScatter's flat-chunk rule
+ * is out_views[k] = {k*c, [c], [1]}.  outs must not alias the inputs (scatter is never in
+ * place, stream.rs:1423). */
+int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32_t n_out,
+                        const void* const* in, const mhip_slice_t* in_view, uint64_t in_numel,
+                        uint32_t n_in, int dtype, int op, mhip_stream_t stream);
+
+/* ====================================================================== */
+/* Block-scaled fp8 (e4m3fn) transfer codec                                 */
+/* ====================================================================== */
+/* No counterpart in the reference (fp8 tensors travel as bytes and are refused by
+ * reductions, torch-sys-cuda/src/nccl.rs:275-278,474-476).  Per `block` consecutive
+ * elements of a flat bf16 buffer (last block may be short):
+ *   absmax = max|x| (NaN ignored) clamped to [2^-40, FLT_MAX];  scales[b] = absmax / 448
+ *   q[i] = e4m3fn_rne(clamp(x[i] * (448 / absmax), -448, 448)), NaN -> fp8 NaN
+ * block must be 1024 (MHIP_ERR_UNSUPPORTED_BLOCK otherwise). */
+int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t numel,
+                      uint32_t block, mhip_stream_t stream);
+/* acc[i] += float(q[i]) * scales[i / block]; product rounded to fp32, then added. */
+int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scales, uint64_t numel,
+                                uint32_t block, mhip_stream_t stream);
+
+/* ====================================================================== */
+/* Runtime pass-through (the cuda-sys / nccl-sys symbols this path uses)   */
+/* ====================================================================== */
+/* cuDeviceGetCount (monarch_rdma/src/test_utils.rs), cudaSetDevice (nccl-sys/build.rs:93-148) */
+int mhip_device_count(int* count);
+int mhip_set_device(int device);
+/* cudaDeviceSynchronize (cuda-sys users in monarch_rdma/src/test_utils.rs) */
+int mhip_device_synchronize(void);
+/* Stream / Event of torch-sys-cuda/src/cuda.rs:30-193; default priority only. */
+int mhip_stream_create(mhip_stream_t* stream);
+int mhip_stream_destroy(mhip_stream_t stream);
+int mhip_stream_synchronize(mhip_stream_t stream);
+int mhip_event_create(mhip_event_t* event);
+int mhip_event_destroy(mhip_event_t event);
+int mhip_event_record(mhip_event_t event, mhip_stream_t stream);
+int mhip_event_synchronize(mhip_event_t event);
+int mhip_event_elapsed_ms(float* ms, mhip_event_t start, mhip_event_t stop);
+int mhip_stream_wait_event(mhip_stream_t stream, mhip_event_t event);
+/* cuMemcpyHtoD_v2 / cuMemcpyDtoH_v2 and device allocation for the staging-buffer test
+ * environment (monarch_rdma/src/test_utils.rs:370-444). */
+int mhip_malloc(void** ptr, size_t bytes);
+int mhip_free(void* ptr);
+int mhip_memcpy_htod(void* dst, const void* src, size_t bytes, mhip_stream_t stream);
+int mhip_memcpy_dtoh(void* dst, const void* src, size_t bytes, mhip_stream_t stream);
+int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MONARCH_HIP_H */

@@ -1,0 +1,215 @@
+// Block-scaled fp8 (OCP e4m3fn) codec for flat bf16 transfer buffers, gfx950.
+//
+// quantize: 3 bytes of HBM traffic per element (2 in, 1 out) + 4 per 1024-element block.
+//   One wavefront owns one 1024-element block: each lane holds 16 elements in registers
+//   (two 128-bit loads, each a fully coalesced 1 KiB wavefront access), the block absmax
+//   is a lane-local max over packed 16-bit magnitudes followed by a DPP butterfly inside
+//   each row of 16 lanes and four readlanes across rows - no LDS, no second pass over
+//   memory - and the 16 codes leave as two 64-bit stores.
+// dequant_accumulate: 9 bytes per element (1 code in, fp32 accumulator in and out).
+//   A 256-thread workgroup step covers exactly one block, so the scale is uniform.
+#include <cfloat>
+
+#include "mhip_device.h"
+
+namespace mhip {
+
+constexpr uint32_t kBlock = 1024;         // elements per scale
+constexpr float kFp8Max = 448.0f;
+constexpr float kAbsmaxFloor = 0x1p-40f;  // keeps 448/absmax finite for all-zero / denormal blocks
+
+// all-reduce max over the 64 lanes of a wavefront, for unsigned 32-bit values
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    // DPP butterfly within each row of 16 lanes
+    uint32_t o;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+    v = v > o ? v : o;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
+    v = v > o ? v : o;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
+    v = v > o ? v : o;
+    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);  // row_mirror
+    v = v > o ? v : o;
+    // one value per row, combined on the scalar unit
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
+    const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
+    const uint32_t r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    const uint32_t a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
+    return a > b ? a : b;
+}
+
+__device__ __forceinline__ void block_factors(uint32_t absmax_bf16_bits, float* scale, float* inv) {
+    float absmax = __uint_as_float(absmax_bf16_bits << 16);
+    absmax = absmax < kAbsmaxFloor ? kAbsmaxFloor : absmax;
+    absmax = absmax > FLT_MAX ? FLT_MAX : absmax;
+    *scale = absmax / kFp8Max;
+    *inv = kFp8Max / absmax;
+}
+
+// two bf16 values (one 32-bit word) -> two fp8 codes in the low or high half of `old`
+template <bool HIGH>
+__device__ __forceinline__ int quant_pair(uint32_t w, float inv, int old) {
+    return __builtin_amdgcn_cvt_pk_fp8_f32(bf16_lo(w) * inv, bf16_hi(w) * inv, old, HIGH);
+}
+
+__device__ __forceinline__ uint8_t quant_one_careful(uint32_t h, float inv) {
+    float y = __uint_as_float(h << 16) * inv;
+    y = y > kFp8Max ? kFp8Max : y;    // comparisons are false for NaN: it passes through
+    y = y < -kFp8Max ? -kFp8Max : y;
+    return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false) & 0xff);
+}
+
+// Careful path for one block, whole wavefront: handles a short final block and blocks
+// holding NaN or Inf (NaN is ignored by the absmax and encodes to an fp8 NaN; Inf
+// saturates to +-448).
+__device__ __noinline__ void quantize_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                    const uint16_t* __restrict__ x, uint64_t begin, uint32_t count,
+                                                    uint64_t b, int lane) {
+    uint32_t m = 0;
+    for (uint32_t i = lane; i < count; i += 64) {
+        const uint32_t a = x[begin + i] & 0x7fffu;
+        if (a <= 0x7f80u && a > m) m = a;
+    }
+    m = wave_max_u32(m);
+    float scale, inv;
+    block_factors(m, &scale, &inv);
+    if (lane == 0) scales[b] = scale;
+    for (uint32_t i = lane; i < count; i += 64) q[begin + i] = quant_one_careful(x[begin + i], inv);
+}
+
+__global__ __launch_bounds__(kThreads) void fp8_quantize_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                                const uint16_t* __restrict__ x, uint64_t numel,
+                                                                uint64_t nblocks) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t nwaves = (uint64_t)gridDim.x * (kThreads / 64);
+    for (uint64_t b = wave; b < nblocks; b += nwaves) {
+        const uint64_t begin = b * kBlock;
+        const uint64_t remain = numel - begin;
+        if (remain < kBlock) {  // wave-uniform
+            quantize_block_careful(q, scales, x, begin, (uint32_t)remain, b, lane);
+            continue;
+        }
+        const char* src = reinterpret_cast<const char*>(x + begin);
+        const uint4 lo = load16_unaligned(src + lane * 16);         // elements [8*lane, 8*lane+8)
+        const uint4 hi = load16_unaligned(src + 1024 + lane * 16);  // elements [512+8*lane, ...)
+        // magnitudes as packed 16-bit integers: bf16 order == integer order for |x|
+        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        uint32_t m = 0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t a = w[k] & 0x7fff7fffu;
+            const uint32_t a0 = a & 0xffffu, a1 = a >> 16;
+            m = a0 > m ? a0 : m;
+            m = a1 > m ? a1 : m;
+        }
+        m = wave_max_u32(m);
+        if (m >= 0x7f80u) {  // Inf or NaN somewhere in the block (wave-uniform, rare)
+            quantize_block_careful(q, scales, x, begin, kBlock, b, lane);
+            continue;
+        }
+        float scale, inv;
+        block_factors(m, &scale, &inv);
+        if (lane == 0) scales[b] = scale;
+        // |x * inv| <= 448 * (1 + 2^-22) for every finite x of the block, which rounds to
+        // at most 448, so no clamp is needed on this path.
+        int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+        c0 = quant_pair<false>(w[0], inv, c0); c0 = quant_pair<true>(w[1], inv, c0);
+        c1 = quant_pair<false>(w[2], inv, c1); c1 = quant_pair<true>(w[3], inv, c1);
+        c2 = quant_pair<false>(w[4], inv, c2); c2 = quant_pair<true>(w[5], inv, c2);
+        c3 = quant_pair<false>(w[6], inv, c3); c3 = quant_pair<true>(w[7], inv, c3);
+        const uint2 out_lo = make_uint2((uint32_t)c0, (uint32_t)c1);
+        const uint2 out_hi = make_uint2((uint32_t)c2, (uint32_t)c3);
+        uint8_t* dst = q + begin;
+        __builtin_memcpy(dst + lane * 8, &out_lo, 8);
+        __builtin_memcpy(dst + 512 + lane * 8, &out_hi, 8);
+    }
+}
+
+// acc[i] += float(q[i]) * scale[i / 1024].  A workgroup step covers 1024 consecutive
+// elements starting at a multiple of 1024, i.e. exactly one block.
+constexpr int kDeqSteps = 4;
+
+__global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float* __restrict__ acc,
+                                                                          const uint8_t* __restrict__ q,
+                                                                          const float* __restrict__ scales,
+                                                                          uint64_t numel, uint64_t ntiles) {
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint64_t b0 = tile * kDeqSteps;
+        uint32_t codes[kDeqSteps];
+        uint4 a[kDeqSteps];
+        float s[kDeqSteps];
+        bool full[kDeqSteps];
+#pragma unroll
+        for (int j = 0; j < kDeqSteps; ++j) {
+            const uint64_t i = (b0 + j) * kBlock + threadIdx.x * 4;
+            full[j] = i + 4 <= numel;
+            if (full[j]) {
+                __builtin_memcpy(&codes[j], q + i, 4);
+                a[j] = load16_unaligned(acc + i);
+                s[j] = scales[b0 + j];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kDeqSteps; ++j) {
+            const uint64_t i = (b0 + j) * kBlock + threadIdx.x * 4;
+            if (full[j]) {
+                const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], false);
+                const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], true);
+                // product rounded to fp32, then added: two roundings (contraction is off)
+                uint4 r;
+                r.x = __float_as_uint(__uint_as_float(a[j].x) + p01[0] * s[j]);
+                r.y = __float_as_uint(__uint_as_float(a[j].y) + p01[1] * s[j]);
+                r.z = __float_as_uint(__uint_as_float(a[j].z) + p23[0] * s[j]);
+                r.w = __float_as_uint(__uint_as_float(a[j].w) + p23[1] * s[j]);
+                store16_unaligned(acc + i, r);
+            } else {
+                for (uint64_t e = i; e < numel && e < i + 4; ++e) {
+                    const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
+                    acc[e] = acc[e] + p[0] * scales[e / kBlock];
+                }
+            }
+        }
+    }
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" {
+
+int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t numel, uint32_t block,
+                      mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (numel == 0) return MHIP_SUCCESS;
+    if (!q || !scales || !x_bf16) return MHIP_ERR_UNDEFINED_TENSOR;
+    if (((uintptr_t)x_bf16 & 1u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
+    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
+    const uint64_t wgs = (nblocks + 3) / 4;
+    const uint64_t cap = 256ull * 32ull;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads), 0, hs, q, scales,
+                       static_cast<const uint16_t*>(x_bf16), numel, nblocks);
+    return launch_status();
+}
+
+int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scales, uint64_t numel, uint32_t block,
+                                mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (numel == 0) return MHIP_SUCCESS;
+    if (!acc || !q || !scales) return MHIP_ERR_UNDEFINED_TENSOR;
+    if (((uintptr_t)acc & 3u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
+    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
+    const uint64_t ntiles = (nblocks + kDeqSteps - 1) / kDeqSteps;
+    const uint64_t cap = 256ull * 64ull;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kThreads), 0,
+                       hs, acc, q, scales, numel, ntiles);
+    return launch_status();
+}
+
+}  // extern "C"

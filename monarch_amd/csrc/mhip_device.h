@@ -1,0 +1,131 @@
+// Device-side helpers shared by the kernel sources (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "mhip_internal.h"
+
+namespace mhip {
+
+constexpr int kThreads = 256;  // 4 wavefronts of 64 lanes
+
+// Kernel-argument form of a CanonSlice: row-major decode of a packed unit index
+// into a unit offset in the strided tensor.
+struct DimsArg {
+    uint64_t run;                      // contiguous units per row
+    uint64_t size[kMaxCanonDims];      // outermost first
+    uint64_t stride[kMaxCanonDims];    // units
+    FastDiv32 run_div;                 // valid in 32-bit mode only
+    FastDiv32 size_div[kMaxCanonDims];
+    int ndim;
+};
+
+inline bool make_dims_arg(const CanonSlice& c, DimsArg* d, bool* fits32) {
+    if (c.ndim > kMaxCanonDims) return false;
+    d->run = c.run;
+    d->ndim = c.ndim;
+    bool small = c.total < kFastDivLimit - 64 && c.run < kFastDivLimit;
+    for (int k = 0; k < kMaxCanonDims; ++k) {
+        d->size[k] = k < c.ndim ? c.dims[k].size : 1;
+        d->stride[k] = k < c.ndim ? c.dims[k].stride : 0;
+        if (d->size[k] >= kFastDivLimit) small = false;
+    }
+    if (small) {
+        d->run_div = FastDiv32((uint32_t)c.run);
+        for (int k = 0; k < kMaxCanonDims; ++k) d->size_div[k] = FastDiv32((uint32_t)d->size[k]);
+    }
+    *fits32 = small;
+    return true;
+}
+
+// Unit offset of packed unit t, and its column within the row (for run-boundary tests).
+template <bool WIDE>
+__device__ __forceinline__ uint64_t decode(const DimsArg& d, uint64_t t, uint64_t* col_out) {
+    if (d.ndim == 0) {
+        *col_out = t;  // one row: run == total
+        return t;
+    }
+    uint64_t off;
+    if constexpr (WIDE) {
+        uint64_t row = t / d.run;
+        uint64_t col = t - row * d.run;
+        *col_out = col;
+        off = col;
+        for (int k = d.ndim - 1; k > 0; --k) {
+            uint64_t q = row / d.size[k];
+            off += (row - q * d.size[k]) * d.stride[k];
+            row = q;
+        }
+        off += row * d.stride[0];
+    } else {
+        uint32_t row, col;
+        d.run_div.divmod((uint32_t)t, row, col);
+        *col_out = col;
+        off = col;
+        for (int k = d.ndim - 1; k > 0; --k) {
+            uint32_t q, r;
+            d.size_div[k].divmod(row, q, r);
+            off += (uint64_t)r * d.stride[k];
+            row = q;
+        }
+        off += (uint64_t)row * d.stride[0];
+    }
+    return off;
+}
+
+template <int U> struct UnitType;
+template <> struct UnitType<1> { using type = uint8_t; };
+template <> struct UnitType<2> { using type = uint16_t; };
+template <> struct UnitType<4> { using type = uint32_t; };
+template <> struct UnitType<8> { using type = uint64_t; };
+template <> struct UnitType<16> { using type = uint4; };
+
+// 16-byte access at an address that is only known to be unit-aligned.  gfx950 under
+// the HSA runtime services unaligned global dwordx4 accesses in hardware, and the
+// compiler emits a single global_load/store_dwordx4 for these.
+__device__ __forceinline__ uint4 load16_unaligned(const void* p) {
+    uint4 v;
+    __builtin_memcpy(&v, p, 16);
+    return v;
+}
+__device__ __forceinline__ void store16_unaligned(void* p, const uint4& v) { __builtin_memcpy(p, &v, 16); }
+
+// bf16 <-> fp32.  Widening is exact; narrowing is round-to-nearest-even with NaN
+// mapped to the canonical quiet NaN 0x7fc0 (what torch's CPU cast produces).
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (u & 0x7fffffffu) > 0x7f800000u ? 0x7fc0u : r;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// Makes the stream's device current for the duration of a launch and restores the
+// caller's device afterwards, so entry points never depend on the current device.
+class DeviceGuard {
+public:
+    explicit DeviceGuard(hipStream_t stream) {
+        if (stream == nullptr) return;
+        int dev = -1;
+        if (hipStreamGetDevice(stream, &dev) != hipSuccess) { (void)hipGetLastError(); return; }
+        if (hipGetDevice(&prev_) != hipSuccess) { prev_ = -1; return; }
+        if (dev != prev_) {
+            if (hipSetDevice(dev) == hipSuccess) restore_ = true;
+        }
+    }
+    ~DeviceGuard() {
+        if (restore_) (void)hipSetDevice(prev_);
+    }
+private:
+    int prev_ = -1;
+    bool restore_ = false;
+};
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? MHIP_SUCCESS : (int)e;
+}
+
+}  // namespace mhip

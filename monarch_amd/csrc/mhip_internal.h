@@ -1,0 +1,43 @@
+// Internal declarations shared by the host-side sources of libmonarch_hip.so.
+#pragma once
+#include <cstdint>
+
+#include "../../include/monarch_hip.h"
+#include "fastdiv.h"
+
+namespace mhip {
+
+int validate_slice(const uint64_t* sizes, uint32_t nsizes, const uint64_t* strides, uint32_t nstrides);
+uint64_t slice_len(const mhip_slice_t& s);
+
+// A Slice reduced to what a copy kernel needs.  Units are `unit` bytes.  Dimensions
+// are in iteration order (outermost first); size-1 dimensions are dropped and
+// neighbours that form one linear run are merged.  When `run` > 0 the innermost
+// `run` units of every row are contiguous in the strided tensor as well, and dims[]
+// holds only the dimensions OUTSIDE that run.
+constexpr int kMaxCanonDims = 8;
+
+struct CanonDim {
+    uint64_t size;
+    uint64_t stride;  // in units
+};
+
+struct CanonSlice {
+    uint64_t offset = 0;  // units, relative to the base pointer
+    uint64_t total = 0;   // units in the packed image
+    uint64_t run = 1;     // contiguous units per row (>= 1)
+    int ndim = 0;         // dimensions outside the run
+    CanonDim dims[MHIP_MAX_DIMS + 1];
+};
+
+// Canonicalise `s` (elements of elem_size bytes) into unit-sized pieces.  `unit` is
+// chosen as the largest power of two <= max_unit that divides the element size, every
+// byte stride, the byte offset, and the alignments passed in `align_mask` (OR of the
+// addresses involved).  Returns false for an empty slice.
+bool canonicalize(const mhip_slice_t& s, uint32_t elem_size, uint64_t align_mask, uint32_t max_unit,
+                  CanonSlice* out, uint32_t* unit);
+
+// Same dimension list for two canonical slices (offsets may differ).
+bool same_shape(const CanonSlice& a, const CanonSlice& b);
+
+}  // namespace mhip

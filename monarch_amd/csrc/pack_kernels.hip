@@ -1,0 +1,359 @@
+// Slice pack/unpack and flat-bucket pack/unpack kernels for gfx950.
+//
+// Every copy is HBM-bound byte movement.  The packed (staging) side is contiguous, so
+// work is cut into 16-byte chunks aligned on the packed address; a thread moves a chunk
+// with one 128-bit access on each side whenever the chunk lies inside one contiguous
+// run of the strided tensor, and unit by unit otherwise (run boundaries, ragged head
+// and tail).  Consecutive lanes take consecutive chunks, so each wavefront instruction
+// touches 1 KiB of contiguous staging memory.
+#include "mhip_device.h"
+
+namespace mhip {
+
+constexpr int kMaxViews = 16;
+constexpr int kUnroll = 4;  // chunks per thread, issued back to back for memory-level parallelism
+
+struct PackArgs {
+    char* base;                  // strided tensor
+    char* packed[kMaxViews];     // staging buffers, one per view
+    uint64_t offset[kMaxViews];  // view offsets, units
+    uint64_t total;              // units per view
+    uint64_t nchunks;            // 16-byte chunks per view, including a ragged first one
+    uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
+    DimsArg dims;
+};
+
+template <int U, bool PACK>
+__device__ __forceinline__ void move_unit(char* strided, char* packed) {
+    using T = typename UnitType<U>::type;
+    if constexpr (PACK)
+        *reinterpret_cast<T*>(packed) = *reinterpret_cast<const T*>(strided);
+    else
+        *reinterpret_cast<T*>(strided) = *reinterpret_cast<const T*>(packed);
+}
+
+template <int U, bool PACK, bool WIDE>
+__global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
+    constexpr int VU = 16 / U;  // units per chunk
+    const int v = blockIdx.y;
+    char* __restrict__ packed = a.packed[v];
+    char* __restrict__ strided = a.base + a.offset[v] * U;
+    const uint64_t c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+
+    uint64_t loc[kUnroll];
+    uint64_t first[kUnroll];  // first packed unit of the chunk (may be "negative": see below)
+    bool vec[kUnroll];
+    bool live[kUnroll];
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) {
+        const uint64_t c = c0 + (uint64_t)i * kThreads;
+        live[i] = c < a.nchunks;
+        const uint64_t tb = c * VU;  // position counted from the aligned-down start
+        vec[i] = false;
+        first[i] = tb - a.shift;     // wraps for a ragged chunk 0; only used when tb >= shift
+        if (live[i] && tb >= a.shift && first[i] + VU <= a.total) {
+            uint64_t col;
+            loc[i] = decode<WIDE>(a.dims, first[i], &col);
+            vec[i] = col + VU <= a.dims.run;
+        }
+    }
+    uint4 data[kUnroll];
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) {
+        if (vec[i]) {
+            if constexpr (PACK)
+                data[i] = load16_unaligned(strided + loc[i] * U);
+            else
+                data[i] = *reinterpret_cast<const uint4*>(packed + first[i] * U);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) {
+        if (vec[i]) {
+            if constexpr (PACK)
+                *reinterpret_cast<uint4*>(packed + first[i] * U) = data[i];
+            else
+                store16_unaligned(strided + loc[i] * U, data[i]);
+        }
+    }
+    if constexpr (VU > 1) {
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            if (live[i] && !vec[i]) {
+                const uint64_t tb = (c0 + (uint64_t)i * kThreads) * VU;
+                for (int j = 0; j < VU; ++j) {
+                    const uint64_t t = tb + j - a.shift;
+                    if (tb + j >= a.shift && t < a.total) {
+                        uint64_t col;
+                        const uint64_t l = decode<WIDE>(a.dims, t, &col);
+                        move_unit<U, PACK>(strided + l * U, packed + t * U);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------- flat bucket <-> ragged tensors ----------------
+
+struct FlatArgs {
+    char* flat;
+    char* const* tensors;     // device table of ntensors pointers
+    const uint64_t* offsets;  // device table of ntensors+1 element offsets
+    uint64_t total;           // units
+    uint64_t nchunks;
+    uint32_t ntensors;
+    uint32_t shift;           // units
+    uint32_t units_per_elem;
+};
+
+// largest t in [lo, hi) with offsets[t] * upe <= unit
+__device__ __forceinline__ uint32_t find_tensor(const uint64_t* __restrict__ offsets, uint32_t upe, uint32_t lo,
+                                                uint32_t hi, uint64_t unit) {
+    while (hi - lo > 1) {
+        const uint32_t mid = lo + ((hi - lo) >> 1);
+        if (offsets[mid] * upe <= unit) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+template <int U, bool PACK>
+__global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
+    constexpr int VU = 16 / U;
+    __shared__ uint32_t s_range[2];
+    const uint64_t block_c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll);
+    if (threadIdx.x < 2) {
+        // tensors holding the first and the last unit this block touches
+        uint64_t c = threadIdx.x == 0 ? block_c0 : block_c0 + kThreads * kUnroll - 1;
+        if (c >= a.nchunks) c = a.nchunks - 1;
+        uint64_t tb = c * VU + (threadIdx.x == 0 ? 0 : VU - 1);
+        uint64_t unit = tb >= a.shift ? tb - a.shift : 0;
+        if (unit >= a.total) unit = a.total - 1;
+        s_range[threadIdx.x] = find_tensor(a.offsets, a.units_per_elem, 0, a.ntensors, unit);
+    }
+    __syncthreads();
+    const uint32_t t_lo = s_range[0], t_hi = s_range[1] + 1;
+    const uint32_t upe = a.units_per_elem;
+
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) {
+        const uint64_t c = block_c0 + (uint64_t)i * kThreads + threadIdx.x;
+        if (c >= a.nchunks) continue;
+        const uint64_t tb = c * VU;
+        const uint64_t first = tb - a.shift;
+        bool done = false;
+        if (tb >= a.shift && first + VU <= a.total) {
+            const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, first);
+            const uint64_t begin = a.offsets[ti] * upe, end = a.offsets[ti + 1] * upe;
+            if (first + VU <= end) {
+                char* t = a.tensors[ti] + (first - begin) * U;
+                char* f = a.flat + first * U;
+                if constexpr (PACK)
+                    *reinterpret_cast<uint4*>(f) = load16_unaligned(t);
+                else
+                    store16_unaligned(t, *reinterpret_cast<const uint4*>(f));
+                done = true;
+            }
+        }
+        if constexpr (VU > 1) {
+            if (!done) {
+                for (int j = 0; j < VU; ++j) {
+                    const uint64_t unit = tb + j - a.shift;
+                    if (tb + j >= a.shift && unit < a.total) {
+                        const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, unit);
+                        char* t = a.tensors[ti] + (unit - a.offsets[ti] * upe) * U;
+                        move_unit<U, PACK>(t, a.flat + unit * U);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------- host side ----------------
+
+template <bool PACK, bool WIDE>
+static void launch_slice_copy(uint32_t unit, dim3 grid, hipStream_t stream, const PackArgs& a) {
+    switch (unit) {
+        case 1: hipLaunchKernelGGL((slice_copy_kernel<1, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((slice_copy_kernel<2, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+        case 4: hipLaunchKernelGGL((slice_copy_kernel<4, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+        case 8: hipLaunchKernelGGL((slice_copy_kernel<8, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+        default: hipLaunchKernelGGL((slice_copy_kernel<16, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+    }
+}
+
+// One view whose canonical form has more dimensions than the kernel decodes: peel the
+// outermost dimension on the host.
+template <bool PACK>
+static int copy_views(char* base, char* const* packed, const mhip_slice_t* views, uint32_t nviews,
+                      uint32_t elem_size, hipStream_t stream);
+
+template <bool PACK>
+static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint32_t elem_size, hipStream_t stream) {
+    // s.ndim > 0 here; split along dimension 0 into sizes[0] views of one dimension fewer
+    uint64_t inner = 1;
+    for (uint32_t k = 1; k < s.ndim; ++k) inner *= s.sizes[k];
+    for (uint64_t i = 0; i < s.sizes[0]; ++i) {
+        mhip_slice_t sub{s.offset + i * s.strides[0], s.ndim - 1, s.sizes + 1, s.strides + 1};
+        char* p = packed + i * inner * elem_size;
+        if (int rc = copy_views<PACK>(base, &p, &sub, 1, elem_size, stream)) return rc;
+    }
+    return MHIP_SUCCESS;
+}
+
+template <bool PACK>
+static int copy_views(char* base, char* const* packed, const mhip_slice_t* views, uint32_t nviews,
+                      uint32_t elem_size, hipStream_t stream) {
+    uint32_t k = 0;
+    while (k < nviews) {
+        CanonSlice first;
+        uint32_t unit = 0;
+        const uint64_t mask0 = (uint64_t)(uintptr_t)base | (uint64_t)(uintptr_t)packed[k];
+        if (!canonicalize(views[k], elem_size, mask0, 16, &first, &unit)) {  // empty view: nothing to move
+            ++k;
+            continue;
+        }
+        PackArgs a{};
+        bool fits32 = false;
+        if (!make_dims_arg(first, &a.dims, &fits32)) {
+            if (int rc = copy_deep_view<PACK>(base, packed[k], views[k], elem_size, stream)) return rc;
+            ++k;
+            continue;
+        }
+        const uint32_t shift_bytes = (uint32_t)((uintptr_t)packed[k] & 15u);
+        a.base = base;
+        a.total = first.total;
+        a.shift = shift_bytes / unit;
+        const uint32_t vu = 16 / unit;
+        a.nchunks = (first.total + a.shift + vu - 1) / vu;
+        a.packed[0] = packed[k];
+        a.offset[0] = first.offset;
+        uint32_t nbatch = 1;
+        // batch following views that differ only in offset and staging pointer
+        while (k + nbatch < nviews && nbatch < (uint32_t)kMaxViews) {
+            CanonSlice next;
+            uint32_t unit2 = 0;
+            const uint64_t mask = (uint64_t)(uintptr_t)base | (uint64_t)(uintptr_t)packed[k + nbatch];
+            if (!canonicalize(views[k + nbatch], elem_size, mask, 16, &next, &unit2)) break;
+            if (unit2 != unit || !same_shape(first, next)) break;
+            if (((uintptr_t)packed[k + nbatch] & 15u) != shift_bytes) break;
+            a.packed[nbatch] = packed[k + nbatch];
+            a.offset[nbatch] = next.offset;
+            ++nbatch;
+        }
+        const uint64_t per_block = (uint64_t)kThreads * kUnroll;
+        const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
+        if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
+        dim3 grid((uint32_t)blocks, nbatch);
+        if (fits32)
+            launch_slice_copy<PACK, false>(unit, grid, stream, a);
+        else
+            launch_slice_copy<PACK, true>(unit, grid, stream, a);
+        if (int rc = launch_status()) return rc;
+        k += nbatch;
+    }
+    return MHIP_SUCCESS;
+}
+
+template <bool PACK>
+static int slice_copy_entry(char* base, char* const* packed, const mhip_slice_t* views, uint32_t nviews,
+                            uint32_t elem_size, mhip_stream_t stream) {
+    if (elem_size == 0 || (nviews && (!views || !packed))) return MHIP_ERR_INVALID_ARGUMENT;
+    for (uint32_t k = 0; k < nviews; ++k) {
+        const mhip_slice_t& s = views[k];
+        if (s.ndim > MHIP_MAX_DIMS || (s.ndim && (!s.sizes || !s.strides))) return MHIP_ERR_INVALID_ARGUMENT;
+        if (int rc = validate_slice(s.sizes, s.ndim, s.strides, s.ndim)) return rc;
+        if (slice_len(s) != 0 && (!base || !packed[k])) return MHIP_ERR_UNDEFINED_TENSOR;
+    }
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    return copy_views<PACK>(base, packed, views, nviews, elem_size, hs);
+}
+
+template <bool PACK>
+static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d_offsets, uint32_t ntensors,
+                           uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+    if (elem_size == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
+    if (!flat || !d_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
+    // unit: the power-of-two part of the element size, limited by the flat buffer's alignment
+    uint32_t unit = 16;
+    while (unit > 1 && ((elem_size | (uintptr_t)flat) & (unit - 1))) unit >>= 1;
+    // tensors are only guaranteed element-aligned, so the unit must divide the element size
+    FlatArgs a{};
+    a.flat = flat;
+    a.tensors = d_tensors;
+    a.offsets = d_offsets;
+    a.units_per_elem = elem_size / unit;
+    a.total = total * a.units_per_elem;
+    a.ntensors = ntensors;
+    a.shift = (uint32_t)(((uintptr_t)flat & 15u) / unit);
+    const uint32_t vu = 16 / unit;
+    a.nchunks = (a.total + a.shift + vu - 1) / vu;
+    const uint64_t per_block = (uint64_t)kThreads * kUnroll;
+    const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
+    if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    dim3 grid((uint32_t)blocks);
+    switch (unit) {
+        case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+        case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+        case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+        case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+        default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+    }
+    return launch_status();
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" {
+
+int mhip_slice_pack(void* dst, const void* src_base, const mhip_slice_t* s, uint32_t elem_size,
+                    mhip_stream_t stream) {
+    if (!s) return MHIP_ERR_INVALID_ARGUMENT;
+    char* p = static_cast<char*>(dst);
+    return slice_copy_entry<true>(const_cast<char*>(static_cast<const char*>(src_base)), &p, s, 1, elem_size, stream);
+}
+
+int mhip_slice_unpack(void* dst_base, const void* src, const mhip_slice_t* s, uint32_t elem_size,
+                      mhip_stream_t stream) {
+    if (!s) return MHIP_ERR_INVALID_ARGUMENT;
+    char* p = const_cast<char*>(static_cast<const char*>(src));
+    return slice_copy_entry<false>(static_cast<char*>(dst_base), &p, s, 1, elem_size, stream);
+}
+
+int mhip_slice_pack_many(void* const* dsts, const void* src_base, const mhip_slice_t* views, uint32_t nviews,
+                         uint32_t elem_size, mhip_stream_t stream) {
+    return slice_copy_entry<true>(const_cast<char*>(static_cast<const char*>(src_base)),
+                                  reinterpret_cast<char* const*>(dsts), views, nviews, elem_size, stream);
+}
+
+int mhip_slice_unpack_many(void* dst_base, const void* const* srcs, const mhip_slice_t* views, uint32_t nviews,
+                           uint32_t elem_size, mhip_stream_t stream) {
+    return slice_copy_entry<false>(static_cast<char*>(dst_base),
+                                   reinterpret_cast<char* const*>(const_cast<void* const*>(
+                                       reinterpret_cast<const void* const*>(srcs))),
+                                   views, nviews, elem_size, stream);
+}
+
+int mhip_flat_pack(void* flat, const void* const* d_tensors, const uint64_t* d_offsets, uint32_t ntensors,
+                   uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+    return flat_copy_entry<true>(static_cast<char*>(flat),
+                                 reinterpret_cast<char* const*>(const_cast<void* const*>(
+                                     reinterpret_cast<const void* const*>(d_tensors))),
+                                 d_offsets, ntensors, total, elem_size, stream);
+}
+
+int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d_offsets, uint32_t ntensors,
+                     uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+    return flat_copy_entry<false>(const_cast<char*>(static_cast<const char*>(flat)),
+                                  reinterpret_cast<char* const*>(d_tensors), d_offsets, ntensors, total,
+                                  elem_size, stream);
+}
+
+}  // extern "C"

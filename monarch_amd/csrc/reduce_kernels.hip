@@ -1,0 +1,460 @@
+// Reduce (sum / avg) over the chunks one GPU holds, with and without scatter.
+//
+// HBM-bound: (n + 1) * numel * sizeof(T) bytes per call.  Each lane moves 16 bytes per
+// input per step; all n loads of a step are issued before the first add so that a
+// wavefront keeps n KiB in flight.  Accumulation is fp32 (fp64 for f64) in rank order,
+// rounded once at the end; out may alias in[0] because a lane reads every input of its
+// own elements before it writes them.
+#include <type_traits>
+
+#include "mhip_device.h"
+
+namespace mhip {
+
+constexpr int kMaxInputs = 64;
+constexpr int kMaxOutputs = 16;
+
+struct ReduceArgs {
+    void* out;
+    const void* in[kMaxInputs];
+    uint64_t numel;
+    uint32_t n;
+    float scale;   // 1/n when n is a power of two and op is Avg (exact), else 0
+    float divisor; // n as a float
+};
+
+// ---- per-type vector traits: 16 bytes <-> accumulator lanes ----
+template <typename T> struct Vec;
+
+template <> struct Vec<float> {
+    static constexpr int V = 4;
+    using acc_t = float;
+    __device__ static void widen(const uint4& r, acc_t* a) {
+        a[0] = __uint_as_float(r.x); a[1] = __uint_as_float(r.y);
+        a[2] = __uint_as_float(r.z); a[3] = __uint_as_float(r.w);
+    }
+    __device__ static uint4 narrow(const acc_t* a) {
+        return make_uint4(__float_as_uint(a[0]), __float_as_uint(a[1]), __float_as_uint(a[2]), __float_as_uint(a[3]));
+    }
+    __device__ static acc_t widen1(const void* p, uint64_t i) { return static_cast<const float*>(p)[i]; }
+    __device__ static void narrow1(void* p, uint64_t i, acc_t v) { static_cast<float*>(p)[i] = v; }
+};
+
+struct bf16_tag {};
+template <> struct Vec<bf16_tag> {
+    static constexpr int V = 8;
+    using acc_t = float;
+    __device__ static void widen(const uint4& r, acc_t* a) {
+        a[0] = bf16_lo(r.x); a[1] = bf16_hi(r.x); a[2] = bf16_lo(r.y); a[3] = bf16_hi(r.y);
+        a[4] = bf16_lo(r.z); a[5] = bf16_hi(r.z); a[6] = bf16_lo(r.w); a[7] = bf16_hi(r.w);
+    }
+    __device__ static uint4 narrow(const acc_t* a) {
+        return make_uint4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(a[4], a[5]),
+                          pack_bf16x2(a[6], a[7]));
+    }
+    __device__ static acc_t widen1(const void* p, uint64_t i) {
+        return __uint_as_float((uint32_t) static_cast<const uint16_t*>(p)[i] << 16);
+    }
+    __device__ static void narrow1(void* p, uint64_t i, acc_t v) {
+        static_cast<uint16_t*>(p)[i] = (uint16_t)f32_to_bf16_bits(v);
+    }
+};
+
+template <> struct Vec<_Float16> {
+    static constexpr int V = 8;
+    using acc_t = float;
+    union U { uint4 r; _Float16 h[8]; };
+    __device__ static void widen(const uint4& r, acc_t* a) {
+        U u; u.r = r;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) a[k] = (float)u.h[k];
+    }
+    __device__ static uint4 narrow(const acc_t* a) {
+        U u;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) u.h[k] = (_Float16)a[k];
+        return u.r;
+    }
+    __device__ static acc_t widen1(const void* p, uint64_t i) { return (float)static_cast<const _Float16*>(p)[i]; }
+    __device__ static void narrow1(void* p, uint64_t i, acc_t v) { static_cast<_Float16*>(p)[i] = (_Float16)v; }
+};
+
+template <> struct Vec<double> {
+    static constexpr int V = 2;
+    using acc_t = double;
+    union U { uint4 r; double d[2]; };
+    __device__ static void widen(const uint4& r, acc_t* a) { U u; u.r = r; a[0] = u.d[0]; a[1] = u.d[1]; }
+    __device__ static uint4 narrow(const acc_t* a) { U u; u.d[0] = a[0]; u.d[1] = a[1]; return u.r; }
+    __device__ static acc_t widen1(const void* p, uint64_t i) { return static_cast<const double*>(p)[i]; }
+    __device__ static void narrow1(void* p, uint64_t i, acc_t v) { static_cast<double*>(p)[i] = v; }
+};
+
+// integers: wrapping sum in the unsigned type of the same width
+template <typename UT> struct IntVec {
+    static constexpr int V = 16 / sizeof(UT);
+    using acc_t = UT;
+    union U { uint4 r; UT e[V]; };
+    __device__ static void widen(const uint4& r, acc_t* a) {
+        U u; u.r = r;
+#pragma unroll
+        for (int k = 0; k < V; ++k) a[k] = u.e[k];
+    }
+    __device__ static uint4 narrow(const acc_t* a) {
+        U u;
+#pragma unroll
+        for (int k = 0; k < V; ++k) u.e[k] = a[k];
+        return u.r;
+    }
+    __device__ static acc_t widen1(const void* p, uint64_t i) { return static_cast<const UT*>(p)[i]; }
+    __device__ static void narrow1(void* p, uint64_t i, acc_t v) { static_cast<UT*>(p)[i] = v; }
+};
+template <> struct Vec<uint8_t> : IntVec<uint8_t> {};
+template <> struct Vec<uint32_t> : IntVec<uint32_t> {};
+template <> struct Vec<uint64_t> : IntVec<uint64_t> {};
+
+template <typename A> __device__ __forceinline__ A finish(A acc, bool avg, float scale, float divisor) {
+    if constexpr (std::is_same<A, float>::value) {
+        if (avg) return scale != 0.0f ? acc * scale : acc / divisor;
+    } else if constexpr (std::is_same<A, double>::value) {
+        if (avg) return acc / (double)divisor;
+    }
+    return acc;
+}
+
+// N > 0: compile-time input count (all loads hoisted); N == 0: runtime count, groups of 4.
+template <typename T, int N, bool AVG>
+__global__ __launch_bounds__(kThreads) void reduce_kernel(ReduceArgs a) {
+    using VT = Vec<T>;
+    using acc_t = typename VT::acc_t;
+    constexpr int V = VT::V;
+    const uint64_t nvec = a.numel / V;
+    const uint64_t stride = (uint64_t)gridDim.x * kThreads;
+    for (uint64_t v = (uint64_t)blockIdx.x * kThreads + threadIdx.x; v < nvec; v += stride) {
+        acc_t acc[V];
+        if constexpr (N > 0) {
+            uint4 raw[N];
+#pragma unroll
+            for (int r = 0; r < N; ++r) raw[r] = load16_unaligned(static_cast<const char*>(a.in[r]) + v * 16);
+            VT::widen(raw[0], acc);
+#pragma unroll
+            for (int r = 1; r < N; ++r) {
+                acc_t x[V];
+                VT::widen(raw[r], x);
+#pragma unroll
+                for (int k = 0; k < V; ++k) acc[k] += x[k];
+            }
+        } else {
+            VT::widen(load16_unaligned(static_cast<const char*>(a.in[0]) + v * 16), acc);
+            uint32_t r = 1;
+            for (; r + 4 <= a.n; r += 4) {
+                uint4 raw[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw[j] = load16_unaligned(static_cast<const char*>(a.in[r + j]) + v * 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc_t x[V];
+                    VT::widen(raw[j], x);
+#pragma unroll
+                    for (int k = 0; k < V; ++k) acc[k] += x[k];
+                }
+            }
+            for (; r < a.n; ++r) {
+                acc_t x[V];
+                VT::widen(load16_unaligned(static_cast<const char*>(a.in[r]) + v * 16), x);
+#pragma unroll
+                for (int k = 0; k < V; ++k) acc[k] += x[k];
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < V; ++k) acc[k] = finish(acc[k], AVG, a.scale, a.divisor);
+        store16_unaligned(static_cast<char*>(a.out) + v * 16, VT::narrow(acc));
+    }
+    // ragged tail: fewer than V elements, one lane each
+    if (blockIdx.x == 0) {
+        const uint64_t i = nvec * V + threadIdx.x;
+        if (threadIdx.x < V && i < a.numel) {
+            acc_t acc = VT::widen1(a.in[0], i);
+            for (uint32_t r = 1; r < a.n; ++r) acc += VT::widen1(a.in[r], i);
+            VT::narrow1(a.out, i, finish(acc, AVG, a.scale, a.divisor));
+        }
+    }
+}
+
+// ---------------- reduce + scatter ----------------
+
+struct ScatterArgs {
+    void* outs[kMaxOutputs];
+    uint64_t out_offset[kMaxOutputs];  // units into the reduced tensor's index space
+    const void* in[kMaxInputs];
+    uint64_t total;                    // units per output
+    uint64_t in_offset;                // units
+    uint32_t n_in;
+    float scale;
+    float divisor;
+    DimsArg out_dims;                  // packed output index -> reduced-tensor index
+    DimsArg in_dims;                   // reduced-tensor index -> input memory
+};
+
+// VEC: a unit is 16 bytes (V elements) and never straddles a row of either view.
+template <typename T, bool VEC, bool AVG, bool WIDE>
+__global__ __launch_bounds__(kThreads) void reduce_scatter_kernel(ScatterArgs a) {
+    using VT = Vec<T>;
+    using acc_t = typename VT::acc_t;
+    constexpr int V = VT::V;
+    const int k = blockIdx.y;
+    const uint64_t stride = (uint64_t)gridDim.x * kThreads;
+    for (uint64_t t = (uint64_t)blockIdx.x * kThreads + threadIdx.x; t < a.total; t += stride) {
+        uint64_t col;
+        const uint64_t i = a.out_offset[k] + decode<WIDE>(a.out_dims, t, &col);
+        const uint64_t loc = a.in_offset + decode<WIDE>(a.in_dims, i, &col);
+        if constexpr (VEC) {
+            acc_t acc[V];
+            VT::widen(load16_unaligned(static_cast<const char*>(a.in[0]) + loc * 16), acc);
+            uint32_t g = 1;
+            for (; g + 4 <= a.n_in; g += 4) {
+                uint4 raw[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) raw[j] = load16_unaligned(static_cast<const char*>(a.in[g + j]) + loc * 16);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc_t x[V];
+                    VT::widen(raw[j], x);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) acc[e] += x[e];
+                }
+            }
+            for (; g < a.n_in; ++g) {
+                acc_t x[V];
+                VT::widen(load16_unaligned(static_cast<const char*>(a.in[g]) + loc * 16), x);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] += x[e];
+            }
+#pragma unroll
+            for (int e = 0; e < V; ++e) acc[e] = finish(acc[e], AVG, a.scale, a.divisor);
+            store16_unaligned(static_cast<char*>(a.outs[k]) + t * 16, VT::narrow(acc));
+        } else {
+            acc_t acc = VT::widen1(a.in[0], loc);
+            for (uint32_t g = 1; g < a.n_in; ++g) acc += VT::widen1(a.in[g], loc);
+            VT::narrow1(a.outs[k], t, finish(acc, AVG, a.scale, a.divisor));
+        }
+    }
+}
+
+// ---------------- host side ----------------
+
+static uint32_t grid_for(uint64_t items) {
+    // one pass when it fits; otherwise a grid-stride loop over 64 blocks per CU
+    const uint64_t blocks = (items + kThreads - 1) / kThreads;
+    const uint64_t cap = 256ull * 64ull;
+    return (uint32_t)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+static int check_dtype_op(int dtype, int op) {
+    switch (dtype) {
+        case MHIP_DTYPE_F8E5M2: case MHIP_DTYPE_F8E4M3FN: case MHIP_DTYPE_F8E5M2FNUZ: case MHIP_DTYPE_F8E4M3FNUZ:
+            return MHIP_ERR_FLOAT8_REDUCTION;  // nccl.rs:474-476
+        case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: case MHIP_DTYPE_I32: case MHIP_DTYPE_I64:
+            if (op == MHIP_OP_AVG) return MHIP_ERR_UNSUPPORTED_OP;
+            break;
+        case MHIP_DTYPE_F16: case MHIP_DTYPE_F32: case MHIP_DTYPE_F64: case MHIP_DTYPE_BF16:
+            break;
+        default:
+            return MHIP_ERR_INVALID_DATA_TYPE;
+    }
+    if (op != MHIP_OP_SUM && op != MHIP_OP_AVG) return MHIP_ERR_UNSUPPORTED_OP;
+    return MHIP_SUCCESS;
+}
+
+static void avg_factors(uint32_t n, int op, float* scale, float* divisor) {
+    *divisor = (float)n;
+    *scale = (op == MHIP_OP_AVG && (n & (n - 1)) == 0) ? 1.0f / (float)n : 0.0f;
+}
+
+template <typename T, bool AVG>
+static void launch_reduce_n(const ReduceArgs& a, hipStream_t s) {
+    const dim3 grid(grid_for(a.numel / Vec<T>::V)), block(kThreads);
+    switch (a.n) {
+        case 1: hipLaunchKernelGGL((reduce_kernel<T, 1, AVG>), grid, block, 0, s, a); break;
+        case 2: hipLaunchKernelGGL((reduce_kernel<T, 2, AVG>), grid, block, 0, s, a); break;
+        case 4: hipLaunchKernelGGL((reduce_kernel<T, 4, AVG>), grid, block, 0, s, a); break;
+        case 8: hipLaunchKernelGGL((reduce_kernel<T, 8, AVG>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((reduce_kernel<T, 0, AVG>), grid, block, 0, s, a); break;
+    }
+}
+
+template <typename T>
+static void launch_reduce(const ReduceArgs& a, int op, hipStream_t s) {
+    if (op == MHIP_OP_AVG) launch_reduce_n<T, true>(a, s); else launch_reduce_n<T, false>(a, s);
+}
+
+template <typename T>
+static void launch_scatter(const ScatterArgs& a, dim3 grid, bool vec, bool avg, bool wide, hipStream_t s) {
+    const dim3 block(kThreads);
+#define MHIP_RS(VEC, AVG, WIDE) hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, WIDE>), grid, block, 0, s, a)
+    if (vec) {
+        if (avg) { if (wide) MHIP_RS(true, true, true); else MHIP_RS(true, true, false); }
+        else     { if (wide) MHIP_RS(true, false, true); else MHIP_RS(true, false, false); }
+    } else {
+        if (avg) { if (wide) MHIP_RS(false, true, true); else MHIP_RS(false, true, false); }
+        else     { if (wide) MHIP_RS(false, false, true); else MHIP_RS(false, false, false); }
+    }
+#undef MHIP_RS
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" {
+
+uint32_t mhip_dtype_size(int dtype) {
+    switch (dtype) {
+        case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: case MHIP_DTYPE_F8E5M2: case MHIP_DTYPE_F8E4M3FN:
+        case MHIP_DTYPE_F8E5M2FNUZ: case MHIP_DTYPE_F8E4M3FNUZ: return 1;
+        case MHIP_DTYPE_F16: case MHIP_DTYPE_BF16: return 2;
+        case MHIP_DTYPE_I32: case MHIP_DTYPE_F32: return 4;
+        case MHIP_DTYPE_I64: case MHIP_DTYPE_F64: return 8;
+        default: return 0;
+    }
+}
+
+int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, int dtype, int op,
+                mhip_stream_t stream) {
+    if (!in || n == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    if (int rc = check_dtype_op(dtype, op)) return rc;
+    if (n > (uint32_t)kMaxInputs) return MHIP_ERR_TOO_MANY_INPUTS;
+    if (numel == 0) return MHIP_SUCCESS;
+    if (!out) return MHIP_ERR_UNDEFINED_TENSOR;
+    const uint32_t esize = mhip_dtype_size(dtype);
+    ReduceArgs a{};
+    a.out = out;
+    uintptr_t align = (uintptr_t)out;
+    for (uint32_t r = 0; r < n; ++r) {
+        if (!in[r]) return MHIP_ERR_UNDEFINED_TENSOR;
+        a.in[r] = in[r];
+        align |= (uintptr_t)in[r];
+    }
+    if (align & (esize - 1)) return MHIP_ERR_INVALID_ARGUMENT;  // not even element-aligned
+    a.numel = numel;
+    a.n = n;
+    avg_factors(n, op, &a.scale, &a.divisor);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    switch (dtype) {
+        case MHIP_DTYPE_F32: launch_reduce<float>(a, op, hs); break;
+        case MHIP_DTYPE_BF16: launch_reduce<bf16_tag>(a, op, hs); break;
+        case MHIP_DTYPE_F16: launch_reduce<_Float16>(a, op, hs); break;
+        case MHIP_DTYPE_F64: launch_reduce<double>(a, op, hs); break;
+        case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_reduce<uint8_t>(a, op, hs); break;
+        case MHIP_DTYPE_I32: launch_reduce<uint32_t>(a, op, hs); break;
+        case MHIP_DTYPE_I64: launch_reduce<uint64_t>(a, op, hs); break;
+        default: return MHIP_ERR_INVALID_DATA_TYPE;
+    }
+    return launch_status();
+}
+
+int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32_t n_out, const void* const* in,
+                        const mhip_slice_t* in_view, uint64_t in_numel, uint32_t n_in, int dtype, int op,
+                        mhip_stream_t stream) {
+    if (!in || n_in == 0 || (n_out && (!outs || !out_views))) return MHIP_ERR_INVALID_ARGUMENT;
+    if (int rc = check_dtype_op(dtype, op)) return rc;
+    if (n_in > (uint32_t)kMaxInputs) return MHIP_ERR_TOO_MANY_INPUTS;
+    const uint32_t esize = mhip_dtype_size(dtype);
+    const uint32_t V = 16 / esize;
+
+    // the reduced tensor's index space
+    const uint64_t one = in_numel, unit_stride = 1;
+    mhip_slice_t dense{0, 1, &one, &unit_stride};
+    const mhip_slice_t& iv = in_view ? *in_view : dense;
+    if (iv.ndim > MHIP_MAX_DIMS || (iv.ndim && (!iv.sizes || !iv.strides))) return MHIP_ERR_INVALID_ARGUMENT;
+    if (int rc = validate_slice(iv.sizes, iv.ndim, iv.strides, iv.ndim)) return rc;
+    const uint64_t reduced_len = slice_len(iv);
+
+    uintptr_t in_align = 0;
+    for (uint32_t g = 0; g < n_in; ++g) {
+        if (!in[g]) return MHIP_ERR_UNDEFINED_TENSOR;
+        in_align |= (uintptr_t)in[g];
+    }
+    if (in_align & (esize - 1)) return MHIP_ERR_INVALID_ARGUMENT;
+
+    for (uint32_t k = 0; k < n_out; ++k) {
+        const mhip_slice_t& ov = out_views[k];
+        if (ov.ndim > MHIP_MAX_DIMS || (ov.ndim && (!ov.sizes || !ov.strides))) return MHIP_ERR_INVALID_ARGUMENT;
+        if (int rc = validate_slice(ov.sizes, ov.ndim, ov.strides, ov.ndim)) return rc;
+        const uint64_t len = slice_len(ov);
+        if (len == 0) continue;
+        if (!outs[k]) return MHIP_ERR_UNDEFINED_TENSOR;
+        if ((uintptr_t)outs[k] & (esize - 1)) return MHIP_ERR_INVALID_ARGUMENT;
+        uint64_t hi = ov.offset;
+        for (uint32_t d = 0; d < ov.ndim; ++d) hi += (ov.sizes[d] - 1) * ov.strides[d];
+        if (hi >= reduced_len) return MHIP_ERR_INPUT_SIZE_MISMATCH;  // view reaches outside the reduced tensor
+    }
+
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    float scale, divisor;
+    avg_factors(n_in, op, &scale, &divisor);
+
+    uint32_t k = 0;
+    while (k < n_out) {
+        if (slice_len(out_views[k]) == 0) { ++k; continue; }
+        // Vector form: units of V elements on both views and 16-byte aligned pointers.
+        // Slices are canonicalised with elem_size 1, i.e. in elements; the alignment mask
+        // carries the pointers divided by the element size.
+        uint32_t max_unit = V;
+        CanonSlice oc, ic;
+        uint32_t ou = 1, iu = 1;
+        for (;;) {
+            const uint64_t omask = ((uintptr_t)outs[k] / esize);
+            const uint64_t imask = (in_align / esize) | 0;  // pointers only
+            canonicalize(out_views[k], 1, omask, max_unit, &oc, &ou);
+            canonicalize(iv, 1, imask, max_unit, &ic, &iu);
+            if (max_unit == 1 || (ou == V && iu == V)) break;
+            max_unit = 1;  // fall back to element granularity for both
+        }
+        // out view offsets are into the reduced index space: with unit u they must be
+        // whole units too, which canonicalize guarantees by folding offset into the mask.
+        const bool vec = max_unit == V;
+        ScatterArgs a{};
+        bool o32 = false, i32 = false;
+        if (!make_dims_arg(oc, &a.out_dims, &o32) || !make_dims_arg(ic, &a.in_dims, &i32))
+            return MHIP_ERR_UNSUPPORTED_OP;
+        // the output decode yields reduced-tensor indices that the input decode divides again
+        const bool wide = !(o32 && i32 && ic.total < kFastDivLimit - 64);
+        a.total = oc.total;
+        a.in_offset = ic.offset;
+        a.n_in = n_in;
+        a.scale = scale;
+        a.divisor = divisor;
+        for (uint32_t g = 0; g < n_in; ++g) a.in[g] = in[g];
+        a.outs[0] = outs[k];
+        a.out_offset[0] = oc.offset;
+        uint32_t nbatch = 1;
+        while (k + nbatch < n_out && nbatch < (uint32_t)kMaxOutputs) {
+            CanonSlice nc;
+            uint32_t nu = 1;
+            if (!canonicalize(out_views[k + nbatch], 1, (uintptr_t)outs[k + nbatch] / esize, max_unit, &nc, &nu)) break;
+            if (nu != ou || !same_shape(oc, nc)) break;
+            a.outs[nbatch] = outs[k + nbatch];
+            a.out_offset[nbatch] = nc.offset;
+            ++nbatch;
+        }
+        dim3 grid(grid_for(a.total), nbatch);
+        const bool avg = op == MHIP_OP_AVG;
+        switch (dtype) {
+            case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_BF16: launch_scatter<bf16_tag>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_F16: launch_scatter<_Float16>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_F64: launch_scatter<double>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_scatter<uint8_t>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_I32: launch_scatter<uint32_t>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_I64: launch_scatter<uint64_t>(a, grid, vec, avg, wide, hs); break;
+            default: return MHIP_ERR_INVALID_DATA_TYPE;
+        }
+        if (int rc = launch_status()) return rc;
+        k += nbatch;
+    }
+    return MHIP_SUCCESS;
+}
+
+}  // extern "C"

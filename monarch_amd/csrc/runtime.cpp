@@ -1,0 +1,90 @@
+// Runtime pass-through and error text: the small part of the HIP runtime that the
+// data path's callers reach through this library instead of through cuda-sys/nccl-sys.
+#include <hip/hip_runtime.h>
+
+#include "mhip_internal.h"
+
+#define MHIP_VERSION 100
+
+extern "C" {
+
+const char* mhip_error_string(int status) {
+    switch (status) {
+        case MHIP_SUCCESS: return "success";
+        case MHIP_ERR_INVALID_DIMS: return "invalid dims: sizes and strides differ in length";
+        case MHIP_ERR_NONRECTANGULAR_SHAPE: return "nonrectangular shape";
+        case MHIP_ERR_NONUNIQUE_STRIDES: return "nonunique strides";
+        case MHIP_ERR_STRIDE_TOO_SMALL: return "stride must be larger than size of previous space";
+        case MHIP_ERR_INDEX_OUT_OF_RANGE: return "index out of range";
+        case MHIP_ERR_VALUE_NOT_IN_SLICE: return "value not in slice";
+        case MHIP_ERR_INCOMPATIBLE_VIEW: return "incompatible view";
+        case MHIP_ERR_NONCONTIGUOUS: return "noncontiguous shape";
+        case MHIP_ERR_EMPTY_RANGE: return "empty range";
+        case MHIP_ERR_DIMENSION_OUT_OF_RANGE: return "dimension out of range";
+        case MHIP_ERR_INVALID_DATA_TYPE: return "invalid data type for a reduction";
+        case MHIP_ERR_NONCONTIGUOUS_TENSOR: return "tensor used in collective must be contiguous";
+        case MHIP_ERR_INVALID_DEVICE: return "tensor must be on a GPU device";
+        case MHIP_ERR_FLOAT8_REDUCTION: return "float8 dtypes are not currently supported for reductions";
+        case MHIP_ERR_TYPE_MISMATCH: return "output tensor must have the same type as input tensor";
+        case MHIP_ERR_OUTPUT_SIZE_MISMATCH: return "output tensor size must be equal to world size times input tensor size";
+        case MHIP_ERR_INPUT_SIZE_MISMATCH: return "input tensor must be the same size as output size times world size";
+        case MHIP_ERR_UNDEFINED_TENSOR: return "undefined tensor (null pointer) used for operation";
+        case MHIP_ERR_INVALID_ARGUMENT: return "an argument has an invalid value";
+        case MHIP_ERR_UNSUPPORTED_OP: return "reduction op not supported for this dtype (Sum and Avg only; Avg on floating types)";
+        case MHIP_ERR_TOO_MANY_INPUTS: return "too many inputs for one reduce (at most 64)";
+        case MHIP_ERR_UNSUPPORTED_BLOCK: return "unsupported fp8 scale block (must be 1024)";
+        default: break;
+    }
+    if (status > 0 && status < 10000) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown status";
+}
+
+int mhip_version(void) { return MHIP_VERSION; }
+
+int mhip_device_count(int* count) { return count ? (int)hipGetDeviceCount(count) : MHIP_ERR_INVALID_ARGUMENT; }
+int mhip_set_device(int device) { return (int)hipSetDevice(device); }
+int mhip_device_synchronize(void) { return (int)hipDeviceSynchronize(); }
+
+int mhip_stream_create(mhip_stream_t* stream) {
+    if (!stream) return MHIP_ERR_INVALID_ARGUMENT;
+    hipStream_t s = nullptr;
+    hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
+    *stream = s;
+    return (int)e;
+}
+int mhip_stream_destroy(mhip_stream_t stream) { return (int)hipStreamDestroy(static_cast<hipStream_t>(stream)); }
+int mhip_stream_synchronize(mhip_stream_t stream) { return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream)); }
+
+int mhip_event_create(mhip_event_t* event) {
+    if (!event) return MHIP_ERR_INVALID_ARGUMENT;
+    hipEvent_t e = nullptr;
+    hipError_t rc = hipEventCreate(&e);
+    *event = e;
+    return (int)rc;
+}
+int mhip_event_destroy(mhip_event_t event) { return (int)hipEventDestroy(static_cast<hipEvent_t>(event)); }
+int mhip_event_record(mhip_event_t event, mhip_stream_t stream) {
+    return (int)hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream));
+}
+int mhip_event_synchronize(mhip_event_t event) { return (int)hipEventSynchronize(static_cast<hipEvent_t>(event)); }
+int mhip_event_elapsed_ms(float* ms, mhip_event_t start, mhip_event_t stop) {
+    if (!ms) return MHIP_ERR_INVALID_ARGUMENT;
+    return (int)hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop));
+}
+int mhip_stream_wait_event(mhip_stream_t stream, mhip_event_t event) {
+    return (int)hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0);
+}
+
+int mhip_malloc(void** ptr, size_t bytes) { return ptr ? (int)hipMalloc(ptr, bytes) : MHIP_ERR_INVALID_ARGUMENT; }
+int mhip_free(void* ptr) { return (int)hipFree(ptr); }
+int mhip_memcpy_htod(void* dst, const void* src, size_t bytes, mhip_stream_t stream) {
+    return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
+}
+int mhip_memcpy_dtoh(void* dst, const void* src, size_t bytes, mhip_stream_t stream) {
+    return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
+}
+int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream) {
+    return (int)hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,98 @@
+"""Block-scaled fp8 (e4m3fn, one fp32 absmax scale per 1024 elements) transfer codec and the
+flat bucket it runs on.
+
+The reference ships fp8 tensors as raw bytes and refuses to reduce them
+(torch-sys-cuda/src/nccl.rs:275-278,474-476); this codec is what makes a compressed
+gradient exchange possible on that path: pack ragged tensors into one flat bf16 buffer
+(the torch.cat / split idiom of python/tests/simulator/test_simulator.py:190-203),
+quantise, move 1 byte per element plus 4 bytes per block, dequantise-and-accumulate
+into an fp32 buffer, unpack.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from . import _torch
+from ._lib import check, lib
+
+BLOCK = 1024
+FP8_MAX = 448.0
+
+
+class FlatBucket:
+    """Offsets table and device pointer table for a list of ragged tensors."""
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        if not tensors:
+            raise ValueError("a bucket needs at least one tensor")
+        self.dtype = tensors[0].dtype
+        self.device = tensors[0].device
+        for t in tensors:
+            _torch.require_contiguous(t)
+            if t.dtype != self.dtype:
+                raise ValueError("all tensors of a bucket must share a dtype")
+        self.sizes = [t.numel() for t in tensors]
+        self.offsets = [0]
+        for n in self.sizes:
+            self.offsets.append(self.offsets[-1] + n)
+        self.total = self.offsets[-1]
+        # device-resident tables, uploaded once and reused by every pack / unpack
+        self.d_offsets = torch.tensor(self.offsets, dtype=torch.int64, device=self.device)
+        self.d_ptrs = self.pointer_table(tensors)
+
+    def pointer_table(self, tensors: Sequence[torch.Tensor]) -> torch.Tensor:
+        if [t.numel() for t in tensors] != self.sizes:
+            raise ValueError("tensor sizes do not match the bucket")
+        return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device=self.device)
+
+    def pack(self, flat: torch.Tensor = None, d_ptrs: torch.Tensor = None, stream=None) -> torch.Tensor:
+        """flat[offsets[t] + j] = tensors[t][j]"""
+        if flat is None:
+            flat = torch.empty(self.total, dtype=self.dtype, device=self.device)
+        ptrs = self.d_ptrs if d_ptrs is None else d_ptrs
+        check(lib().mhip_flat_pack(flat.data_ptr(), ptrs.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
+                                   self.total, flat.element_size(), _torch.stream_handle(stream)))
+        return flat
+
+    def unpack(self, flat: torch.Tensor, outs: Sequence[torch.Tensor], stream=None) -> None:
+        """outs[t][j] = flat[offsets[t] + j]; ``flat`` may have any dtype of the outs' element size."""
+        for t in outs:
+            _torch.require_contiguous(t)
+            if t.element_size() != flat.element_size():
+                raise ValueError("element size mismatch")
+        ptrs = self.pointer_table(outs)
+        check(lib().mhip_flat_unpack(ptrs.data_ptr(), flat.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
+                                     self.total, flat.element_size(), _torch.stream_handle(stream)))
+        # keep the table alive until the launch that reads it has been enqueued and ordered
+        # behind later work on the same stream
+        self._last_unpack_table = ptrs
+
+
+def quantize(flat_bf16: torch.Tensor, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None):
+    """Returns ``(q uint8[numel], scales f32[ceil(numel/1024)])``."""
+    _torch.require_contiguous(flat_bf16)
+    if flat_bf16.dtype != torch.bfloat16:
+        raise ValueError("quantize expects a bf16 buffer")
+    n = flat_bf16.numel()
+    nb = (n + BLOCK - 1) // BLOCK
+    if q is None:
+        q = torch.empty(n, dtype=torch.uint8, device=flat_bf16.device)
+    if scales is None:
+        scales = torch.empty(nb, dtype=torch.float32, device=flat_bf16.device)
+    check(lib().mhip_fp8_quantize(q.data_ptr(), scales.data_ptr(), flat_bf16.data_ptr(), n, BLOCK,
+                                  _torch.stream_handle(stream)))
+    return q, scales
+
+
+def dequant_accumulate(acc: torch.Tensor, q: torch.Tensor, scales: torch.Tensor, stream=None) -> None:
+    """acc[i] += float(q[i]) * scales[i // 1024] (fp32, product rounded before the add)."""
+    for t in (acc, q, scales):
+        _torch.require_contiguous(t)
+    if acc.dtype != torch.float32 or scales.dtype != torch.float32 or q.element_size() != 1:
+        raise ValueError("acc and scales must be fp32 and q one byte per element")
+    if acc.numel() != q.numel() or scales.numel() != (q.numel() + BLOCK - 1) // BLOCK:
+        raise ValueError("size mismatch between acc, q and scales")
+    check(lib().mhip_fp8_dequant_accumulate(acc.data_ptr(), q.data_ptr(), scales.data_ptr(), q.numel(), BLOCK,
+                                            _torch.stream_handle(stream)))

@@ -1,0 +1,155 @@
+"""Staging transfers: Slice views <-> contiguous ``RDMABuffer`` bytes on one GPU.
+
+``RDMABuffer`` keeps the reference's contract (python/monarch/_src/tensor_engine/rdma.py:80-207):
+it only accepts 1-D contiguous ``uint8`` memory and moves flat byte ranges
+(monarch_rdma/src/rdma_components.rs:94-171).  ``TensorBuffer`` is the API that file
+leaves as a TODO (rdma.py:91-97): a non-contiguous, multi-byte-per-element tensor view is
+gathered into such a buffer in ``Slice::iter`` order before ``read_into`` and scattered
+back after ``write_from``.  All data movement happens in the library's HIP kernels.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _torch
+from ._lib import check, lib, ptr_array
+from .ndslice import Slice, slice_array
+
+
+def _assert_tensor_is_1d_contiguous_uint8(t: torch.Tensor) -> None:
+    # rdma.py:80-86, same messages
+    if t.ndim != 1:
+        raise ValueError(f"Tensor must be 1D, got {t.ndim}D")
+    if t.dtype != torch.uint8:
+        raise ValueError(f"Tensor must be uint8, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError("Tensor must be contiguous")
+
+
+def _check_view_fits(base: torch.Tensor, s: Slice) -> None:
+    if len(s) == 0:
+        return
+    _, hi = s.bounds()
+    storage_elems = base.untyped_storage().nbytes() // base.element_size()
+    if hi >= storage_elems:
+        raise ValueError(f"slice reaches element {hi} but the storage holds {storage_elems}")
+
+
+def pack(base: torch.Tensor, s: Slice, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """``out[i] = storage(base)[s.get(i)]``; returns a 1-D tensor of ``base.dtype``."""
+    _torch.require_device(base)
+    _check_view_fits(base, s)
+    n = len(s)
+    if out is None:
+        out = torch.empty(n, dtype=base.dtype, device=base.device)
+    elif out.numel() * out.element_size() != n * base.element_size() or not out.is_contiguous():
+        raise ValueError("staging buffer must be contiguous and hold exactly len(slice) elements")
+    check(lib().mhip_slice_pack(out.data_ptr(), _torch.storage_ptr(base), C.byref(s.c), base.element_size(),
+                                _torch.stream_handle(stream)))
+    return out
+
+
+def unpack(base: torch.Tensor, s: Slice, src: torch.Tensor, stream=None) -> None:
+    """``storage(base)[s.get(i)] = src[i]``; elements outside the view keep their values."""
+    _torch.require_device(base)
+    _torch.require_contiguous(src)
+    _check_view_fits(base, s)
+    if src.numel() * src.element_size() != len(s) * base.element_size():
+        raise ValueError("staging buffer must hold exactly len(slice) elements")
+    check(lib().mhip_slice_unpack(_torch.storage_ptr(base), src.data_ptr(), C.byref(s.c), base.element_size(),
+                                  _torch.stream_handle(stream)))
+
+
+def pack_many(base: torch.Tensor, views: Sequence[Slice], outs: Optional[List[torch.Tensor]] = None,
+              stream=None) -> List[torch.Tensor]:
+    """Packs several views of one tensor (a reshard's column blocks) in as few launches as possible."""
+    _torch.require_device(base)
+    for s in views:
+        _check_view_fits(base, s)
+    if outs is None:
+        outs = [torch.empty(len(s), dtype=base.dtype, device=base.device) for s in views]
+    arr = slice_array(views)
+    check(lib().mhip_slice_pack_many(ptr_array([o.data_ptr() for o in outs]), _torch.storage_ptr(base), arr,
+                                     len(views), base.element_size(), _torch.stream_handle(stream)))
+    return outs
+
+
+def unpack_many(base: torch.Tensor, views: Sequence[Slice], srcs: Sequence[torch.Tensor], stream=None) -> None:
+    _torch.require_device(base)
+    for s, src in zip(views, srcs):
+        _check_view_fits(base, s)
+        _torch.require_contiguous(src)
+        if src.numel() * src.element_size() != len(s) * base.element_size():
+            raise ValueError("staging buffer must hold exactly len(slice) elements")
+    arr = slice_array(views)
+    check(lib().mhip_slice_unpack_many(_torch.storage_ptr(base), ptr_array([t.data_ptr() for t in srcs]), arr,
+                                       len(views), base.element_size(), _torch.stream_handle(stream)))
+
+
+class RDMABuffer:
+    """A registered contiguous byte range ``{addr, size}`` (rdma_components.rs:94-102).
+
+    On one GPU the transport is a flat device copy; the names keep the reference's
+    direction: ``buf.read_into(dst)`` copies the buffer's bytes into ``dst`` and
+    ``buf.write_from(src)`` copies ``src`` into the buffer.
+    """
+
+    def __init__(self, data: torch.Tensor) -> None:
+        _assert_tensor_is_1d_contiguous_uint8(data)
+        _torch.require_device(data)
+        self._data = data
+        self.addr = data.data_ptr()
+        self.size = data.numel()
+
+    @property
+    def data(self) -> torch.Tensor:
+        return self._data
+
+    def _copy(self, dst_ptr: int, src_ptr: int, nbytes: int, stream) -> None:
+        flat = Slice.new_row_major([nbytes])
+        check(lib().mhip_slice_pack(dst_ptr, src_ptr, C.byref(flat.c), 1, _torch.stream_handle(stream)))
+
+    def read_into(self, dst: torch.Tensor, offset: int = 0, stream=None) -> int:
+        _assert_tensor_is_1d_contiguous_uint8(dst)
+        _torch.require_device(dst)
+        size = dst.numel()
+        if offset + size > self.size:
+            raise ValueError(f"offset + size ({offset + size}) must be <= buffer size ({self.size})")
+        self._copy(dst.data_ptr(), self.addr + offset, size, stream)
+        return size
+
+    def write_from(self, src: torch.Tensor, offset: int = 0, stream=None) -> None:
+        _assert_tensor_is_1d_contiguous_uint8(src)
+        _torch.require_device(src)
+        size = src.numel()
+        if size + offset > self.size:
+            raise ValueError(f"size + offset ({size + offset}) must be <= buffer size ({self.size})")
+        self._copy(self.addr + offset, src.data_ptr(), size, stream)
+
+
+class TensorBuffer:
+    """A tensor view staged through an ``RDMABuffer``: pack before the transfer out,
+    unpack after the transfer in."""
+
+    def __init__(self, view: torch.Tensor, staging: Optional[torch.Tensor] = None) -> None:
+        _torch.require_device(view)
+        self.view = view
+        self.slice = Slice.of_tensor(view)
+        nbytes = len(self.slice) * view.element_size()
+        if staging is None:
+            staging = torch.empty(nbytes, dtype=torch.uint8, device=view.device)
+        self.buffer = RDMABuffer(staging)
+        if self.buffer.size != nbytes:
+            raise ValueError(f"staging buffer holds {self.buffer.size} bytes, the view needs {nbytes}")
+
+    def stage(self, stream=None) -> RDMABuffer:
+        """Gather the view into the staging bytes (call before ``buffer.read_into``)."""
+        pack(self.view, self.slice, out=self.buffer.data, stream=stream)
+        return self.buffer
+
+    def commit(self, stream=None) -> None:
+        """Scatter the staging bytes back into the view (call after ``buffer.write_from``)."""
+        unpack(self.view, self.slice, self.buffer.data, stream=stream)

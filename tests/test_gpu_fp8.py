@@ -1,0 +1,181 @@
+"""GPU parity: block-scaled fp8 codec and flat bucket pack/unpack against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from monarch_amd import fp8
+from util import bits, sync
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _c5_like(n, seed, device="cpu"):
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn(n, generator=g, device=device)
+    out = torch.rand(n, generator=g, device=device) < 1e-3
+    return torch.where(out, x * 50, x).bfloat16()
+
+
+def _check_quant(x: torch.Tensor):
+    q, s = fp8.quantize(x.to(DEV))
+    sync()
+    wq, ws = oracle.fp8_quantize(bits(x), 1024)
+    gq = q.cpu().numpy()
+    nan = (wq & 0x7F) == 0x7F
+    assert np.array_equal((gq & 0x7F) == 0x7F, nan)
+    assert np.array_equal(gq[~nan], wq[~nan])
+    assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
+    return q, s
+
+
+def test_every_bf16_pattern_at_unit_scale():
+    # blocks whose absmax is exactly 448 have inv == 1: the codes are the bare e4m3fn RNE conversion of
+    # every finite bf16 value up to 448 (pinned against the format via the oracle's torch-checked encoder)
+    h = torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16)
+    vals = h[(h.float().abs() <= 448) & ~h.float().isnan()]
+    per = 1023
+    nblk = (vals.numel() + per - 1) // per
+    x = torch.zeros(nblk * 1024, dtype=torch.bfloat16)
+    xv = x.view(nblk, 1024)
+    xv[:, 0] = 448.0
+    pad = torch.zeros(nblk * per, dtype=torch.bfloat16)
+    pad[: vals.numel()] = vals
+    xv[:, 1:] = pad.view(nblk, per)
+    q, s = _check_quant(x)
+    assert torch.all(s == 1.0)
+    direct = np.array([oracle.e4m3fn_encode(float(v), True) for v in x.float().numpy()], dtype=np.uint8)
+    assert np.array_equal(q.cpu().numpy(), direct)
+
+
+def test_every_bf16_pattern_mixed_scales():
+    h = torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16)
+    g = torch.Generator().manual_seed(0)
+    perm = torch.randperm(65536, generator=g)
+    _check_quant(h[perm])            # NaN / Inf blocks take the careful path
+    finite = h[~h.float().isnan() & ~h.float().isinf()]
+    _check_quant(finite[torch.randperm(finite.numel(), generator=g)])
+    _check_quant(finite.sort().values)  # blocks of similar magnitude, including all-denormal ones
+
+
+def test_edge_blocks():
+    z = torch.zeros(2048, dtype=torch.bfloat16)
+    z[1024:] = -0.0
+    q, s = _check_quant(z)
+    assert torch.all(q[:1024] == 0) and torch.all(q[1024:] == 0x80)
+    x = torch.ones(4096, dtype=torch.bfloat16)
+    x[3] = float("nan")
+    x[5] = -2.0
+    x[1024 + 7] = float("inf")
+    x[1024 + 8] = float("-inf")
+    x[2048 + 10] = 50.0
+    x[3072:] = 1e-30
+    q, s = _check_quant(x)
+    qc = q.cpu()
+    assert (qc[3] & 0x7F) == 0x7F and qc[5] == 0xFE and qc[1024 + 7] == 0x7E and qc[1024 + 8] == 0xFE
+    for n in (1, 5, 1023, 1025, 2047, 4097):  # short tails
+        _check_quant(_c5_like(n, seed=n))
+
+
+def test_quantize_dequant_accumulate_ragged():
+    g = torch.Generator().manual_seed(5000)
+    sizes = torch.exp(torch.rand(40, generator=g) * (np.log(2**17) - np.log(2**10)) + np.log(2**10)).round().long().tolist()
+    sizes += [1, 2, 1024, 1023, 1025]
+    tensors = [_c5_like(n, seed=5000 + i) for i, n in enumerate(sizes)]
+    dev = [t.to(DEV) for t in tensors]
+    bucket = fp8.FlatBucket(dev)
+    flat = bucket.pack()
+    sync()
+    hflat = oracle.flat_pack([bits(t) for t in tensors], bucket.offsets)
+    assert np.array_equal(bits(flat), hflat)
+    q, s = fp8.quantize(flat)
+    sync()
+    wq, ws = oracle.fp8_quantize(hflat, 1024)
+    assert np.array_equal(q.cpu().numpy(), wq) and np.array_equal(s.cpu().numpy(), ws)
+    rng = np.random.default_rng(1)
+    acc_h = rng.normal(size=bucket.total).astype(np.float32)
+    acc = torch.from_numpy(acc_h.copy()).to(DEV)
+    for _ in range(3):  # accumulate the same payload three times
+        fp8.dequant_accumulate(acc, q, s)
+        oracle.fp8_dequant_accumulate(acc_h, wq, ws, 1024)
+    sync()
+    assert np.array_equal(acc.cpu().numpy().view(np.uint32), acc_h.view(np.uint32))
+    outs = [torch.empty(n, dtype=torch.float32, device=DEV) for n in sizes]
+    bucket.unpack(acc, outs)
+    sync()
+    want = oracle.flat_unpack(acc_h, bucket.offsets)
+    for o, w in zip(outs, want):
+        assert np.array_equal(o.cpu().numpy(), w)
+
+
+def test_flat_pack_alignment_and_empty_tensors():
+    g = torch.Generator().manual_seed(3)
+    for dtype, sizes in ((torch.uint8, [3, 0, 17, 1, 4096, 0, 5]), (torch.bfloat16, [1, 3, 0, 8, 1025, 7]),
+                         (torch.float32, [5, 1, 0, 2049]), (torch.float64, [3, 1, 1000])):
+        tensors = [torch.randint(0, 255, (n,), generator=g).to(dtype) for n in sizes]
+        store = [torch.zeros(n + 4, dtype=dtype, device=DEV) for n in sizes]
+        dev = []
+        for i, (t, st) in enumerate(zip(tensors, store)):
+            v = st[i % 3: i % 3 + t.numel()]  # staggered, only element-aligned
+            v.copy_(t)
+            dev.append(v)
+        bucket = fp8.FlatBucket(dev)
+        for shift in (0, 1, 3):  # flat buffer alignment
+            fstore = torch.zeros(bucket.total + 8, dtype=dtype, device=DEV)
+            flat = fstore[shift: shift + bucket.total]
+            bucket.pack(flat)
+            sync()
+            want = oracle.flat_pack([bits(t) for t in tensors], bucket.offsets)
+            assert np.array_equal(bits(flat), want)
+            assert fstore[:shift].abs().sum() == 0 and fstore[shift + bucket.total:].abs().sum() == 0
+            outs = [torch.zeros(n + 2, dtype=dtype, device=DEV)[1: 1 + n] for n in sizes]
+            bucket.unpack(flat, outs)
+            sync()
+            for o, t in zip(outs, tensors):
+                assert torch.equal(o.cpu(), t)
+
+
+def test_config5_full_size_properties():
+    # 1500 tensors, log-uniform sizes in [2^10, 2^22]; checked through size-independent properties on the
+    # GPU plus the oracle on a sample of blocks
+    rng = np.random.default_rng(5000)
+    sizes = np.round(np.exp(rng.uniform(np.log(2**10), np.log(2**22), size=1500))).astype(np.int64).tolist()
+    total = sum(sizes)
+    big = _c5_like(total, seed=5001, device=DEV)  # one draw, carved into the 1500 tensors
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    tensors = [big[offs[i]: offs[i + 1]].clone() for i in range(1500)]
+    bucket = fp8.FlatBucket(tensors)
+    flat = bucket.pack()
+    sync()
+    assert torch.equal(flat.view(torch.int16), big.view(torch.int16))
+    q, s = fp8.quantize(flat)
+    sync()
+    nb = s.numel()
+    pad = nb * 1024 - total
+    xf = torch.cat([flat.float(), torch.zeros(pad, device=DEV)]).view(nb, 1024)
+    amax = xf.abs().amax(1)
+    assert torch.equal(s, amax / 448.0)
+    qp = torch.cat([q, torch.zeros(pad, dtype=torch.uint8, device=DEV)]).view(nb, 1024)
+    assert torch.all((qp & 0x7F).amax(1) == 0x7E)  # every block's largest magnitude maps to +-448
+    xhat = qp.view(torch.float8_e4m3fn).float() * s[:, None]
+    code_e = ((qp & 0x7F) >> 3).float()
+    spacing = torch.where(code_e == 0, torch.tensor(2.0**-9, device=DEV), torch.exp2(code_e - 10))
+    assert torch.all((xf - xhat).abs() <= 0.5 * spacing * s[:, None] * 1.001)
+    acc = torch.zeros(total, dtype=torch.float32, device=DEV)
+    fp8.dequant_accumulate(acc, q, s)
+    fp8.dequant_accumulate(acc, q, s)
+    sync()
+    assert torch.equal(acc, (xhat.view(-1)[:total] + xhat.view(-1)[:total]))  # x + x is exact
+    # oracle on sampled blocks (first, last, and every 997th)
+    hflat, hq, hs = bits(flat), q.cpu().numpy(), s.cpu().numpy()
+    for b in sorted(set([0, nb - 1, nb - 2] + list(range(0, nb, 997)))):
+        lo, hi = b * 1024, min((b + 1) * 1024, total)
+        wq, ws = oracle.fp8_quantize(hflat[lo:hi], 1024)
+        assert np.array_equal(hq[lo:hi], wq) and hs[b] == ws[0]
+    outs = [torch.empty(n, dtype=torch.float32, device=DEV) for n in sizes]
+    bucket.unpack(acc, outs)
+    sync()
+    for i in (0, 1, 749, 1498, 1499):
+        assert torch.equal(outs[i], acc[offs[i]: offs[i + 1]])
+    assert torch.equal(torch.cat(outs), acc)

@@ -1,0 +1,229 @@
+"""GPU parity: mhip_slice_pack / unpack (+ _many) against the CPU oracle, bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from monarch_amd import Slice, staging
+from util import bits, fuzz_slices, oslice, span, sync
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _storage(nbytes, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, 256, (nbytes,), dtype=torch.uint8, generator=g)
+
+
+def _roundtrip(s: Slice, elem_size: int, seed: int, misalign: int = 0, dst_misalign: int = 0):
+    """pack and unpack one slice of `elem_size`-byte elements; compare with the oracle bytes."""
+    n_elems = span(s)
+    host = _storage((n_elems + 2) * elem_size + misalign, seed)
+    dev = host.to(DEV)
+    base = dev[misalign: misalign + n_elems * elem_size]
+    hbase = host.numpy()[misalign: misalign + n_elems * elem_size]
+    n = len(s)
+    # oracle works on structured elements of elem_size bytes
+    dt = np.dtype((np.void, elem_size))
+    want = oracle.pack(hbase.view(dt), oslice(s)).view(np.uint8)
+    out_store = torch.full((n * elem_size + dst_misalign + 32,), 0xAB, dtype=torch.uint8, device=DEV)
+    out = out_store[dst_misalign: dst_misalign + n * elem_size]
+    from monarch_amd._lib import check, lib
+    import ctypes as C
+    check(lib().mhip_slice_pack(out.data_ptr(), base.data_ptr(), C.byref(s.c), elem_size,
+                                torch.cuda.current_stream().cuda_stream))
+    sync()
+    got = out_store.cpu().numpy()
+    assert np.array_equal(got[dst_misalign: dst_misalign + n * elem_size], want), (s, elem_size, misalign)
+    assert np.all(got[:dst_misalign] == 0xAB) and np.all(got[dst_misalign + n * elem_size:] == 0xAB)
+    # unpack into a canvas of 0x5C: view positions get the packed bytes, the rest stays
+    canvas = torch.full_like(dev, 0x5C)
+    cbase = canvas[misalign: misalign + n_elems * elem_size]
+    check(lib().mhip_slice_unpack(cbase.data_ptr(), out.data_ptr(), C.byref(s.c), elem_size,
+                                  torch.cuda.current_stream().cuda_stream))
+    sync()
+    hcanvas = np.full(host.numel(), 0x5C, dtype=np.uint8)
+    oracle.unpack(hcanvas[misalign: misalign + n_elems * elem_size].view(dt), want.view(dt), oslice(s))
+    assert np.array_equal(canvas.cpu().numpy(), hcanvas), (s, elem_size, misalign)
+
+
+NAMED = [
+    dict(offset=0, sizes=[3, 4], strides=[4, 1]),
+    dict(offset=0, sizes=[3, 4], strides=[1, 4]),        # column-major: a transpose
+    dict(offset=1, sizes=[3], strides=[2]),
+    dict(offset=1, sizes=[3, 3], strides=[12, 2]),
+    dict(offset=0, sizes=[4, 3, 8], strides=[48, 16, 2]),
+    dict(offset=24, sizes=[4, 3, 8], strides=[96, 16, 2]),
+    dict(offset=37, sizes=[], strides=[]),               # 0-d: one element
+    dict(offset=0, sizes=[2, 2, 2], strides=[4, 32, 1]),
+    dict(offset=10, sizes=[10, 2], strides=[10, 5]),
+    dict(offset=5, sizes=[3, 0], strides=[1, 3]),        # empty: nothing moves
+    dict(offset=3, sizes=[1, 1, 7], strides=[1, 1, 1]),
+    dict(offset=0, sizes=[64, 100], strides=[128, 1]),   # runs of 100 elements, not a multiple of 16 bytes
+    dict(offset=7, sizes=[33, 50], strides=[64, 1]),
+]
+
+
+@pytest.mark.parametrize("elem_size", [1, 2, 4, 8, 16, 3, 6, 12])
+def test_named_slices(elem_size):
+    for i, kw in enumerate(NAMED):
+        _roundtrip(Slice(**kw), elem_size, seed=i)
+
+
+@pytest.mark.parametrize("elem_size", [1, 2, 4, 8])
+def test_fuzz_slices(elem_size):
+    for i, s in enumerate(fuzz_slices(120, seed=elem_size)):
+        _roundtrip(s, elem_size, seed=i, misalign=(i % 4) * elem_size, dst_misalign=(i % 3) * elem_size)
+
+
+def test_odd_byte_alignment():
+    for i, s in enumerate(fuzz_slices(40, seed=99)):
+        _roundtrip(s, 1, seed=i, misalign=1 + (i % 15), dst_misalign=(i * 7) % 16)
+    _roundtrip(Slice(offset=3, sizes=[5000], strides=[1]), 1, seed=1, misalign=5, dst_misalign=9)
+    _roundtrip(Slice(offset=3, sizes=[40, 300], strides=[301, 1]), 2, seed=2, misalign=2, dst_misalign=6)
+
+
+def test_many_dims_peels_on_host():
+    # 10 dims that cannot merge (every stride leaves a gap): more than the kernel decodes at once
+    sizes = [2] * 10
+    strides, acc = [], 1
+    for _ in sizes:
+        strides.append(acc)
+        acc *= 3
+    s = Slice(offset=1, sizes=sizes, strides=list(reversed(strides)))
+    _roundtrip(s, 4, seed=5)
+    # and the same with the dims in scrambled (non-monotone stride) order
+    perm = [3, 0, 7, 1, 9, 2, 8, 4, 6, 5]
+    s = Slice(offset=0, sizes=[sizes[p] for p in perm], strides=[list(reversed(strides))[p] for p in perm])
+    _roundtrip(s, 2, seed=6)
+
+
+def test_config1_f32_every_other_row():
+    # fp32 [4,256,256], view {0,[4,128,256],[65536,512,1]}: pack, unpack back
+    rng = np.random.default_rng(1000)
+    x = rng.uniform(-1, 1, size=(4, 256, 256)).astype(np.float32)
+    s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
+    dev = torch.from_numpy(x).to(DEV)
+    packed = staging.pack(dev, s)
+    sync()
+    want = oracle.pack(x.reshape(-1), oslice(s))
+    assert np.array_equal(packed.cpu().numpy(), want)
+    assert np.array_equal(want.reshape(4, 128, 256), x[:, ::2, :])  # the view itself
+    back = torch.zeros_like(dev)
+    staging.unpack(back, s, packed)
+    sync()
+    ref = np.zeros_like(x)
+    ref[:, ::2, :] = x[:, ::2, :]
+    assert np.array_equal(back.cpu().numpy(), ref)
+
+
+def test_config3_column_blocks_full_size():
+    # bf16 [4096,14336]; 8 views {k*1792,[4096,1792],[14336,1]} -> 8 send buffers -> zeroed tensor
+    g = torch.Generator(device=DEV).manual_seed(3000)
+    w = (torch.randn(4096, 14336, generator=g, device=DEV) * 0.02).bfloat16()
+    views = [Slice(offset=k * 1792, sizes=[4096, 1792], strides=[14336, 1]) for k in range(8)]
+    bufs = staging.pack_many(w, views)
+    sync()
+    hw = bits(w).reshape(-1)
+    for k in (0, 3, 7):
+        want = oracle.pack(hw, oslice(views[k]), runs=True)
+        assert np.array_equal(bits(bufs[k]), want)
+    for k in range(8):  # every buffer equals the column block
+        assert torch.equal(bufs[k].view(4096, 1792), w[:, k * 1792:(k + 1) * 1792])
+    back = torch.zeros_like(w)
+    staging.unpack_many(back, views, bufs)
+    sync()
+    assert torch.equal(back.view(torch.int16), w.view(torch.int16))  # the 8 views tile the tensor
+    # single-view entry point gives the same bytes
+    one = staging.pack(w, views[5])
+    sync()
+    assert torch.equal(one.view(torch.int16), bufs[5].view(torch.int16))
+
+
+def test_contiguous_pack_is_memcmp():
+    g = torch.Generator(device=DEV).manual_seed(2001)
+    x = (torch.randn(25_165_824, generator=g, device=DEV) * 0.02).bfloat16()
+    s = Slice.new_row_major([x.numel()])
+    out = staging.pack(x, s)
+    sync()
+    assert torch.equal(out.view(torch.int16), x.view(torch.int16))
+    back = torch.empty_like(x)
+    staging.unpack(back, s, out)
+    sync()
+    assert torch.equal(back.view(torch.int16), x.view(torch.int16))
+
+
+def test_transposed_matrix():
+    g = torch.Generator().manual_seed(7)
+    x = torch.randint(-2**31, 2**31 - 1, (257, 515), dtype=torch.int32, generator=g)
+    dev = x.to(DEV)
+    s = Slice(offset=0, sizes=[515, 257], strides=[1, 515])  # iterate columns: packs x.T
+    out = staging.pack(dev, s)
+    sync()
+    assert np.array_equal(out.cpu().numpy(), x.numpy().T.reshape(-1))
+    assert np.array_equal(out.cpu().numpy(), oracle.pack(x.numpy().reshape(-1), oslice(s)))
+
+
+def test_pack_many_mixed_views_and_alignment():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randint(0, 2**15, (64, 96), dtype=torch.int16, generator=g)
+    dev = x.to(DEV)
+    views = [Slice(offset=0, sizes=[64, 32], strides=[96, 1]), Slice(offset=32, sizes=[64, 32], strides=[96, 1]),
+             Slice(offset=64, sizes=[64, 31], strides=[96, 1]), Slice(offset=95, sizes=[64], strides=[96]),
+             Slice(offset=0, sizes=[0], strides=[1])]
+    store = torch.zeros(64 * 96 + 64, dtype=torch.int16, device=DEV)
+    outs, pos = [], 0
+    for i, v in enumerate(views):
+        pos += i  # staggers the staging alignment
+        outs.append(store[pos: pos + len(v)])
+        pos += len(v)
+    staging.pack_many(dev, views, outs)
+    sync()
+    for v, o in zip(views, outs):
+        assert np.array_equal(o.cpu().numpy(), oracle.pack(x.numpy().reshape(-1), oslice(v)))
+    back = torch.zeros_like(dev)
+    staging.unpack_many(back, views, outs)
+    sync()
+    assert torch.equal(back, dev)
+
+
+def test_wide_index_path_over_2g_units():
+    # more than 2^31 one-byte units (odd addresses force unit = 1): exercises 64-bit decode
+    n = 2**31 + 4096 + 2
+    src = torch.empty(n + 2, dtype=torch.uint8, device=DEV)
+    src.view(torch.int16)[:] = torch.arange((n + 2) // 2, device=DEV, dtype=torch.int32).to(torch.int16)
+    dst = torch.zeros(n + 2, dtype=torch.uint8, device=DEV)
+    s = Slice(offset=0, sizes=[n], strides=[1])
+    import ctypes as C
+    from monarch_amd._lib import check, lib
+    check(lib().mhip_slice_pack(dst.data_ptr() + 1, src.data_ptr() + 1, C.byref(s.c), 1,
+                                torch.cuda.current_stream().cuda_stream))
+    sync()
+    assert dst[0].item() == 0 and dst[n + 1].item() == 0
+    assert torch.equal(dst[1: n + 1], src[1: n + 1])
+
+
+def test_tensor_buffer_round_trip():
+    # the RDMABuffer contract: 1-D contiguous uint8 only; TensorBuffer stages a strided view through it
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(10, 10, generator=g).to(DEV)
+    view = x[2:8, 1:9:2]
+    tb = staging.TensorBuffer(view)
+    buf = tb.stage()
+    remote = torch.zeros(buf.size, dtype=torch.uint8, device=DEV)
+    buf.read_into(remote)
+    y = torch.zeros(10, 10, device=DEV)
+    tb2 = staging.TensorBuffer(y[2:8, 1:9:2])
+    tb2.buffer.write_from(remote)
+    tb2.commit()
+    sync()
+    ref = torch.zeros(10, 10)
+    ref[2:8, 1:9:2] = x.cpu()[2:8, 1:9:2]
+    assert torch.equal(y.cpu(), ref)
+    with pytest.raises(ValueError, match="Tensor must be 1D"):
+        staging.RDMABuffer(x)
+    with pytest.raises(ValueError, match="Tensor must be uint8"):
+        staging.RDMABuffer(x.flatten())
+    with pytest.raises(ValueError, match="must be <="):
+        buf.read_into(torch.zeros(buf.size + 1, dtype=torch.uint8, device=DEV))

@@ -1,0 +1,327 @@
+"""GPU parity: mhip_reduce / mhip_reduce_scatter and the Reduce host semantics."""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from monarch_amd import DeviceMesh, Slice, _lib
+from monarch_amd import reduce as R
+from monarch_amd._lib import MhipError
+from oracle import AVG, SUM
+from util import bits, oslice, sync
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def vec(golden_dir):
+    with open(os.path.join(golden_dir, "ndslice_vectors.json")) as f:
+        return json.load(f)
+
+
+def _rand(dtype, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    if dtype in (torch.float32, torch.float64):
+        return (torch.rand(n, generator=g, dtype=dtype) * 2 - 1)
+    if dtype in (torch.bfloat16, torch.float16):
+        return (torch.randn(n, generator=g) * 0.02).to(dtype)
+    if dtype == torch.uint8:
+        return torch.randint(0, 256, (n,), dtype=dtype, generator=g)
+    info = torch.iinfo(dtype)
+    return torch.randint(info.min, info.max, (n,), dtype=dtype, generator=g)
+
+
+def _oracle_reduce(hosts, op, dtype):
+    if dtype == torch.float16:
+        # the oracle has no fp16 kernel: fp32 accumulate in rank order, one rounding (same rule as bf16)
+        acc = hosts[0].float()
+        for h in hosts[1:]:
+            acc = acc + h.float()
+        if op == AVG:
+            acc = acc / np.float32(len(hosts))
+        return bits(acc.to(torch.float16))
+    return oracle.reduce([bits(h) for h in hosts], op)
+
+
+def test_golden_vectors(vec):
+    for case in vec["reduce"]:
+        ins = [torch.tensor(x, dtype=torch.float32, device=DEV) for x in case["inputs"]]
+        if case["kind"] == "sum":
+            out = torch.empty_like(ins[0])
+            R.all_reduce(out, ins, R.ReduceOp.Sum)
+            sync()
+            assert out.cpu().tolist() == case["expected"], case["src"]
+        else:
+            for r, want in enumerate(case["expected_per_rank"]):
+                out = torch.full((len(want),), 1.0, device=DEV)
+                R.reduce_scatter_tensor(out, ins, r, R.ReduceOp.Sum)
+                sync()
+                assert out.cpu().tolist() == want, case["src"]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64])
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8, 9, 16, 17, 64])
+def test_reduce_float_bit_exact(dtype, n):
+    for numel in (1, 7, 8, 1000, 4099, (1 << 18) + 3):
+        hosts = [_rand(dtype, numel, 100 * n + r) for r in range(n)]
+        devs = [h.to(DEV) for h in hosts]
+        for op, code in ((R.ReduceOp.Sum, SUM), (R.ReduceOp.Avg, AVG)):
+            out = torch.empty_like(devs[0])
+            R.all_reduce(out, devs, op)
+            sync()
+            want = _oracle_reduce(hosts, code, dtype)
+            assert np.array_equal(bits(out), want), (dtype, n, numel, op)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int8, torch.int32, torch.int64])
+def test_reduce_integer_sum_wraps(dtype):
+    for n, numel in ((2, 5), (3, 4099), (8, 65536 + 1)):
+        hosts = [_rand(dtype, numel, 7 * n + r) for r in range(n)]
+        devs = [h.to(DEV) for h in hosts]
+        out = torch.empty_like(devs[0])
+        R.all_reduce(out, devs, R.ReduceOp.Sum)
+        sync()
+        hs = [h.view(torch.uint8) if dtype == torch.int8 else h for h in hosts]
+        want = oracle.reduce([bits(h) for h in hs], SUM)
+        got = bits(out.view(torch.uint8) if dtype == torch.int8 else out)
+        assert np.array_equal(got, want)
+    with pytest.raises(MhipError) as e:
+        R.all_reduce(out, devs, R.ReduceOp.Avg)
+    assert e.value.name == "UnsupportedOp"
+
+
+def test_reduce_in_place_and_misaligned():
+    n, numel = 8, 10007
+    hosts = [_rand(torch.bfloat16, numel + 3, r) for r in range(n)]
+    # element-aligned only: every pointer 2 bytes off a 16-byte boundary
+    devs = [h.to(DEV)[1: 1 + numel] for h in hosts]
+    want = oracle.reduce([bits(h)[1: 1 + numel] for h in hosts], AVG)
+    for alias in (0, 5):  # in place on the first member, and on another one
+        work = [d.clone() for d in devs]
+        keep = [torch.cat([torch.zeros(1, dtype=torch.bfloat16, device=DEV), w, torch.zeros(2, dtype=torch.bfloat16, device=DEV)])
+                for w in work]
+        views = [k[1: 1 + numel] for k in keep]
+        R.all_reduce(views[alias], views, R.ReduceOp.Avg)
+        sync()
+        assert np.array_equal(bits(views[alias]), want)
+        for r in range(n):
+            if r != alias:
+                assert torch.equal(views[r].view(torch.int16), devs[r].view(torch.int16))  # inputs untouched
+            assert keep[r][0].item() == 0 and keep[r][-1].item() == 0
+
+
+def test_reduce_nan_inf_bf16():
+    x = torch.tensor([float("nan"), float("inf"), -float("inf"), 1.0, 3.3895314e38, 0.0, -0.0, 1e-40],
+                     dtype=torch.float32).bfloat16()
+    y = torch.tensor([1.0, 1.0, float("inf"), float("nan"), 3.3895314e38, -0.0, -0.0, 1e-40],
+                     dtype=torch.float32).bfloat16()
+    out = torch.empty(8, dtype=torch.bfloat16, device=DEV)
+    for op, code in ((R.ReduceOp.Sum, SUM), (R.ReduceOp.Avg, AVG)):
+        R.all_reduce(out, [x.to(DEV), y.to(DEV)], op)
+        sync()
+        assert np.array_equal(bits(out), oracle.reduce([bits(x), bits(y)], code))
+
+
+def test_reduce_argument_errors():
+    x = torch.zeros(16, device=DEV)
+    out = torch.empty_like(x)
+    with pytest.raises(MhipError) as e:  # nccl.rs:474-476
+        R.all_reduce(out.to(torch.float8_e4m3fn), [x.to(torch.float8_e4m3fn)], R.ReduceOp.Sum)
+    assert e.value.name == "Float8Reduction"
+    with pytest.raises(MhipError) as e:
+        R.all_reduce(out, [x] * 65, R.ReduceOp.Sum)
+    assert e.value.name == "TooManyInputs"
+    with pytest.raises(MhipError) as e:
+        R.all_reduce(out, [x], R.ReduceOp.Max)
+    assert e.value.name == "UnsupportedOp"
+    with pytest.raises(MhipError) as e:
+        R.all_reduce(out, [x.double()], R.ReduceOp.Sum)
+    assert e.value.name == "TypeMismatch"
+    with pytest.raises(MhipError) as e:  # check order of nccl.rs:300-316: device before contiguity
+        R.all_reduce(out, [torch.zeros(16)], R.ReduceOp.Sum)
+    assert e.value.name == "InvalidDevice"
+    with pytest.raises(MhipError) as e:
+        R.all_reduce(out, [torch.zeros(16, 2, device=DEV)[:, 0]], R.ReduceOp.Sum)
+    assert e.value.name == "NoncontiguousTensor"
+    with pytest.raises(MhipError) as e:  # nccl.rs:683
+        R.reduce_scatter_tensor(torch.empty(5, device=DEV), [x, x], 0, R.ReduceOp.Sum)
+    assert e.value.name == "InputSizeMismatch"
+    import ctypes as C
+    from monarch_amd._lib import lib, ptr_array
+    rc = lib().mhip_reduce(out.data_ptr(), ptr_array([x.data_ptr(), 0]), 2, 16, _lib.DTYPE_F32, 0, None)
+    assert rc == _lib.ERR_UNDEFINED_TENSOR
+    rc = lib().mhip_reduce(out.data_ptr(), ptr_array([x.data_ptr()]), 1, 16, 2, 0, None)  # Short: no NCCL type
+    assert rc == _lib.ERR_INVALID_DATA_TYPE
+
+
+def test_config2_bf16_bucket_full_size():
+    n, numel = 8, 25_165_824
+    g = torch.Generator(device=DEV).manual_seed(2000)
+    devs = [(torch.randn(numel, generator=g, device=DEV) * 0.02).bfloat16() for _ in range(n)]
+    hosts = [bits(d) for d in devs]
+    want = oracle.reduce(hosts, AVG)
+    out = torch.empty_like(devs[0])
+    R.all_reduce(out, devs, R.ReduceOp.Avg)  # out of place
+    sync()
+    assert np.array_equal(bits(out), want)
+    # library cross-check: within 1 bf16 ulp of torch's fp32 path
+    ref = (torch.stack([d.float() for d in devs]).sum(0) / n).bfloat16()
+    diff = (out.view(torch.int16).int() - ref.view(torch.int16).int()).abs().max().item()
+    assert diff <= 1
+    first = devs[0].clone()
+    R.all_reduce(devs[0], devs, R.ReduceOp.Avg)  # in place on input 0
+    sync()
+    assert np.array_equal(bits(devs[0]), want)
+    # linearity on exact data: sum of 8 copies == 8 * x in bf16 (exact scaling by a power of two)
+    R.all_reduce(out, [first] * 8, R.ReduceOp.Sum)
+    sync()
+    assert torch.equal(out.view(torch.int16), (first.float() * 8).bfloat16().view(torch.int16))
+
+
+def test_config1_sum_of_8_packed_chunks():
+    from monarch_amd import staging
+    s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
+    chunks, hosts = [], []
+    for k in range(8):
+        rng = np.random.default_rng(1000 + k)
+        x = rng.uniform(-1, 1, size=(4, 256, 256)).astype(np.float32)
+        chunks.append(staging.pack(torch.from_numpy(x).to(DEV), s))
+        hosts.append(oracle.pack(x.reshape(-1), oslice(s)))
+    out = torch.empty_like(chunks[0])
+    R.all_reduce(out, chunks, R.ReduceOp.Sum)
+    sync()
+    assert np.array_equal(out.cpu().numpy(), oracle.reduce(hosts, SUM))
+    np.testing.assert_allclose(out.cpu().numpy(), np.sum(np.stack(hosts).astype(np.float64), 0), rtol=1e-6, atol=1e-6)
+
+
+def _c4(H, G, Rr, Cc, K, seed, dtype=torch.float32):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    x = (torch.rand(H, G, Rr, Cc, generator=g, device=DEV) * 2 - 1).to(dtype)
+    slab = Rr * Cc
+    flat = x.view(-1)
+    group = [flat[gi * slab:] for gi in range(G)]
+    in_view = Slice(offset=0, sizes=[H, Rr, Cc], strides=[G * slab, Cc, 1])
+    w = Cc // K
+    out_views = [Slice(offset=k * w, sizes=[H, Rr, w], strides=[Rr * Cc, Cc, 1]) for k in range(K)]
+    return x, group, in_view, out_views, w
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 8, 16, 64, 8), (2, 3, 5, 40, 5), (1, 2, 7, 9, 3), (2, 8, 4, 56, 7)])
+def test_reduce_scatter_mesh_dim_small(dtype, shape):
+    H, G, Rr, Cc, K = shape
+    x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=sum(shape), dtype=dtype)
+    for op, code in ((R.ReduceOp.Sum, SUM), (R.ReduceOp.Avg, AVG)):
+        outs = [torch.empty(H * Rr * w, dtype=dtype, device=DEV) for _ in range(K)]
+        R.reduce_scatter_views(outs, out_views, group, in_view, op)
+        sync()
+        hx = bits(x).reshape(-1)
+        slab = Rr * Cc
+        want = oracle.reduce_scatter([hx[g * slab:] for g in range(G)], oslice(in_view),
+                                     [oslice(v) for v in out_views], code)
+        for k in range(K):
+            assert np.array_equal(bits(outs[k]), want[k]), (shape, k, op)
+
+
+def test_config4_mesh_dim_reduce_scatter_full_size():
+    H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
+    x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=4000)
+    outs = [torch.empty(H * Rr * w, dtype=torch.float32, device=DEV) for _ in range(K)]
+    R.reduce_scatter_views(outs, out_views, group, in_view, R.ReduceOp.Sum)
+    sync()
+    # exact: fp32 adds in gpu order, which torch reproduces with explicit adds
+    acc = x[:, 0].clone()
+    for g in range(1, G):
+        acc = acc + x[:, g]
+    for k in range(K):
+        assert torch.equal(outs[k].view(H, Rr, w), acc[:, :, k * w:(k + 1) * w])
+    # oracle on two of the outputs (the div/mod walk is slow at full size)
+    hx = x.cpu().numpy().reshape(-1)
+    slab = Rr * Cc
+    for k in (0, 7):
+        want = oracle.reduce_scatter([hx[g * slab:] for g in range(G)], oslice(in_view), [oslice(out_views[k])], SUM)[0]
+        assert np.array_equal(outs[k].cpu().numpy(), want)
+    np.testing.assert_allclose(torch.cat([o.view(H, Rr, w) for o in outs], dim=2).cpu().numpy(),
+                               x.sum(1).cpu().numpy(), rtol=1e-6, atol=1e-6)
+
+
+def test_reduce_scatter_dim0_rule_all_ranks():
+    # ncclReduceScatter: rank r receives the reduced flat chunk r (nccl.rs:683,693-701)
+    n, c = 4, 1031
+    hosts = [_rand(torch.float32, n * c, 40 + r) for r in range(n)]
+    devs = [h.to(DEV) for h in hosts]
+    total = oracle.reduce([h.numpy() for h in hosts], SUM)
+    for r in range(n):
+        out = torch.empty(c, device=DEV)
+        R.reduce_scatter_tensor(out, devs, r, R.ReduceOp.Sum)
+        sync()
+        assert np.array_equal(out.cpu().numpy(), total[r * c:(r + 1) * c])
+
+
+def test_stream_reduce_placement_and_errors():
+    # test_controller.py:188-254 on a [2 hosts, 2 gpus] mesh: x[h,g] = 24h + 12g + arange(12)
+    mesh_slice = Slice(offset=0, sizes=[2, 2], strides=[2, 1])
+    xs = {(h, g): (24 * h + 12 * g + torch.arange(12, device=DEV).reshape(3, 4)).float()
+          for h, g in itertools.product(range(2), range(2))}
+    world = {2 * h + g: t for (h, g), t in xs.items()}
+    mesh = DeviceMesh(["host", "gpu"], mesh_slice, 0)
+    y = R.reduce(world, mesh, "gpu", "sum")
+    g = R.reduce(world, mesh, "gpu", "stack")
+    sync()
+    assert torch.equal(y, xs[(0, 0)] + xs[(0, 1)])
+    assert torch.equal(g, torch.stack([xs[(0, 0)], xs[(0, 1)]]))
+    with pytest.raises(TypeError, match="When scattering"):
+        R.reduce(world, mesh, "gpu", "sum", scatter=True)
+    w2 = {r: t.reshape(2, 6) for r, t in world.items()}
+    rs = R.reduce(w2, mesh, "gpu", "sum", scatter=True)
+    atoa = R.reduce(w2, mesh, "gpu", "stack", scatter=True)
+    rad = R.reduce(w2, mesh, (), "sum")
+    rade = R.reduce(w2, mesh, ("gpu", "host"), "sum")
+    sync()
+    total = sum(xs.values()).reshape(2, 6)
+    assert torch.equal(rs, (w2[0] + w2[1])[0]) and rs.shape == (6,)
+    assert torch.equal(atoa, torch.stack([w2[0][0], w2[1][0]]))
+    assert torch.equal(rad, total) and torch.equal(rade, total)
+    for kw in (dict(scatter=True), dict(reduction="stack"), dict(reduction="stack", scatter=True)):
+        with pytest.raises(ValueError, match="is not valid for multiple dimensions"):
+            R.reduce(w2, mesh, (), **{"reduction": "sum", **kw})
+    with pytest.raises(KeyError):
+        R.reduce(w2, mesh, "nope")
+    with pytest.raises(ValueError, match="reducing the same dimension twice"):
+        R.reduce(w2, mesh, ("gpu", "gpu"))
+    # test_reduce_out (test_controller.py:256-270): wrong out shape is refused
+    with pytest.raises(ValueError, match="Reduce expects the shape to be torch.Size"):
+        R.reduce(w2, mesh, "host", "sum", scatter=True, out=torch.empty(2, 4, device=DEV))
+    # placement (stream.rs:1437-1458): in place aliases the input; out= is returned; default is a fresh tensor
+    mine = w2[0].clone()
+    w3 = dict(w2)
+    w3[0] = mine
+    r1 = R.reduce(w3, mesh, "gpu", "sum", inplace=True)
+    assert r1.data_ptr() == mine.data_ptr()
+    o = torch.empty(2, 6, device=DEV)
+    r2 = R.reduce(w2, mesh, "gpu", "avg", out=o)
+    r3 = R.reduce(w2, mesh, "gpu", "sum")
+    sync()
+    assert r2.data_ptr() == o.data_ptr() and r3.data_ptr() not in (w2[0].data_ptr(), o.data_ptr())
+    assert torch.equal(r1, w2[0] + w2[1]) and torch.equal(r2, (w2[0] + w2[1]) / 2) and torch.equal(r3, r1)
+    with pytest.raises(ValueError, match="cannot be used with inplace"):
+        R.reduce(w2, mesh, "gpu", "sum", inplace=True, out=o)
+    with pytest.raises(ValueError, match="not valid for in-place"):
+        R.reduce(w2, mesh, "gpu", "sum", scatter=True, inplace=True)
+    # an input that errored upstream is replaced by zeros of the factory (stream.rs:976-989)
+    group = [None, w2[1]]
+    r4 = R.stream_reduce(group, 1, R.Factory.of(w2[1]), R.Reduction.from_str("sum"), False, False)
+    sync()
+    assert torch.equal(r4, w2[1])
+    # worker_reduce (comm.rs:1258-1431): ones(2,3) over a [2,2] mesh -> 2.0 over "x", 4.0 over "x","y"
+    ones = {r: torch.ones(2, 3, device=DEV) for r in range(4)}
+    m2 = DeviceMesh(["x", "y"], Slice(offset=0, sizes=[2, 2], strides=[2, 1]), 3)
+    a = R.reduce(ones, m2, "x", "sum")
+    b = R.reduce(ones, m2, ("x", "y"), "sum")
+    sync()
+    assert torch.all(a == 2.0) and torch.all(b == 4.0)

@@ -1,0 +1,54 @@
+"""Helpers shared by the GPU parity tests."""
+import random
+
+import numpy as np
+import torch
+
+from monarch_amd import Slice
+from oracle import OSlice
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    """Host numpy array with the tensor's raw element bits (bf16 -> uint16)."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype == torch.bfloat16:
+        return t.view(torch.uint16).numpy()
+    if t.dtype == torch.float16:
+        return t.view(torch.uint16).numpy()
+    return t.numpy()
+
+
+def oslice(s: Slice) -> OSlice:
+    return OSlice.unchecked(s.offset, s.sizes, s.strides)
+
+
+def span(s) -> int:
+    """Number of storage elements a slice needs."""
+    if any(z == 0 for z in s.sizes):
+        return s.offset + 1
+    return s.offset + sum((z - 1) * st for z, st in zip(s.sizes, s.strides)) + 1
+
+
+def fuzz_slices(n, seed, max_size=10, max_offset=10000):
+    """The generator of python/tests/_monarch/test_ndslice.py:143-167 (rejection sampling)."""
+    gen = random.Random(seed)
+    out = []
+    while len(out) < n:
+        ndim = gen.choices([1, 2, 3, 4], [1, 2, 3, 4])[0]
+        sizes = [gen.randrange(1, max_size) for _ in range(ndim)]
+        strides, run = [], 1
+        for j in range(ndim):
+            run *= gen.randrange(1 if j == 0 else 2, 4)
+            strides.append(run)
+        order = list(range(ndim))
+        gen.shuffle(order)
+        try:
+            out.append(Slice(offset=gen.randrange(max_offset), sizes=[sizes[o] for o in order],
+                             strides=[strides[o] for o in order]))
+        except ValueError:
+            continue
+    return out
+
+
+def sync():
+    torch.cuda.synchronize()
