@@ -33,6 +33,7 @@ class FlatBucket:
             _torch.require_contiguous(t)
             if t.dtype != self.dtype:
                 raise ValueError("all tensors of a bucket must share a dtype")
+        self.tensors = list(tensors)  # the pointer table below is only valid while these are alive
         self.sizes = [t.numel() for t in tensors]
         self.offsets = [0]
         for n in self.sizes:
@@ -65,9 +66,8 @@ class FlatBucket:
         ptrs = self.pointer_table(outs)
         check(lib().mhip_flat_unpack(ptrs.data_ptr(), flat.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
                                      self.total, flat.element_size(), _torch.stream_handle(stream)))
-        # keep the table alive until the launch that reads it has been enqueued and ordered
-        # behind later work on the same stream
-        self._last_unpack_table = ptrs
+        # the launch reads the table asynchronously: keep it (and the outputs) alive
+        self._last_unpack = (ptrs, list(outs))
 
 
 def quantize(flat_bf16: torch.Tensor, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None):
