@@ -78,52 +78,67 @@ __device__ __noinline__ void quantize_block_careful(uint8_t* __restrict__ q, flo
     for (uint32_t i = lane; i < count; i += 64) q[begin + i] = quant_one_careful(x[begin + i], inv);
 }
 
+// One wavefront quantises kQuantBlocks consecutive blocks per step: all of their loads
+// (2 per block and lane) are issued before the first max, to keep 4 KiB per wavefront in flight.
+constexpr int kQuantBlocks = 2;
+
 __global__ __launch_bounds__(kThreads) void fp8_quantize_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                 const uint16_t* __restrict__ x, uint64_t numel,
                                                                 uint64_t nblocks) {
     const int lane = threadIdx.x & 63;
     const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
     const uint64_t nwaves = (uint64_t)gridDim.x * (kThreads / 64);
-    for (uint64_t b = wave; b < nblocks; b += nwaves) {
-        const uint64_t begin = b * kBlock;
-        const uint64_t remain = numel - begin;
-        if (remain < kBlock) {  // wave-uniform
-            quantize_block_careful(q, scales, x, begin, (uint32_t)remain, b, lane);
-            continue;
-        }
-        const char* src = reinterpret_cast<const char*>(x + begin);
-        const uint4 lo = load16_unaligned(src + lane * 16);         // elements [8*lane, 8*lane+8)
-        const uint4 hi = load16_unaligned(src + 1024 + lane * 16);  // elements [512+8*lane, ...)
-        // magnitudes as packed 16-bit integers: bf16 order == integer order for |x|
-        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-        uint32_t m = 0;
+    for (uint64_t b0 = wave * kQuantBlocks; b0 < nblocks; b0 += nwaves * kQuantBlocks) {
+        uint4 lo[kQuantBlocks], hi[kQuantBlocks];
+        bool full[kQuantBlocks];
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const uint32_t a = w[k] & 0x7fff7fffu;
-            const uint32_t a0 = a & 0xffffu, a1 = a >> 16;
-            m = a0 > m ? a0 : m;
-            m = a1 > m ? a1 : m;
+        for (int j = 0; j < kQuantBlocks; ++j) {
+            const uint64_t begin = (b0 + j) * kBlock;
+            full[j] = b0 + j < nblocks && numel - begin >= kBlock;  // wave-uniform
+            if (full[j]) {
+                const char* src = reinterpret_cast<const char*>(x + begin);
+                lo[j] = load16_unaligned(src + lane * 16);         // elements [8*lane, 8*lane+8)
+                hi[j] = load16_unaligned(src + 1024 + lane * 16);  // elements [512+8*lane, ...)
+            }
         }
-        m = wave_max_u32(m);
-        if (m >= 0x7f80u) {  // Inf or NaN somewhere in the block (wave-uniform, rare)
-            quantize_block_careful(q, scales, x, begin, kBlock, b, lane);
-            continue;
+#pragma unroll
+        for (int j = 0; j < kQuantBlocks; ++j) {
+            const uint64_t b = b0 + j;
+            if (b >= nblocks) break;
+            const uint64_t begin = b * kBlock;
+            if (!full[j]) {  // short final block
+                quantize_block_careful(q, scales, x, begin, (uint32_t)(numel - begin), b, lane);
+                continue;
+            }
+            // magnitudes as 16-bit integers: bf16 order == integer order for |x|
+            const uint32_t w[8] = {lo[j].x, lo[j].y, lo[j].z, lo[j].w, hi[j].x, hi[j].y, hi[j].z, hi[j].w};
+            uint32_t m = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t a = w[k] & 0x7fff7fffu;
+                const uint32_t a0 = a & 0xffffu, a1 = a >> 16;
+                m = a0 > m ? a0 : m;
+                m = a1 > m ? a1 : m;
+            }
+            m = wave_max_u32(m);
+            if (m >= 0x7f80u) {  // Inf or NaN somewhere in the block (wave-uniform, rare)
+                quantize_block_careful(q, scales, x, begin, kBlock, b, lane);
+                continue;
+            }
+            float scale, inv;
+            block_factors(m, &scale, &inv);
+            if (lane == 0) scales[b] = scale;
+            // |x * inv| <= 448 * (1 + 2^-22) for every finite x of the block, which rounds to
+            // at most 448, so no clamp is needed on this path.
+            int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+            c0 = quant_pair<false>(w[0], inv, c0); c0 = quant_pair<true>(w[1], inv, c0);
+            c1 = quant_pair<false>(w[2], inv, c1); c1 = quant_pair<true>(w[3], inv, c1);
+            c2 = quant_pair<false>(w[4], inv, c2); c2 = quant_pair<true>(w[5], inv, c2);
+            c3 = quant_pair<false>(w[6], inv, c3); c3 = quant_pair<true>(w[7], inv, c3);
+            uint8_t* dst = q + begin;
+            store8_unaligned(dst + lane * 8, (uint32_t)c0, (uint32_t)c1);
+            store8_unaligned(dst + 512 + lane * 8, (uint32_t)c2, (uint32_t)c3);
         }
-        float scale, inv;
-        block_factors(m, &scale, &inv);
-        if (lane == 0) scales[b] = scale;
-        // |x * inv| <= 448 * (1 + 2^-22) for every finite x of the block, which rounds to
-        // at most 448, so no clamp is needed on this path.
-        int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
-        c0 = quant_pair<false>(w[0], inv, c0); c0 = quant_pair<true>(w[1], inv, c0);
-        c1 = quant_pair<false>(w[2], inv, c1); c1 = quant_pair<true>(w[3], inv, c1);
-        c2 = quant_pair<false>(w[4], inv, c2); c2 = quant_pair<true>(w[5], inv, c2);
-        c3 = quant_pair<false>(w[6], inv, c3); c3 = quant_pair<true>(w[7], inv, c3);
-        const uint2 out_lo = make_uint2((uint32_t)c0, (uint32_t)c1);
-        const uint2 out_hi = make_uint2((uint32_t)c2, (uint32_t)c3);
-        uint8_t* dst = q + begin;
-        __builtin_memcpy(dst + lane * 8, &out_lo, 8);
-        __builtin_memcpy(dst + 512 + lane * 8, &out_hi, 8);
     }
 }
 
@@ -146,7 +161,7 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float*
             const uint64_t i = (b0 + j) * kBlock + threadIdx.x * 4;
             full[j] = i + 4 <= numel;
             if (full[j]) {
-                __builtin_memcpy(&codes[j], q + i, 4);
+                codes[j] = load4_unaligned(q + i);
                 a[j] = load16_unaligned(acc + i);
                 s[j] = scales[b0 + j];
             }
@@ -187,8 +202,9 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
     if (!q || !scales || !x_bf16) return MHIP_ERR_UNDEFINED_TENSOR;
     if (((uintptr_t)x_bf16 & 1u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
     const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
-    const uint64_t wgs = (nblocks + 3) / 4;
-    const uint64_t cap = 256ull * 32ull;
+    const uint64_t per_wg = (kThreads / 64) * kQuantBlocks;
+    const uint64_t wgs = (nblocks + per_wg - 1) / per_wg;
+    const uint64_t cap = 0x7fffffffull;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads), 0, hs, q, scales,
@@ -204,7 +220,7 @@ int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scale
     if (((uintptr_t)acc & 3u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
     const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
     const uint64_t ntiles = (nblocks + kDeqSteps - 1) / kDeqSteps;
-    const uint64_t cap = 256ull * 64ull;
+    const uint64_t cap = 0x7fffffffull;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kThreads), 0,

@@ -11,7 +11,7 @@
 namespace mhip {
 
 constexpr int kMaxViews = 16;
-constexpr int kUnroll = 4;  // chunks per thread, issued back to back for memory-level parallelism
+constexpr int kUnroll = 8;  // chunks per thread: 8 loads issued back to back, then 8 stores (32 KiB per workgroup)
 
 struct PackArgs {
     char* base;                  // strided tensor
@@ -64,14 +64,14 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
             if constexpr (PACK)
                 data[i] = load16_unaligned(strided + loc[i] * U);
             else
-                data[i] = *reinterpret_cast<const uint4*>(packed + first[i] * U);
+                data[i] = load16_aligned(packed + first[i] * U);
         }
     }
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
         if (vec[i]) {
             if constexpr (PACK)
-                *reinterpret_cast<uint4*>(packed + first[i] * U) = data[i];
+                store16_aligned(packed + first[i] * U, data[i]);
             else
                 store16_unaligned(strided + loc[i] * U, data[i]);
         }
@@ -149,9 +149,9 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
                 char* t = a.tensors[ti] + (first - begin) * U;
                 char* f = a.flat + first * U;
                 if constexpr (PACK)
-                    *reinterpret_cast<uint4*>(f) = load16_unaligned(t);
+                    store16_aligned(f, load16_unaligned(t));
                 else
-                    store16_unaligned(t, *reinterpret_cast<const uint4*>(f));
+                    store16_unaligned(t, load16_aligned(f));
                 done = true;
             }
         }
