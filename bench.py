@@ -28,7 +28,9 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    "c2": 452_348_918,  # profiles/reduce_kernel_bf16_c2.md: 0.9986 x the algorithmic bytes
+}
 
 
 def _load():

@@ -1,0 +1,95 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/monarch_hip.h declares."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+from monarch_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "monarch_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(mhip_[a-z0-9_]+)\s*\(", text))
+
+
+def test_header_binding_and_library_agree():
+    decl = declared_symbols()
+    assert decl == set(_lib.SIGNATURES), decl ^ set(_lib.SIGNATURES)
+    lib = _lib.lib()  # binds every symbol or raises
+    for name in decl:
+        assert hasattr(lib, name)
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True).stdout
+    exported = set(re.findall(r"\bT (mhip_[a-z0-9_]+)", out))
+    assert decl <= exported, decl - exported
+
+
+def test_header_compiles_as_plain_c():
+    src = '#include "monarch_hip.h"\nint main(void) { mhip_slice_t s; (void)s; return MHIP_SUCCESS; }\n'
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-x", "c", "-",
+                        "-fsyntax-only"], input=src, text=True, capture_output=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_status_text_and_host_only_calls():
+    lib = _lib.lib()
+    assert lib.mhip_version() >= 100
+    assert b"stride" in lib.mhip_error_string(_lib.ERR_STRIDE_TOO_SMALL)
+    assert b"float8" in lib.mhip_error_string(_lib.ERR_FLOAT8_REDUCTION)
+    assert lib.mhip_error_string(0) == b"success"
+    assert lib.mhip_dtype_size(_lib.DTYPE_BF16) == 2 and lib.mhip_dtype_size(_lib.DTYPE_F64) == 8
+    assert lib.mhip_dtype_size(2) == 0
+    # argument checks that precede any launch run without a GPU (torch-sys-cuda/src/nccl.rs:300-316,474-476)
+    one = (C.c_void_p * 1)(16)
+    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F8E4M3FN, 0, None) == _lib.ERR_FLOAT8_REDUCTION
+    assert lib.mhip_reduce(16, one, 1, 4, 2, 0, None) == _lib.ERR_INVALID_DATA_TYPE
+    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F32, 2, None) == _lib.ERR_UNSUPPORTED_OP
+    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_I32, 4, None) == _lib.ERR_UNSUPPORTED_OP
+    assert lib.mhip_reduce(16, one, 0, 4, _lib.DTYPE_F32, 0, None) == _lib.ERR_INVALID_ARGUMENT
+    many = (C.c_void_p * 65)(*([16] * 65))
+    assert lib.mhip_reduce(16, many, 65, 4, _lib.DTYPE_F32, 0, None) == _lib.ERR_TOO_MANY_INPUTS
+    assert lib.mhip_reduce(None, one, 1, 4, _lib.DTYPE_F32, 0, None) == _lib.ERR_UNDEFINED_TENSOR
+    assert lib.mhip_reduce(16, one, 1, 0, _lib.DTYPE_F32, 0, None) == 0  # nothing to do
+    assert lib.mhip_fp8_quantize(16, 16, 16, 10, 512, None) == _lib.ERR_UNSUPPORTED_BLOCK
+    from monarch_amd import Slice
+    bad = Slice(offset=0, sizes=[2, 2], strides=[2, 2], _validate=False)
+    assert lib.mhip_slice_pack(16, 16, C.byref(bad.c), 4, None) == _lib.ERR_NONUNIQUE_STRIDES
+    empty = Slice(offset=0, sizes=[0], strides=[1])
+    assert lib.mhip_slice_pack(None, None, C.byref(empty.c), 4, None) == 0
+
+
+def test_fastdiv_exhaustive_on_host(tmp_path):
+    src = r'''
+#include "fastdiv.h"
+#include <cstdio>
+#include <cstdint>
+int main() {
+  const uint32_t ds[] = {1,2,3,5,7,8,9,10,224,255,256,257,1000,1792,4096,14336,65535,65536,65537,1000003,
+                         0x3fffffffu,0x40000000u,0x40000001u,0x7ffffffdu,0x7ffffffeu};
+  uint64_t bad = 0;
+  for (uint32_t d : ds) {
+    mhip::FastDiv32 f(d);
+    for (uint64_t n = 0; n < 0x7fffffffull; n += (n < 70000 ? 1 : 9973)) {
+      uint32_t q, r; f.divmod((uint32_t)n, q, r);
+      if (q != n / d || r != n % d) ++bad;
+    }
+    for (uint64_t n = 0x7fffffffull - 70000; n < 0x7fffffffull; ++n) {
+      if (f.div((uint32_t)n) != n / d) ++bad;
+    }
+    for (uint64_t k = 1; k * d < 0x7fffffffull && k < 200000; ++k) {  // multiples and their neighbours
+      uint64_t n = k * d;
+      if (f.div((uint32_t)n) != k || f.div((uint32_t)(n - 1)) != (n - 1) / d) ++bad;
+    }
+  }
+  std::printf("%llu\n", (unsigned long long)bad);
+  return bad != 0;
+}
+'''
+    cpp = tmp_path / "t.cpp"
+    cpp.write_text(src)
+    exe = tmp_path / "t"
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-I", os.path.join(ROOT, "monarch_amd", "csrc"), str(cpp), "-o", str(exe)])
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout
