@@ -1,0 +1,151 @@
+//! Rust FFI bindings for `libmonarch_hip.so` (C ABI: `include/monarch_hip.h`).
+//!
+//! The sibling of the reference's `cuda-sys` / `nccl-sys` crates for the mesh
+//! data-movement / reduce path on MI355X: `ndslice::Slice`-described pack/unpack into
+//! `RdmaBuffer` staging memory, the local combine of `Communicator::all_reduce` /
+//! `reduce_scatter_tensor`, and the block-scaled fp8 codec.  Every function returns a
+//! status (`0` = success, `1..9999` = `hipError_t`, `>= 10000` = library classes, see
+//! `status` below); device functions enqueue on the given `hipStream_t` and never block.
+//!
+//! This crate is written against the header by hand (no bindgen) and has not been
+//! compiled in the build environment of this repository, which ships no Rust toolchain;
+//! `tests/test_abi.py` checks that the function names here and in the header agree.
+#![allow(non_camel_case_types)]
+
+use std::os::raw::{c_char, c_int, c_void};
+
+/// `hipStream_t`; replaces `cudaStream_t` of `nccl-sys` on this path.
+pub type mhip_stream_t = *mut c_void;
+/// `hipEvent_t`.
+pub type mhip_event_t = *mut c_void;
+
+/// `ndslice::Slice` as the C ABI sees it: `sizes`/`strides` point at `ndim` `usize`s
+/// (`Slice::sizes().as_ptr()` / `Slice::strides().as_ptr()` on a 64-bit target).
+#[repr(C)]
+#[derive(Debug, Clone, Copy)]
+pub struct mhip_slice_t {
+    pub offset: u64,
+    pub ndim: u32,
+    pub sizes: *const u64,
+    pub strides: *const u64,
+}
+
+pub mod status {
+    pub const SUCCESS: i32 = 0;
+    pub const INVALID_DIMS: i32 = 10001;
+    pub const NONRECTANGULAR_SHAPE: i32 = 10002;
+    pub const NONUNIQUE_STRIDES: i32 = 10003;
+    pub const STRIDE_TOO_SMALL: i32 = 10004;
+    pub const INDEX_OUT_OF_RANGE: i32 = 10005;
+    pub const VALUE_NOT_IN_SLICE: i32 = 10006;
+    pub const INCOMPATIBLE_VIEW: i32 = 10007;
+    pub const NONCONTIGUOUS: i32 = 10008;
+    pub const EMPTY_RANGE: i32 = 10009;
+    pub const DIMENSION_OUT_OF_RANGE: i32 = 10010;
+    pub const INVALID_DATA_TYPE: i32 = 10101;
+    pub const NONCONTIGUOUS_TENSOR: i32 = 10102;
+    pub const INVALID_DEVICE: i32 = 10103;
+    pub const FLOAT8_REDUCTION: i32 = 10104;
+    pub const TYPE_MISMATCH: i32 = 10105;
+    pub const OUTPUT_SIZE_MISMATCH: i32 = 10106;
+    pub const INPUT_SIZE_MISMATCH: i32 = 10107;
+    pub const UNDEFINED_TENSOR: i32 = 10108;
+    pub const INVALID_ARGUMENT: i32 = 10201;
+    pub const UNSUPPORTED_OP: i32 = 10202;
+    pub const TOO_MANY_INPUTS: i32 = 10203;
+    pub const UNSUPPORTED_BLOCK: i32 = 10204;
+}
+
+/// `c10::ScalarType` numbering, as carried by `monarch_messages::worker::Factory::dtype`.
+pub mod dtype {
+    pub const U8: i32 = 0;
+    pub const I8: i32 = 1;
+    pub const I32: i32 = 3;
+    pub const I64: i32 = 4;
+    pub const F16: i32 = 5;
+    pub const F32: i32 = 6;
+    pub const F64: i32 = 7;
+    pub const BF16: i32 = 15;
+    pub const F8E5M2: i32 = 23;
+    pub const F8E4M3FN: i32 = 24;
+    pub const F8E5M2FNUZ: i32 = 25;
+    pub const F8E4M3FNUZ: i32 = 26;
+}
+
+/// `ncclRedOp_t` numbering (`torch_sys_cuda::nccl::ReduceOp as i32`).
+pub mod op {
+    pub const SUM: i32 = 0;
+    pub const PROD: i32 = 1;
+    pub const MAX: i32 = 2;
+    pub const MIN: i32 = 3;
+    pub const AVG: i32 = 4;
+}
+
+extern "C" {
+    pub fn mhip_error_string(status: c_int) -> *const c_char;
+    pub fn mhip_version() -> c_int;
+    pub fn mhip_dtype_size(dtype: c_int) -> u32;
+    pub fn mhip_slice_validate(offset: usize, sizes: *mut u64, nsizes: u32, strides: *mut u64, nstrides: u32) -> c_int;
+    pub fn mhip_slice_len(s: *const mhip_slice_t, len: *mut u64) -> c_int;
+    pub fn mhip_slice_is_contiguous(s: *const mhip_slice_t, result: *mut c_int) -> c_int;
+    pub fn mhip_slice_get(s: *const mhip_slice_t, index: usize, loc: *mut u64) -> c_int;
+    pub fn mhip_slice_location(s: *const mhip_slice_t, coord: *mut u64, ncoord: u32, loc: *mut u64) -> c_int;
+    pub fn mhip_slice_coordinates(s: *const mhip_slice_t, value: usize, coords: *mut u64) -> c_int;
+    pub fn mhip_slice_index(s: *const mhip_slice_t, value: usize, index: *mut u64) -> c_int;
+    pub fn mhip_slice_iter(s: *const mhip_slice_t, start: usize, count: usize, locs: *mut c_void, written: *mut u64) -> c_int;
+    pub fn mhip_slice_select(s: *const mhip_slice_t, dim: u32, begin: usize, end: usize, step: usize, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_at(s: *const mhip_slice_t, dim: u32, index: usize, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_subview(s: *const mhip_slice_t, starts: *mut u64, nstarts: u32, lens: *mut u64, nlens: u32, out_offset: *mut u64) -> c_int;
+    pub fn mhip_slice_view(s: *const mhip_slice_t, new_sizes: *mut u64, nnew: u32, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_enforce_embedding(s: *const mhip_slice_t, other: *const mhip_slice_t) -> c_int;
+    pub fn mhip_slice_bounds(s: *const mhip_slice_t, min_loc: *mut u64, max_loc: *mut u64) -> c_int;
+    pub fn mhip_mesh_dim_members(ranks: *const mhip_slice_t, rank: usize, dim: u32, members: *mut u64, dim_rank: *mut u64) -> c_int;
+    pub fn mhip_mesh_ranks_for_dims(ranks: *const mhip_slice_t, rank: usize, dims: *const u32, ndims: u32, out: *mut u64, cap: usize, count: *mut u64) -> c_int;
+    pub fn mhip_slice_pack(dst: *mut c_void, src_base: *mut c_void, s: *const mhip_slice_t, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_slice_unpack(dst_base: *mut c_void, src: *mut c_void, s: *const mhip_slice_t, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_slice_pack_many(dsts: *const *mut c_void, src_base: *mut c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_slice_unpack_many(dst_base: *mut c_void, srcs: *const *mut c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_flat_pack(flat: *mut c_void, d_tensors: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: usize, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_flat_unpack(d_tensors: *mut c_void, flat: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: usize, elem_size: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_reduce(out: *mut c_void, input: *const *mut c_void, n: u32, numel: usize, dtype: c_int, op: c_int, stream: *mut c_void) -> c_int;
+    pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *mut c_void, in_view: *const mhip_slice_t, in_numel: usize, n_in: u32, dtype: c_int, op: c_int, stream: *mut c_void) -> c_int;
+    pub fn mhip_fp8_quantize(q: *mut c_void, scales: *mut c_void, x_bf16: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate(acc: *mut c_void, q: *mut c_void, scales: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_device_count(count: *mut c_int) -> c_int;
+    pub fn mhip_set_device(device: c_int) -> c_int;
+    pub fn mhip_device_synchronize() -> c_int;
+    pub fn mhip_stream_create(stream: *const *mut c_void) -> c_int;
+    pub fn mhip_stream_destroy(stream: *mut c_void) -> c_int;
+    pub fn mhip_stream_synchronize(stream: *mut c_void) -> c_int;
+    pub fn mhip_event_create(event: *const *mut c_void) -> c_int;
+    pub fn mhip_event_destroy(event: *mut c_void) -> c_int;
+    pub fn mhip_event_record(event: *mut c_void, stream: *mut c_void) -> c_int;
+    pub fn mhip_event_synchronize(event: *mut c_void) -> c_int;
+    pub fn mhip_event_elapsed_ms(ms: *mut f32, start: *mut c_void, stop: *mut c_void) -> c_int;
+    pub fn mhip_stream_wait_event(stream: *mut c_void, event: *mut c_void) -> c_int;
+    pub fn mhip_malloc(ptr: *const *mut c_void, bytes: usize) -> c_int;
+    pub fn mhip_free(ptr: *mut c_void) -> c_int;
+    pub fn mhip_memcpy_htod(dst: *mut c_void, src: *mut c_void, bytes: usize, stream: *mut c_void) -> c_int;
+    pub fn mhip_memcpy_dtoh(dst: *mut c_void, src: *mut c_void, bytes: usize, stream: *mut c_void) -> c_int;
+    pub fn mhip_memset(dst: *mut c_void, value: c_int, bytes: usize, stream: *mut c_void) -> c_int;
+}
+
+#[cfg(test)]
+mod tests {
+    use super::*;
+
+    #[test]
+    fn sanity() {
+        // SAFETY: testing bindings; host-only calls, no GPU needed
+        unsafe {
+            assert!(mhip_version() >= 100);
+            let sizes = [2u64, 3];
+            let strides = [3u64, 1];
+            assert_eq!(mhip_slice_validate(0, sizes.as_ptr() as *mut u64, 2, strides.as_ptr() as *mut u64, 2), status::SUCCESS);
+            let s = mhip_slice_t { offset: 0, ndim: 2, sizes: sizes.as_ptr(), strides: strides.as_ptr() };
+            let mut loc = 0u64;
+            assert_eq!(mhip_slice_get(&s, 4, &mut loc), status::SUCCESS);
+            assert_eq!(loc, 4);
+        }
+    }
+}

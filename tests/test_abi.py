@@ -93,3 +93,13 @@ int main() {
     subprocess.check_call(["g++", "-O2", "-std=c++17", "-I", os.path.join(ROOT, "monarch_amd", "csrc"), str(cpp), "-o", str(exe)])
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0 and r.stdout.strip() == "0", r.stdout
+
+
+def test_rust_extern_block_names_match_header():
+    text = open(os.path.join(ROOT, "hip-sys", "src", "lib.rs")).read()
+    rust = set(re.findall(r"pub fn (mhip_[a-z0-9_]+)\(", text))
+    assert rust == declared_symbols(), rust ^ declared_symbols()
+    # status codes in the Rust module equal the header's
+    header = open(os.path.join(ROOT, "include", "monarch_hip.h")).read()
+    for name, value in re.findall(r"MHIP_ERR_([A-Z0-9_]+) = (\d+)", header):
+        assert re.search(rf"pub const {name}: i32 = {value};", text), name
