@@ -194,6 +194,40 @@ def wl_c3(torch, unpack=False, sets=3):
     return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 
 
+def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
+    from monarch_amd import Slice, staging
+    n = int(os.environ.get("MONARCH_BENCH_TRANSPOSE_N", "8192"))
+    dt = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
+    g = torch.Generator(device="cuda:0").manual_seed(6000)
+    s = Slice(offset=0, sizes=[n, n], strides=[1, n])  # iterate columns first: packs x.T
+    bufs = [(torch.randn(n, n, generator=g, device="cuda:0").to(dt), torch.empty(n * n, dtype=dt, device="cuda:0"))
+            for _ in range(sets)]
+    es = bufs[0][0].element_size()
+    nbytes = 2 * n * n * es
+    for x, st in bufs:
+        staging.pack(x, s, out=st)
+    if unpack:
+        calls = [prepared("mhip_slice_unpack", x.data_ptr(), st.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+    else:
+        calls = [prepared("mhip_slice_pack", st.data_ptr(), x.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import oracle
+        m = 2048
+        h = bufs[0][0][:m, :m].contiguous().cpu().view(torch.uint16 if es == 2 else torch.int32).numpy().reshape(-1)
+        t0 = time.perf_counter()
+        oracle.pack(h, oracle.OSlice(0, [m, m], [1, m]))
+        dt_ = (time.perf_counter() - t0) * (n * n / (m * m))
+        return {"value": nbytes / dt_ / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"{m}x{m} corner through the per-element Slice::get walk, scaled to {n}x{n}"}
+
+    name = f"transpose_{dtype_name}_{n}x{n}_" + ("unpack" if unpack else "pack")
+    return name, nbytes, launch, cpu, "slice_transpose_kernel", "u8"
+
+
 def wl_c4(torch, sets=2):
     from monarch_amd import Slice, _lib
     from monarch_amd._lib import ptr_array
@@ -304,6 +338,9 @@ WORKLOADS = {
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
     "c4": wl_c4,
+    "tr_f32_pack": lambda t: wl_transpose(t, "f32", False),
+    "tr_f32_unpack": lambda t: wl_transpose(t, "f32", True),
+    "tr_bf16_pack": lambda t: wl_transpose(t, "bf16", False),
     "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
     "c5_quantize": lambda t: wl_c5(t, "quantize"),
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),

@@ -7,6 +7,7 @@
 // and tail).  Consecutive lanes take consecutive chunks, so each wavefront instruction
 // touches 1 KiB of contiguous staging memory.
 #include "mhip_device.h"
+#include "pack_internal.h"
 
 namespace mhip {
 
@@ -57,7 +58,28 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
             vec[i] = col + VU <= a.dims.run;
         }
     }
+    bool all_vec = true;
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) all_vec = all_vec && vec[i];
     uint4 data[kUnroll];
+    if (all_vec) {
+        // the common case, free of per-chunk predicates: 8 loads in flight, then 8 stores
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            if constexpr (PACK)
+                data[i] = load16_unaligned(strided + loc[i] * U);
+            else
+                data[i] = load16_aligned(packed + first[i] * U);
+        }
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            if constexpr (PACK)
+                store16_aligned(packed + first[i] * U, data[i]);
+            else
+                store16_unaligned(strided + loc[i] * U, data[i]);
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
         if (vec[i]) {
@@ -135,35 +157,56 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     const uint32_t t_lo = s_range[0], t_hi = s_range[1] + 1;
     const uint32_t upe = a.units_per_elem;
 
+    // phase 1: resolve every chunk of this lane to (tensor address, flat address)
+    char* tptr[kUnroll];
+    char* fptr[kUnroll];
+    bool vec[kUnroll];
+    bool all_vec = true;
+#pragma unroll
+    for (int i = 0; i < kUnroll; ++i) {
+        const uint64_t c = block_c0 + (uint64_t)i * kThreads + threadIdx.x;
+        const uint64_t tb = c * VU;
+        const uint64_t first = tb - a.shift;
+        vec[i] = false;
+        if (c < a.nchunks && tb >= a.shift && first + VU <= a.total) {
+            const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, first);
+            const uint64_t begin = a.offsets[ti] * upe, end = a.offsets[ti + 1] * upe;
+            if (first + VU <= end) {
+                tptr[i] = a.tensors[ti] + (first - begin) * U;
+                fptr[i] = a.flat + first * U;
+                vec[i] = true;
+            }
+        }
+        all_vec = all_vec && vec[i];
+    }
+    // phase 2: move them; without predicates when every chunk is a plain 16-byte move
+    uint4 data[kUnroll];
+    if (all_vec) {
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) data[i] = PACK ? load16_unaligned(tptr[i]) : load16_aligned(fptr[i]);
+#pragma unroll
+        for (int i = 0; i < kUnroll; ++i) {
+            if constexpr (PACK) store16_aligned(fptr[i], data[i]); else store16_unaligned(tptr[i], data[i]);
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
         const uint64_t c = block_c0 + (uint64_t)i * kThreads + threadIdx.x;
         if (c >= a.nchunks) continue;
-        const uint64_t tb = c * VU;
-        const uint64_t first = tb - a.shift;
-        bool done = false;
-        if (tb >= a.shift && first + VU <= a.total) {
-            const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, first);
-            const uint64_t begin = a.offsets[ti] * upe, end = a.offsets[ti + 1] * upe;
-            if (first + VU <= end) {
-                char* t = a.tensors[ti] + (first - begin) * U;
-                char* f = a.flat + first * U;
-                if constexpr (PACK)
-                    store16_aligned(f, load16_unaligned(t));
-                else
-                    store16_unaligned(t, load16_aligned(f));
-                done = true;
-            }
+        if (vec[i]) {
+            if constexpr (PACK) store16_aligned(fptr[i], load16_unaligned(tptr[i]));
+            else store16_unaligned(tptr[i], load16_aligned(fptr[i]));
+            continue;
         }
         if constexpr (VU > 1) {
-            if (!done) {
-                for (int j = 0; j < VU; ++j) {
-                    const uint64_t unit = tb + j - a.shift;
-                    if (tb + j >= a.shift && unit < a.total) {
-                        const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, unit);
-                        char* t = a.tensors[ti] + (unit - a.offsets[ti] * upe) * U;
-                        move_unit<U, PACK>(t, a.flat + unit * U);
-                    }
+            const uint64_t tb = c * VU;
+            for (int j = 0; j < VU; ++j) {
+                const uint64_t unit = tb + j - a.shift;
+                if (tb + j >= a.shift && unit < a.total) {
+                    const uint32_t ti = find_tensor(a.offsets, upe, t_lo, t_hi, unit);
+                    char* t = a.tensors[ti] + (unit - a.offsets[ti] * upe) * U;
+                    move_unit<U, PACK>(t, a.flat + unit * U);
                 }
             }
         }
@@ -213,6 +256,14 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         if (!canonicalize(views[k], elem_size, mask0, 16, &first, &unit)) {  // empty view: nothing to move
             ++k;
             continue;
+        }
+        {
+            int trc = MHIP_SUCCESS;
+            if (try_transpose_copy<PACK>(base, packed[k], first, unit, stream, &trc)) {
+                if (trc) return trc;
+                ++k;
+                continue;
+            }
         }
         PackArgs a{};
         bool fits32 = false;

@@ -1,0 +1,204 @@
+// LDS-tiled transposing pack / unpack for Slices whose innermost iteration dimension is
+// NOT the memory-contiguous one (column-major views, permuted dims).
+//
+// Let c be the (unique) dimension with unit stride, and let q enumerate, row-major, all
+// dimensions that come after c in iteration order (Q = product of their sizes).  In the
+// packed image, q is the fast index; in memory, c is.  A workgroup moves a TILE x TILE
+// tile: it reads rows that are contiguous along c, parks them in LDS, and writes rows
+// that are contiguous along q, so that both HBM sides see coalesced wavefront accesses
+// (the direct gather would fetch a whole 64-byte sector per element on one side).
+// The LDS tile is padded by one element per row: the transposed read then walks
+// consecutive banks instead of hitting one bank 64 times.
+#include "mhip_device.h"
+#include "pack_internal.h"
+
+namespace mhip {
+
+struct TransArgs {
+    char* base;
+    char* packed;
+    uint64_t offset;   // units (elements), start of the view in memory
+    uint64_t ntiles;   // nbatch * qtiles * ctiles
+    uint32_t Sc, Q;    // extent along c and along q
+    uint32_t ctiles, qtiles;
+    uint32_t group;    // tiles are walked in group x group blocks so that concurrently running workgroups
+    uint32_t cgroups;  // touch neighbouring segments on BOTH sides (DRAM row locality); cgroups = ceil(ctiles/group)
+    int n_inner;       // dimensions after c (decode q -> memory offset), outermost first
+    int n_outer;       // dimensions before c (decode batch -> memory offset), outermost first
+    uint32_t inner_size[kMaxCanonDims];
+    FastDiv32 inner_div[kMaxCanonDims];
+    uint64_t inner_stride[kMaxCanonDims];
+    uint32_t outer_size[kMaxCanonDims];
+    FastDiv32 outer_div[kMaxCanonDims];
+    uint64_t outer_stride[kMaxCanonDims];
+};
+
+// Unlike the streaming copies, these accesses are NOT marked non-temporal: a wavefront
+// touches only 64 elements of a row (128-256 bytes), so L2 write-combining and line reuse
+// between neighbouring workgroups matter (measured: bf16 4.4 TB/s cached vs 2.4 TB/s with nt).
+template <typename T> __device__ __forceinline__ T ldg(const T* p) { return *p; }
+template <typename T> __device__ __forceinline__ void stg(T* p, T v) { *p = v; }
+
+template <typename T, int TILE, bool PACK>
+__global__ __launch_bounds__(kThreads) void slice_transpose_kernel(TransArgs a) {
+    __shared__ T tile[TILE][TILE + 1];  // [q][c]
+    __shared__ uint64_t s_off[TILE];
+    constexpr int ROWS_PER_PASS = kThreads / TILE;
+    const int lane_x = threadIdx.x % TILE;  // position along the contiguous side of a pass
+    const int lane_y = threadIdx.x / TILE;
+    T* __restrict__ mem = reinterpret_cast<T*>(a.base) + a.offset;
+    T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
+    const uint64_t per_batch = (uint64_t)a.cgroups * ((a.qtiles + a.group - 1) / a.group) * a.group * a.group;
+
+    for (uint64_t tile_id = blockIdx.x; tile_id < a.ntiles; tile_id += gridDim.x) {
+        const uint64_t b = tile_id / per_batch;
+        const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
+        const uint32_t gsz = a.group * a.group;
+        const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
+        const uint32_t gq = grp / a.cgroups, gc = grp - gq * a.cgroups;
+        const uint32_t qt = gq * a.group + within / a.group, ct = gc * a.group + within % a.group;
+        if (qt >= a.qtiles || ct >= a.ctiles) continue;  // padding of the blocked walk (uniform per workgroup)
+        const uint32_t q0 = qt * TILE, c0 = ct * TILE;
+        // memory offset of the batch: decode b over the dimensions before c
+        uint64_t batch_off = 0;
+        {
+            uint64_t rem = b;
+            for (int k = a.n_outer - 1; k >= 0; --k) {
+                const uint64_t qd = rem / a.outer_size[k];
+                batch_off += (rem - qd * a.outer_size[k]) * a.outer_stride[k];
+                rem = qd;
+            }
+        }
+        if (threadIdx.x < TILE) {
+            uint32_t q = q0 + threadIdx.x;
+            uint64_t off = 0;
+            if (q < a.Q) {
+                for (int k = a.n_inner - 1; k > 0; --k) {
+                    uint32_t qd, r;
+                    a.inner_div[k].divmod(q, qd, r);
+                    off += (uint64_t)r * a.inner_stride[k];
+                    q = qd;
+                }
+                off += (uint64_t)q * a.inner_stride[0];
+            }
+            s_off[threadIdx.x] = off;
+        }
+        __syncthreads();
+        const uint64_t packed_row0 = (b * a.Sc + c0) * (uint64_t)a.Q + q0;  // packed index of tile element (c0, q0)
+        // Interior tiles take loops without bounds tests, so that all 16 loads of a lane are in
+        // flight before the first LDS write; edge tiles take the predicated form.
+        const bool full = q0 + TILE <= a.Q && c0 + TILE <= a.Sc;
+        const T* mem_tile = mem + batch_off + c0 + lane_x;              // + s_off[r] per row
+        T* mem_tile_w = mem + batch_off + c0 + lane_x;
+        T* packed_tile = packed + packed_row0 + lane_x;                 // + cc * Q per column
+        if constexpr (PACK) {
+            // memory -> LDS: lanes run along c
+            if (full) {
+                T v[TILE / ROWS_PER_PASS];
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i) v[i] = ldg(mem_tile + s_off[lane_y + i * ROWS_PER_PASS]);
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i) tile[lane_y + i * ROWS_PER_PASS][lane_x] = v[i];
+            } else {
+                for (int r = lane_y; r < TILE; r += ROWS_PER_PASS)
+                    if (q0 + r < a.Q && c0 + lane_x < a.Sc) tile[r][lane_x] = ldg(mem_tile + s_off[r]);
+            }
+            __syncthreads();
+            // LDS -> packed: lanes run along q
+            if (full) {
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i) {
+                    const int cc = lane_y + i * ROWS_PER_PASS;
+                    stg(packed_tile + (uint64_t)cc * a.Q, tile[lane_x][cc]);
+                }
+            } else {
+                for (int cc = lane_y; cc < TILE; cc += ROWS_PER_PASS)
+                    if (c0 + cc < a.Sc && q0 + lane_x < a.Q) stg(packed_tile + (uint64_t)cc * a.Q, tile[lane_x][cc]);
+            }
+        } else {
+            if (full) {
+                T v[TILE / ROWS_PER_PASS];
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i)
+                    v[i] = ldg(packed_tile + (uint64_t)(lane_y + i * ROWS_PER_PASS) * a.Q);
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i) tile[lane_x][lane_y + i * ROWS_PER_PASS] = v[i];
+            } else {
+                for (int cc = lane_y; cc < TILE; cc += ROWS_PER_PASS)
+                    if (c0 + cc < a.Sc && q0 + lane_x < a.Q) tile[lane_x][cc] = ldg(packed_tile + (uint64_t)cc * a.Q);
+            }
+            __syncthreads();
+            if (full) {
+#pragma unroll
+                for (int i = 0; i < TILE / ROWS_PER_PASS; ++i) {
+                    const int r = lane_y + i * ROWS_PER_PASS;
+                    stg(mem_tile_w + s_off[r], tile[r][lane_x]);
+                }
+            } else {
+                for (int r = lane_y; r < TILE; r += ROWS_PER_PASS)
+                    if (q0 + r < a.Q && c0 + lane_x < a.Sc) stg(mem_tile_w + s_off[r], tile[r][lane_x]);
+            }
+        }
+        __syncthreads();  // the tile and s_off are reused by the next iteration
+    }
+}
+
+template <bool PACK>
+bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t unit, hipStream_t stream, int* rc) {
+    if (c.run != 1 || c.ndim < 2 || c.ndim > kMaxCanonDims) return false;
+    int cd = -1;
+    for (int k = 0; k < c.ndim; ++k)
+        if (c.dims[k].stride == 1) cd = k;
+    if (cd < 0 || cd == c.ndim - 1) return false;
+    TransArgs a{};
+    uint64_t Q = 1, nbatch = 1;
+    for (int k = cd + 1; k < c.ndim; ++k) {
+        if (c.dims[k].size >= kFastDivLimit) return false;
+        Q *= c.dims[k].size;
+        if (Q >= kFastDivLimit) return false;
+        const int j = a.n_inner++;
+        a.inner_size[j] = (uint32_t)c.dims[k].size;
+        a.inner_div[j] = FastDiv32((uint32_t)c.dims[k].size);
+        a.inner_stride[j] = c.dims[k].stride;
+    }
+    for (int k = 0; k < cd; ++k) {
+        if (c.dims[k].size >= kFastDivLimit) return false;
+        nbatch *= c.dims[k].size;
+        const int j = a.n_outer++;
+        a.outer_size[j] = (uint32_t)c.dims[k].size;
+        a.outer_div[j] = FastDiv32((uint32_t)c.dims[k].size);
+        a.outer_stride[j] = c.dims[k].stride;
+    }
+    const uint64_t Sc = c.dims[cd].size;
+    // worth it only when both sides have something to coalesce
+    if (Sc < 8 || Q < 8 || Sc >= kFastDivLimit) return false;
+    const uint32_t tile = unit >= 8 ? 32 : 64;
+    a.base = base;
+    a.packed = packed;
+    a.offset = c.offset;
+    a.Sc = (uint32_t)Sc;
+    a.Q = (uint32_t)Q;
+    a.ctiles = (uint32_t)((Sc + tile - 1) / tile);
+    a.qtiles = (uint32_t)((Q + tile - 1) / tile);
+    a.group = 4;  // 4 x 4 tiles per block of the walk: +7% over a plain row-major walk at 8192^2 fp32
+    a.cgroups = (a.ctiles + a.group - 1) / a.group;
+    const uint64_t qgroups = (a.qtiles + a.group - 1) / a.group;
+    a.ntiles = nbatch * a.cgroups * qgroups * a.group * a.group;
+    const uint64_t cap = 0x7fffffffull;
+    const dim3 grid((uint32_t)(a.ntiles < cap ? a.ntiles : cap)), block(kThreads);
+    switch (unit) {
+        case 1: hipLaunchKernelGGL((slice_transpose_kernel<uint8_t, 64, PACK>), grid, block, 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((slice_transpose_kernel<uint16_t, 64, PACK>), grid, block, 0, stream, a); break;
+        case 4: hipLaunchKernelGGL((slice_transpose_kernel<uint32_t, 64, PACK>), grid, block, 0, stream, a); break;
+        case 8: hipLaunchKernelGGL((slice_transpose_kernel<uint64_t, 32, PACK>), grid, block, 0, stream, a); break;
+        case 16: hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), grid, block, 0, stream, a); break;
+        default: return false;
+    }
+    *rc = launch_status();
+    return true;
+}
+
+template bool try_transpose_copy<true>(char*, char*, const CanonSlice&, uint32_t, hipStream_t, int*);
+template bool try_transpose_copy<false>(char*, char*, const CanonSlice&, uint32_t, hipStream_t, int*);
+
+}  // namespace mhip

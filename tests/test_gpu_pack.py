@@ -227,3 +227,48 @@ def test_tensor_buffer_round_trip():
         staging.RDMABuffer(x.flatten())
     with pytest.raises(ValueError, match="must be <="):
         buf.read_into(torch.zeros(buf.size + 1, dtype=torch.uint8, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64, torch.complex128])
+def test_transposing_views_lds_path(dtype):
+    # permuted views: the memory-contiguous dimension is not the innermost iteration dimension
+    g = torch.Generator().manual_seed(11)
+    cases = [((70, 130), (1, 0)), ((64, 64), (1, 0)), ((5, 67, 33), (0, 2, 1)), ((5, 67, 33), (2, 1, 0)),
+             ((3, 4, 40, 50), (1, 3, 0, 2)), ((9, 200), (1, 0)), ((200, 9), (1, 0)), ((2, 3, 129, 65), (3, 0, 2, 1)),
+             ((33, 8, 8), (2, 1, 0))]
+    for shape, perm in cases:
+        n = int(np.prod(shape))
+        if dtype == torch.complex128:
+            host = torch.view_as_complex(torch.randn(n, 2, generator=g, dtype=torch.float64)).reshape(shape)
+        else:
+            info = torch.iinfo(dtype)
+            host = torch.randint(info.min, info.max, shape, dtype=dtype, generator=g)
+        dev = host.to(DEV)
+        view = dev.permute(perm)[..., 1:] if len(shape) > 2 else dev.permute(perm)
+        hview = host.permute(perm)[..., 1:] if len(shape) > 2 else host.permute(perm)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.cpu(), hview.contiguous().flatten()), (shape, perm, dtype)
+        back = torch.zeros_like(dev)
+        staging.unpack(back, s, out)
+        sync()
+        ref = torch.zeros_like(host)
+        (ref.permute(perm)[..., 1:] if len(shape) > 2 else ref.permute(perm)).copy_(hview)
+        assert torch.equal(back.cpu(), ref), (shape, perm, dtype)
+        if dtype in (torch.int16, torch.int32):
+            hb = host.numpy().reshape(-1)
+            assert np.array_equal(out.cpu().numpy(), oracle.pack(hb, oslice(s)))
+
+
+def test_transpose_large_square():
+    g = torch.Generator(device=DEV).manual_seed(12)
+    x = (torch.randn(4096, 4096, generator=g, device=DEV)).bfloat16()
+    s = Slice(offset=0, sizes=[4096, 4096], strides=[1, 4096])
+    out = staging.pack(x, s)
+    sync()
+    assert torch.equal(out.view(4096, 4096).view(torch.int16), x.t().contiguous().view(torch.int16))
+    back = torch.zeros_like(x)
+    staging.unpack(back, s, out)
+    sync()
+    assert torch.equal(back.view(torch.int16), x.view(torch.int16))
