@@ -38,9 +38,12 @@ inline bool make_dims_arg(const CanonSlice& c, DimsArg* d, bool* fits32) {
 }
 
 // Unit offset of packed unit t, and its column within the row (for run-boundary tests).
-template <bool WIDE>
+// NDIM >= 0 fixes the number of dimensions outside the run at compile time (no loop, no
+// kernel-argument loads inside the decode); NDIM < 0 reads it from the arguments.
+template <bool WIDE, int NDIM = -1>
 __device__ __forceinline__ uint64_t decode(const DimsArg& d, uint64_t t, uint64_t* col_out) {
-    if (d.ndim == 0) {
+    const int ndim = NDIM >= 0 ? NDIM : d.ndim;
+    if (ndim == 0) {
         *col_out = t;  // one row: run == total
         return t;
     }
@@ -50,7 +53,7 @@ __device__ __forceinline__ uint64_t decode(const DimsArg& d, uint64_t t, uint64_
         uint64_t col = t - row * d.run;
         *col_out = col;
         off = col;
-        for (int k = d.ndim - 1; k > 0; --k) {
+        for (int k = ndim - 1; k > 0; --k) {
             uint64_t q = row / d.size[k];
             off += (row - q * d.size[k]) * d.stride[k];
             row = q;
@@ -61,11 +64,21 @@ __device__ __forceinline__ uint64_t decode(const DimsArg& d, uint64_t t, uint64_
         d.run_div.divmod((uint32_t)t, row, col);
         *col_out = col;
         off = col;
-        for (int k = d.ndim - 1; k > 0; --k) {
-            uint32_t q, r;
-            d.size_div[k].divmod(row, q, r);
-            off += (uint64_t)r * d.stride[k];
-            row = q;
+        if constexpr (NDIM >= 0) {
+#pragma unroll
+            for (int k = NDIM - 1; k > 0; --k) {
+                uint32_t q, r;
+                d.size_div[k].divmod(row, q, r);
+                off += (uint64_t)r * d.stride[k];
+                row = q;
+            }
+        } else {
+            for (int k = ndim - 1; k > 0; --k) {
+                uint32_t q, r;
+                d.size_div[k].divmod(row, q, r);
+                off += (uint64_t)r * d.stride[k];
+                row = q;
+            }
         }
         off += (uint64_t)row * d.stride[0];
     }

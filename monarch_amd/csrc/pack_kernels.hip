@@ -33,13 +33,36 @@ __device__ __forceinline__ void move_unit(char* strided, char* packed) {
         *reinterpret_cast<T*>(strided) = *reinterpret_cast<const T*>(packed);
 }
 
-template <int U, bool PACK, bool WIDE>
+template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     constexpr int VU = 16 / U;  // units per chunk
     const int v = blockIdx.y;
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+
+    if constexpr (NDIM == 0) {
+        // Contiguous view: when the whole 32 KiB tile of this workgroup lies inside the
+        // buffer (decided on the scalar unit), no per-chunk tests are needed at all.
+        const uint64_t tile_first = (uint64_t)blockIdx.x * (kThreads * kUnroll) * VU;
+        const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
+        if (tile_first >= a.shift && tile_end - a.shift <= a.total) {
+            char* __restrict__ p = packed + (c0 * VU - a.shift) * U;
+            char* __restrict__ s = strided + (c0 * VU - a.shift) * U;
+            uint4 d[kUnroll];
+#pragma unroll
+            for (int i = 0; i < kUnroll; ++i) {
+                if constexpr (PACK) d[i] = load16_unaligned(s + (size_t)i * kThreads * 16);
+                else d[i] = load16_aligned(p + (size_t)i * kThreads * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < kUnroll; ++i) {
+                if constexpr (PACK) store16_aligned(p + (size_t)i * kThreads * 16, d[i]);
+                else store16_unaligned(s + (size_t)i * kThreads * 16, d[i]);
+            }
+            return;
+        }
+    }
 
     uint64_t loc[kUnroll];
     uint64_t first[kUnroll];  // first packed unit of the chunk (may be "negative": see below)
@@ -54,7 +77,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
         first[i] = tb - a.shift;     // wraps for a ragged chunk 0; only used when tb >= shift
         if (live[i] && tb >= a.shift && first[i] + VU <= a.total) {
             uint64_t col;
-            loc[i] = decode<WIDE>(a.dims, first[i], &col);
+            loc[i] = decode<WIDE, NDIM>(a.dims, first[i], &col);
             vec[i] = col + VU <= a.dims.run;
         }
     }
@@ -107,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
                     const uint64_t t = tb + j - a.shift;
                     if (tb + j >= a.shift && t < a.total) {
                         uint64_t col;
-                        const uint64_t l = decode<WIDE>(a.dims, t, &col);
+                        const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
                         move_unit<U, PACK>(strided + l * U, packed + t * U);
                     }
                 }
@@ -215,14 +238,29 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
 
 // ---------------- host side ----------------
 
-template <bool PACK, bool WIDE>
-static void launch_slice_copy(uint32_t unit, dim3 grid, hipStream_t stream, const PackArgs& a) {
+template <int U, bool PACK>
+static void launch_slice_copy_u(bool wide, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
+    const dim3 block(kThreads);
+    if (wide) {
+        hipLaunchKernelGGL((slice_copy_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
+        return;
+    }
+    switch (ndim) {  // the common shapes get a decode without loops
+        case 0: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 0>), grid, block, 0, stream, a); break;
+        case 1: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
+    }
+}
+
+template <bool PACK>
+static void launch_slice_copy(uint32_t unit, bool wide, dim3 grid, hipStream_t stream, const PackArgs& a) {
     switch (unit) {
-        case 1: hipLaunchKernelGGL((slice_copy_kernel<1, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((slice_copy_kernel<2, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
-        case 4: hipLaunchKernelGGL((slice_copy_kernel<4, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
-        case 8: hipLaunchKernelGGL((slice_copy_kernel<8, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
-        default: hipLaunchKernelGGL((slice_copy_kernel<16, PACK, WIDE>), grid, dim3(kThreads), 0, stream, a); break;
+        case 1: launch_slice_copy_u<1, PACK>(wide, a.dims.ndim, grid, stream, a); break;
+        case 2: launch_slice_copy_u<2, PACK>(wide, a.dims.ndim, grid, stream, a); break;
+        case 4: launch_slice_copy_u<4, PACK>(wide, a.dims.ndim, grid, stream, a); break;
+        case 8: launch_slice_copy_u<8, PACK>(wide, a.dims.ndim, grid, stream, a); break;
+        default: launch_slice_copy_u<16, PACK>(wide, a.dims.ndim, grid, stream, a); break;
     }
 }
 
@@ -297,10 +335,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
         if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
         dim3 grid((uint32_t)blocks, nbatch);
-        if (fits32)
-            launch_slice_copy<PACK, false>(unit, grid, stream, a);
-        else
-            launch_slice_copy<PACK, true>(unit, grid, stream, a);
+        launch_slice_copy<PACK>(unit, !fits32, grid, stream, a);
         if (int rc = launch_status()) return rc;
         k += nbatch;
     }
