@@ -28,8 +28,11 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
-MEASURED_TRAFFIC = {
-    "c2": 452_348_918,  # profiles/reduce_kernel_bf16_c2.md: 0.9986 x the algorithmic bytes
+MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
+    "c2": 452_659_750, "c2_inplace": 452_659_692, "c2p_pack": 100_663_296, "c2p_unpack": 100_661_715,
+    "c3_pack": 234_810_402, "c3_unpack": 234_815_974, "c4": 603_524_872,
+    "c5_flat_pack": 3_210_331_152, "c5_quantize": 2_361_569_907, "c5_dequant": 7_100_632_520,
+    "c5_flat_unpack": 6_100_598_486, "tr_f32_pack": 536_653_207, "tr_bf16_pack": 268_365_014,
 }
 
 
