@@ -21,6 +21,7 @@ struct PackArgs {
     uint64_t total;              // units per view
     uint64_t nchunks;            // 16-byte chunks per view, including a ragged first one
     uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
+    uint32_t nviews;             // views handled by this launch
     DimsArg dims;
 };
 
@@ -36,15 +37,19 @@ __device__ __forceinline__ void move_unit(char* strided, char* packed) {
 template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     constexpr int VU = 16 / U;  // units per chunk
-    const int v = blockIdx.y;
+    // The view index is the fastest-varying part of the workgroup id, so that workgroups
+    // running side by side work on the same rows of neighbouring views (for column blocks
+    // of one tensor: neighbouring segments of the same rows).
+    const uint32_t v = blockIdx.x % a.nviews;
+    const uint64_t tile = blockIdx.x / a.nviews;
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
-    const uint64_t c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll) + threadIdx.x;
+    const uint64_t c0 = tile * (kThreads * kUnroll) + threadIdx.x;
 
     if constexpr (NDIM == 0) {
         // Contiguous view: when the whole 32 KiB tile of this workgroup lies inside the
         // buffer (decided on the scalar unit), no per-chunk tests are needed at all.
-        const uint64_t tile_first = (uint64_t)blockIdx.x * (kThreads * kUnroll) * VU;
+        const uint64_t tile_first = tile * (kThreads * kUnroll) * VU;
         const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
         if (tile_first >= a.shift && tile_end - a.shift <= a.total) {
             char* __restrict__ p = packed + (c0 * VU - a.shift) * U;
@@ -333,8 +338,9 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         }
         const uint64_t per_block = (uint64_t)kThreads * kUnroll;
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
-        if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
-        dim3 grid((uint32_t)blocks, nbatch);
+        if (blocks * nbatch > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
+        a.nviews = nbatch;
+        dim3 grid((uint32_t)(blocks * nbatch));
         launch_slice_copy<PACK>(unit, !fits32, grid, stream, a);
         if (int rc = launch_status()) return rc;
         k += nbatch;

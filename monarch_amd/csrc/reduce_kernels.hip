@@ -195,6 +195,7 @@ struct ScatterArgs {
     uint64_t total;                    // units per output
     uint64_t in_offset;                // units
     uint32_t n_in;
+    uint32_t n_out;                    // outputs handled by this launch
     float scale;
     float divisor;
     DimsArg out_dims;                  // packed output index -> reduced-tensor index
@@ -207,9 +208,14 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
     using VT = Vec<T>;
     using acc_t = typename VT::acc_t;
     constexpr int V = VT::V;
-    const int k = blockIdx.y;
-    const uint64_t stride = (uint64_t)gridDim.x * kReduceThreads;
-    for (uint64_t t = (uint64_t)blockIdx.x * kReduceThreads + threadIdx.x; t < a.total; t += stride) {
+    // The output index is the FASTEST-varying part of the workgroup id: workgroups that run
+    // side by side handle the same position of neighbouring outputs, which for column-block
+    // scatters are neighbouring segments of the same input rows (sequential HBM reads).
+    const uint32_t nk = a.n_out;
+    const uint32_t k = blockIdx.x % nk;
+    const uint64_t tile0 = blockIdx.x / nk;
+    const uint64_t stride = (uint64_t)(gridDim.x / nk) * kReduceThreads;
+    for (uint64_t t = tile0 * kReduceThreads + threadIdx.x; t < a.total; t += stride) {
         uint64_t col;
         const uint64_t i = a.out_offset[k] + decode<WIDE>(a.out_dims, t, &col);
         const uint64_t loc = a.in_offset + decode<WIDE>(a.in_dims, i, &col);
@@ -446,7 +452,10 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
             a.out_offset[nbatch] = nc.offset;
             ++nbatch;
         }
-        dim3 grid(grid_for(a.total), nbatch);
+        a.n_out = nbatch;
+        uint64_t tiles = grid_for(a.total);
+        while (tiles * nbatch > 0x7fffffffull) tiles = (tiles + 1) / 2;  // grid-stride takes over
+        dim3 grid((uint32_t)(tiles * nbatch));
         const bool avg = op == MHIP_OP_AVG;
         switch (dtype) {
             case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, avg, wide, hs); break;
