@@ -19,14 +19,19 @@ struct DimsArg {
     int ndim;
 };
 
-inline bool make_dims_arg(const CanonSlice& c, DimsArg* d, bool* fits32) {
-    if (c.ndim > kMaxCanonDims) return false;
+// `pad_to` > 0 left-pads the dimension list with (size 1, stride 0) entries up to that many
+// dimensions, so that a kernel compiled for a fixed count can decode shorter slices.
+inline bool make_dims_arg(const CanonSlice& c, DimsArg* d, bool* fits32, int pad_to = 0) {
+    if (c.ndim > kMaxCanonDims || pad_to > kMaxCanonDims) return false;
+    const int nd = pad_to > c.ndim ? pad_to : c.ndim;
+    const int lead = nd - c.ndim;
     d->run = c.run;
-    d->ndim = c.ndim;
+    d->ndim = nd;
     bool small = c.total < kFastDivLimit - 64 && c.run < kFastDivLimit;
     for (int k = 0; k < kMaxCanonDims; ++k) {
-        d->size[k] = k < c.ndim ? c.dims[k].size : 1;
-        d->stride[k] = k < c.ndim ? c.dims[k].stride : 0;
+        const bool real = k >= lead && k < nd;
+        d->size[k] = real ? c.dims[k - lead].size : 1;
+        d->stride[k] = real ? c.dims[k - lead].stride : 0;
         if (d->size[k] >= kFastDivLimit) small = false;
     }
     if (small) {

@@ -40,8 +40,8 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
-    const uint32_t v = blockIdx.x % a.nviews;
     const uint64_t tile = blockIdx.x / a.nviews;
+    const uint32_t v = blockIdx.x % a.nviews;
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = tile * (kThreads * kUnroll) + threadIdx.x;

@@ -203,7 +203,9 @@ struct ScatterArgs {
 };
 
 // VEC: a unit is 16 bytes (V elements) and never straddles a row of either view.
-template <typename T, bool VEC, bool AVG, bool WIDE>
+// D: number of dimensions (outside the run) both decodes are compiled for; shorter views
+// are padded on the host.  D < 0 reads the counts from the arguments.
+template <typename T, bool VEC, bool AVG, bool WIDE, int D>
 __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterArgs a) {
     using VT = Vec<T>;
     using acc_t = typename VT::acc_t;
@@ -211,14 +213,16 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
     // The output index is the FASTEST-varying part of the workgroup id: workgroups that run
     // side by side handle the same position of neighbouring outputs, which for column-block
     // scatters are neighbouring segments of the same input rows (sequential HBM reads).
+    // (Rotating k by the tile number, so that an output is not pinned to one XCD, was
+    // measured and does not help: -6% on flat chunks, +0.5% on column blocks.)
     const uint32_t nk = a.n_out;
-    const uint32_t k = blockIdx.x % nk;
     const uint64_t tile0 = blockIdx.x / nk;
+    const uint32_t k = blockIdx.x % nk;
     const uint64_t stride = (uint64_t)(gridDim.x / nk) * kReduceThreads;
     for (uint64_t t = tile0 * kReduceThreads + threadIdx.x; t < a.total; t += stride) {
         uint64_t col;
-        const uint64_t i = a.out_offset[k] + decode<WIDE>(a.out_dims, t, &col);
-        const uint64_t loc = a.in_offset + decode<WIDE>(a.in_dims, i, &col);
+        const uint64_t i = a.out_offset[k] + decode<WIDE, D>(a.out_dims, t, &col);
+        const uint64_t loc = a.in_offset + decode<WIDE, D>(a.in_dims, i, &col);
         if constexpr (VEC) {
             acc_t acc[V];
             VT::widen(load16_unaligned(static_cast<const char*>(a.in[0]) + loc * 16), acc);
@@ -300,18 +304,27 @@ static void launch_reduce(const ReduceArgs& a, int op, hipStream_t s) {
     if (op == MHIP_OP_AVG) launch_reduce_n<T, true>(a, s); else launch_reduce_n<T, false>(a, s);
 }
 
-template <typename T>
-static void launch_scatter(const ScatterArgs& a, dim3 grid, bool vec, bool avg, bool wide, hipStream_t s) {
+template <typename T, bool VEC, bool AVG>
+static void launch_scatter_d(const ScatterArgs& a, dim3 grid, bool wide, int d, hipStream_t s) {
     const dim3 block(kReduceThreads);
-#define MHIP_RS(VEC, AVG, WIDE) hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, WIDE>), grid, block, 0, s, a)
-    if (vec) {
-        if (avg) { if (wide) MHIP_RS(true, true, true); else MHIP_RS(true, true, false); }
-        else     { if (wide) MHIP_RS(true, false, true); else MHIP_RS(true, false, false); }
-    } else {
-        if (avg) { if (wide) MHIP_RS(false, true, true); else MHIP_RS(false, true, false); }
-        else     { if (wide) MHIP_RS(false, false, true); else MHIP_RS(false, false, false); }
+    if (wide) { hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, true, -1>), grid, block, 0, s, a); return; }
+    switch (d) {
+        case 2: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, 2>), grid, block, 0, s, a); break;
+        case 4: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, 4>), grid, block, 0, s, a); break;
+        default: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, -1>), grid, block, 0, s, a); break;
     }
-#undef MHIP_RS
+}
+
+template <typename T>
+static void launch_scatter(const ScatterArgs& a, dim3 grid, bool vec, bool avg, bool wide, int d, hipStream_t s) {
+    constexpr bool kFloat = std::is_floating_point<typename Vec<T>::acc_t>::value;
+    if constexpr (kFloat) {
+        if (avg) {
+            if (vec) launch_scatter_d<T, true, true>(a, grid, wide, d, s); else launch_scatter_d<T, false, true>(a, grid, wide, d, s);
+            return;
+        }
+    }
+    if (vec) launch_scatter_d<T, true, false>(a, grid, wide, d, s); else launch_scatter_d<T, false, false>(a, grid, wide, d, s);
 }
 
 }  // namespace mhip
@@ -430,7 +443,9 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         const bool vec = max_unit == V;
         ScatterArgs a{};
         bool o32 = false, i32 = false;
-        if (!make_dims_arg(oc, &a.out_dims, &o32) || !make_dims_arg(ic, &a.in_dims, &i32))
+        const int nd = oc.ndim > ic.ndim ? oc.ndim : ic.ndim;
+        const int d = nd <= 2 ? 2 : (nd <= 4 ? 4 : -1);  // compiled decode depths
+        if (!make_dims_arg(oc, &a.out_dims, &o32, d > 0 ? d : 0) || !make_dims_arg(ic, &a.in_dims, &i32, d > 0 ? d : 0))
             return MHIP_ERR_UNSUPPORTED_OP;
         // the output decode yields reduced-tensor indices that the input decode divides again
         const bool wide = !(o32 && i32 && ic.total < kFastDivLimit - 64);
@@ -458,13 +473,13 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         dim3 grid((uint32_t)(tiles * nbatch));
         const bool avg = op == MHIP_OP_AVG;
         switch (dtype) {
-            case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_BF16: launch_scatter<bf16_tag>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_F16: launch_scatter<_Float16>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_F64: launch_scatter<double>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_scatter<uint8_t>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_I32: launch_scatter<uint32_t>(a, grid, vec, avg, wide, hs); break;
-            case MHIP_DTYPE_I64: launch_scatter<uint64_t>(a, grid, vec, avg, wide, hs); break;
+            case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_BF16: launch_scatter<bf16_tag>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_F16: launch_scatter<_Float16>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_F64: launch_scatter<double>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_scatter<uint8_t>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_I32: launch_scatter<uint32_t>(a, grid, vec, avg, wide, d, hs); break;
+            case MHIP_DTYPE_I64: launch_scatter<uint64_t>(a, grid, vec, avg, wide, d, hs); break;
             default: return MHIP_ERR_INVALID_DATA_TYPE;
         }
         if (int rc = launch_status()) return rc;
