@@ -217,10 +217,18 @@ _REDUCE = {"float32": "o_reduce_f32", "float64": "o_reduce_f64", "uint16": "o_re
 SUM, AVG = 0, 4
 
 
-def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = None) -> np.ndarray:
-    """Elementwise Sum/Avg over ``ins``.  bf16 data is passed as uint16 bit patterns."""
+def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = None, half: bool = False) -> np.ndarray:
+    """Elementwise Sum/Avg over ``ins``.  bf16 data is passed as uint16 bit patterns
+    (``half=True``: the uint16 patterns are IEEE binary16 instead)."""
     ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
     dt = ins[0].dtype
+    if half:
+        assert dt == np.uint16
+        if out is None:
+            out = np.empty_like(ins[0])
+        ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+        lib().o_reduce_f16(_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint64(ins[0].size), C.c_int(op))
+        return out
     if out is None:
         out = np.empty_like(ins[0])
     ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
@@ -258,6 +266,20 @@ def f32_to_bf16(x: np.ndarray) -> np.ndarray:
     x = np.ascontiguousarray(x, dtype=np.float32)
     out = np.empty(x.shape, dtype=np.uint16)
     lib().o_f32_to_bf16(_ptr(out), _ptr(x), C.c_uint64(x.size))
+    return out
+
+
+def f16_to_f32(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().o_f16_to_f32(_ptr(out), _ptr(x), C.c_uint64(x.size))
+    return out
+
+
+def f32_to_f16(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().o_f32_to_f16(_ptr(out), _ptr(x), C.c_uint64(x.size))
     return out
 
 

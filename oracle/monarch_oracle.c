@@ -330,6 +330,55 @@ void o_f32_to_bf16(uint16_t* out, const float* in, uint64_t n) {
     for (uint64_t i = 0; i < n; i++) out[i] = f32_to_bf16_rne(in[i]);
 }
 
+/* ---- IEEE binary16 helpers (widening exact, narrowing round-to-nearest-even) ---- */
+static inline float f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1f, m = h & 0x3ffu;
+    float v;
+    if (e == 0)
+        v = ldexpf((float)m, -24); /* zero and subnormals */
+    else if (e == 31) {
+        uint32_t u = 0x7f800000u | (m << 13);
+        memcpy(&v, &u, 4);
+    } else
+        v = ldexpf((float)(m | 0x400u), (int)e - 25);
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    u |= sign;
+    memcpy(&v, &u, 4);
+    return v;
+}
+static inline uint16_t f32_to_f16_rne(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u); /* NaN -> quiet NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u); /* >= 65536: infinity (also catches inf) */
+    float av;
+    memcpy(&av, &a, 4);
+    if (a < 0x38800000u) { /* below 2^-14: subnormal grid of 2^-24 */
+        uint32_t m = (uint32_t)rintf(ldexpf(av, 24));
+        return (uint16_t)(sign | m); /* m == 1024 lands on the smallest normal */
+    }
+    int ex;
+    float fr = frexpf(av, &ex); /* av = fr * 2^ex, fr in [0.5, 1) */
+    uint32_t m = (uint32_t)rintf((2.0f * fr - 1.0f) * 1024.0f);
+    int e = ex - 1 + 15;
+    if (m == 1024) {
+        m = 0;
+        e += 1;
+    }
+    if (e >= 31) return (uint16_t)(sign | 0x7c00u); /* 65520 and above round to infinity */
+    return (uint16_t)(sign | ((uint32_t)e << 10) | m);
+}
+void o_f16_to_f32(float* out, const uint16_t* in, uint64_t n) {
+    for (uint64_t i = 0; i < n; i++) out[i] = f16_to_f32(in[i]);
+}
+void o_f32_to_f16(uint16_t* out, const float* in, uint64_t n) {
+    for (uint64_t i = 0; i < n; i++) out[i] = f32_to_f16_rne(in[i]);
+}
+
 /* ---- Reduce, non-scatter: out = op over the n chunks this GPU holds ----
  * Semantics of StreamActor::reduce's all_reduce branch
  * (monarch_tensor_worker/src/stream.rs:1437-1462; python/monarch/worker/worker.py:251-255):
@@ -352,6 +401,14 @@ void o_reduce_bf16(uint16_t* out, const uint16_t* const* in, uint32_t n, uint64_
         for (uint32_t r = 1; r < n; r++) acc += bf16_to_f32(in[r][i]);
         if (op == 4) acc = acc / (float)n;
         out[i] = f32_to_bf16_rne(acc);
+    }
+}
+void o_reduce_f16(uint16_t* out, const uint16_t* const* in, uint32_t n, uint64_t numel, int op) {
+    for (uint64_t i = 0; i < numel; i++) {
+        float acc = f16_to_f32(in[0][i]);
+        for (uint32_t r = 1; r < n; r++) acc += f16_to_f32(in[r][i]);
+        if (op == 4) acc = acc / (float)n;
+        out[i] = f32_to_f16_rne(acc);
     }
 }
 void o_reduce_f64(double* out, const double* const* in, uint32_t n, uint64_t numel, int op) {

@@ -37,15 +37,7 @@ def _rand(dtype, n, seed):
 
 
 def _oracle_reduce(hosts, op, dtype):
-    if dtype == torch.float16:
-        # the oracle has no fp16 kernel: fp32 accumulate in rank order, one rounding (same rule as bf16)
-        acc = hosts[0].float()
-        for h in hosts[1:]:
-            acc = acc + h.float()
-        if op == AVG:
-            acc = acc / np.float32(len(hosts))
-        return bits(acc.to(torch.float16))
-    return oracle.reduce([bits(h) for h in hosts], op)
+    return oracle.reduce([bits(h) for h in hosts], op, half=dtype == torch.float16)
 
 
 def test_golden_vectors(vec):

@@ -44,6 +44,32 @@ def test_bf16_round_matches_torch():
     assert np.array_equal(back.view(np.uint32), h.astype(np.uint32) << 16)
 
 
+def test_f16_round_matches_torch():
+    h = np.arange(65536, dtype=np.uint16)
+    want = torch.from_numpy(h.view(np.int16).copy()).view(torch.float16).float().numpy()
+    got = oracle.f16_to_f32(h)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan) and np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    rng = np.random.default_rng(1)
+    u = rng.integers(0, 2**32, size=1_000_000, dtype=np.uint64).astype(np.uint32)
+    small = rng.normal(0, 1e-4, size=300_000).astype(np.float32).view(np.uint32)   # subnormal halves and ties
+    edge = np.array([65504.0, 65519.9, 65520.0, 65536.0, 1e9, 2.0**-24, 2.0**-25, 1.5 * 2.0**-25, 2.0**-14, 0.0, -0.0],
+                    dtype=np.float32).view(np.uint32)
+    ties = ((rng.integers(0, 2**19, size=100_000, dtype=np.uint64).astype(np.uint32) << 13) | 0x1000) + 0x38000000
+    u = np.concatenate([u, small, edge, ties, ties + 1, ties - 1])
+    f = u.view(np.float32)
+    got = oracle.f32_to_f16(f)
+    want = torch.from_numpy(f).to(torch.float16).view(torch.int16).numpy().view(np.uint16)
+    nan = np.isnan(f)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all((got[nan] & 0x7FFF) > 0x7C00)
+    a = torch.randn(5000).half()
+    b = torch.randn(5000).half()
+    got = oracle.reduce([a.view(torch.int16).numpy().view(np.uint16), b.view(torch.int16).numpy().view(np.uint16)], AVG, half=True)
+    want = ((a.float() + b.float()) / 2).half().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+
+
 def test_reduce_golden(vec):
     for case in vec["reduce"]:
         ins = [np.array(x, dtype=np.float32) for x in case["inputs"]]
