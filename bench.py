@@ -300,6 +300,17 @@ def wl_c5(torch, stage="quantize"):
     elif stage == "quantize":
         nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_kernel"
         launch = prepared("mhip_fp8_quantize", q.data_ptr(), s.data_ptr(), flat.data_ptr(), total, 1024, STREAM())
+    elif stage == "quantize_bucket":
+        nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_bucket_kernel"
+        launch = prepared("mhip_fp8_quantize_bucket", q.data_ptr(), s.data_ptr(), bucket.d_ptrs.data_ptr(),
+                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, STREAM())
+    elif stage == "dequant_bucket":
+        nbytes, kern = 9 * total + 4 * nblk, "fp8_dequant_accumulate_bucket_kernel"
+        accs = [torch.zeros(n, device="cuda:0") for n in sizes]
+        aptrs = bucket.pointer_table(accs)
+        launch = prepared("mhip_fp8_dequant_accumulate_bucket", aptrs.data_ptr(), q.data_ptr(), s.data_ptr(),
+                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, STREAM())
+        launch.keep = accs
     elif stage == "dequant_accumulate":
         nbytes, kern = 9 * total + 4 * nblk, "fp8_dequant_accumulate_kernel"
         launch = prepared("mhip_fp8_dequant_accumulate", acc.data_ptr(), q.data_ptr(), s.data_ptr(), total, 1024,
@@ -317,9 +328,9 @@ def wl_c5(torch, stage="quantize"):
         sample = min(total, 64 * 1024 * 1024)
         h = flat[:sample].cpu().view(torch.uint16).numpy()
         t0 = time.perf_counter()
-        if stage == "quantize":
+        if stage in ("quantize", "quantize_bucket"):
             oracle.fp8_quantize(h, 1024)
-        elif stage == "dequant_accumulate":
+        elif stage in ("dequant_accumulate", "dequant_bucket"):
             hq, hs = q[:sample].cpu().numpy(), s[: (sample + 1023) // 1024].cpu().numpy()
             ha = np.zeros(sample, dtype=np.float32)
             t0 = time.perf_counter()
@@ -347,6 +358,8 @@ WORKLOADS = {
     "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
     "c5_quantize": lambda t: wl_c5(t, "quantize"),
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
+    "c5_quantize_bucket": lambda t: wl_c5(t, "quantize_bucket"),
+    "c5_dequant_bucket": lambda t: wl_c5(t, "dequant_bucket"),
     "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
 }
 

@@ -191,8 +191,8 @@ int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d
 
 /* out[i] = op_r in[r][i], r in [0, n): the local combine of Communicator::all_reduce
  * (torch-sys-cuda/src/nccl.rs:464-489) as StreamActor::reduce uses it
- * (monarch_tensor_worker/src/stream.rs:1437-1462).  out may alias in[0] (the in-place
- * form); any other overlap is undefined.  Floating types accumulate in fp32 (f64 in f64)
+ * (monarch_tensor_worker/src/stream.rs:1437-1462).  out may coincide with exactly one of
+ * the inputs (the in-place form); any other overlap is undefined.  Floating types accumulate in fp32 (f64 in f64)
  * in rank order and round once; Avg divides the sum by n.  Integer Sum wraps.
  * Argument checks follow nccl.rs:300-316,474-476: null pointer -> UNDEFINED_TENSOR,
  * unknown dtype -> INVALID_DATA_TYPE, fp8 dtype -> FLOAT8_REDUCTION; ops other than
@@ -225,6 +225,19 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
 /* acc[i] += float(q[i]) * scales[i / block]; product rounded to fp32, then added. */
 int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scales, uint64_t numel,
                                 uint32_t block, mhip_stream_t stream);
+
+/* Fused forms on a tensor bucket (device tables as for mhip_flat_pack): bit-identical to
+ * mhip_flat_pack (bf16) + mhip_fp8_quantize, resp. to mhip_fp8_dequant_accumulate on a flat
+ * fp32 accumulator + mhip_flat_unpack, without materialising the flat buffers.  Blocks are
+ * still counted over the bucket's flat index space.  d_tensors: bf16 inputs;
+ * d_acc_tensors: fp32 accumulators, updated in place. */
+int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_tensors,
+                             const uint64_t* d_offsets, uint32_t ntensors, uint64_t total,
+                             uint32_t block, mhip_stream_t stream);
+int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t* q,
+                                       const float* scales, const uint64_t* d_offsets,
+                                       uint32_t ntensors, uint64_t total, uint32_t block,
+                                       mhip_stream_t stream);
 
 /* ====================================================================== */
 /* Runtime pass-through (the cuda-sys / nccl-sys symbols this path uses)   */

@@ -8,57 +8,9 @@
 //   memory - and the 16 codes leave as two 64-bit stores.
 // dequant_accumulate: 9 bytes per element (1 code in, fp32 accumulator in and out).
 //   A 256-thread workgroup step covers exactly one block, so the scale is uniform.
-#include <cfloat>
-
-#include "mhip_device.h"
+#include "fp8_common.h"
 
 namespace mhip {
-
-constexpr uint32_t kBlock = 1024;         // elements per scale
-constexpr float kFp8Max = 448.0f;
-constexpr float kAbsmaxFloor = 0x1p-40f;  // keeps 448/absmax finite for all-zero / denormal blocks
-
-// all-reduce max over the 64 lanes of a wavefront, for unsigned 32-bit values
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-    // DPP butterfly within each row of 16 lanes
-    uint32_t o;
-    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
-    v = v > o ? v : o;
-    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true);   // quad_perm [2,3,0,1]
-    v = v > o ? v : o;
-    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true);  // row_half_mirror
-    v = v > o ? v : o;
-    o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xF, 0xF, true);  // row_mirror
-    v = v > o ? v : o;
-    // one value per row, combined on the scalar unit
-    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0);
-    const uint32_t r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
-    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32);
-    const uint32_t r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
-    const uint32_t a = r0 > r1 ? r0 : r1, b = r2 > r3 ? r2 : r3;
-    return a > b ? a : b;
-}
-
-__device__ __forceinline__ void block_factors(uint32_t absmax_bf16_bits, float* scale, float* inv) {
-    float absmax = __uint_as_float(absmax_bf16_bits << 16);
-    absmax = absmax < kAbsmaxFloor ? kAbsmaxFloor : absmax;
-    absmax = absmax > FLT_MAX ? FLT_MAX : absmax;
-    *scale = absmax / kFp8Max;
-    *inv = kFp8Max / absmax;
-}
-
-// two bf16 values (one 32-bit word) -> two fp8 codes in the low or high half of `old`
-template <bool HIGH>
-__device__ __forceinline__ int quant_pair(uint32_t w, float inv, int old) {
-    return __builtin_amdgcn_cvt_pk_fp8_f32(bf16_lo(w) * inv, bf16_hi(w) * inv, old, HIGH);
-}
-
-__device__ __forceinline__ uint8_t quant_one_careful(uint32_t h, float inv) {
-    float y = __uint_as_float(h << 16) * inv;
-    y = y > kFp8Max ? kFp8Max : y;    // comparisons are false for NaN: it passes through
-    y = y < -kFp8Max ? -kFp8Max : y;
-    return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false) & 0xff);
-}
 
 // Careful path for one block, whole wavefront: handles a short final block and blocks
 // holding NaN or Inf (NaN is ignored by the absmax and encodes to an fp8 NaN; Inf

@@ -7,6 +7,7 @@
 // and tail).  Consecutive lanes take consecutive chunks, so each wavefront instruction
 // touches 1 KiB of contiguous staging memory.
 #include "mhip_device.h"
+#include "fp8_common.h"
 #include "pack_internal.h"
 
 namespace mhip {
@@ -157,29 +158,26 @@ struct FlatArgs {
     uint32_t units_per_elem;
 };
 
-// largest t in [lo, hi) with offsets[t] * upe <= unit
-__device__ __forceinline__ uint32_t find_tensor(const uint64_t* __restrict__ offsets, uint32_t upe, uint32_t lo,
-                                                uint32_t hi, uint64_t unit) {
-    while (hi - lo > 1) {
-        const uint32_t mid = lo + ((hi - lo) >> 1);
-        if (offsets[mid] * upe <= unit) lo = mid; else hi = mid;
-    }
-    return lo;
-}
-
 template <int U, bool PACK>
 __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     constexpr int VU = 16 / U;
     __shared__ uint32_t s_range[2];
     const uint64_t block_c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll);
-    if (threadIdx.x < 2) {
-        // tensors holding the first and the last unit this block touches
-        uint64_t c = threadIdx.x == 0 ? block_c0 : block_c0 + kThreads * kUnroll - 1;
-        if (c >= a.nchunks) c = a.nchunks - 1;
-        uint64_t tb = c * VU + (threadIdx.x == 0 ? 0 : VU - 1);
-        uint64_t unit = tb >= a.shift ? tb - a.shift : 0;
-        if (unit >= a.total) unit = a.total - 1;
-        s_range[threadIdx.x] = find_tensor(a.offsets, a.units_per_elem, 0, a.ntensors, unit);
+    if (threadIdx.x < 64) {
+        // wavefront 0 finds the tensors holding the first and the last unit this block touches
+        uint64_t c_last = block_c0 + kThreads * kUnroll - 1;
+        if (c_last >= a.nchunks) c_last = a.nchunks - 1;
+        const uint64_t tb_first = block_c0 * VU, tb_last = c_last * VU + VU - 1;
+        uint64_t u_first = tb_first >= a.shift ? tb_first - a.shift : 0;
+        uint64_t u_last = tb_last >= a.shift ? tb_last - a.shift : 0;
+        if (u_first >= a.total) u_first = a.total - 1;
+        if (u_last >= a.total) u_last = a.total - 1;
+        const uint32_t lo = wave_find_tensor(a.offsets, a.units_per_elem, 0, a.ntensors, u_first);
+        const uint32_t hi = wave_find_tensor(a.offsets, a.units_per_elem, lo, a.ntensors, u_last);
+        if (threadIdx.x == 0) {
+            s_range[0] = lo;
+            s_range[1] = hi;
+        }
     }
     __syncthreads();
     const uint32_t t_lo = s_range[0], t_hi = s_range[1] + 1;

@@ -70,6 +70,34 @@ class FlatBucket:
         self._last_unpack = (ptrs, list(outs))
 
 
+def quantize_bucket(bucket: FlatBucket, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None):
+    """Same codes and scales as ``quantize(bucket.pack())`` without the flat bf16 buffer."""
+    if bucket.dtype != torch.bfloat16:
+        raise ValueError("quantize_bucket expects a bf16 bucket")
+    n = bucket.total
+    if q is None:
+        q = torch.empty(n, dtype=torch.uint8, device=bucket.device)
+    if scales is None:
+        scales = torch.empty((n + BLOCK - 1) // BLOCK, dtype=torch.float32, device=bucket.device)
+    check(lib().mhip_fp8_quantize_bucket(q.data_ptr(), scales.data_ptr(), bucket.d_ptrs.data_ptr(),
+                                         bucket.d_offsets.data_ptr(), len(bucket.sizes), n, BLOCK,
+                                         _torch.stream_handle(stream)))
+    return q, scales
+
+
+def dequant_accumulate_bucket(bucket: FlatBucket, q: torch.Tensor, scales: torch.Tensor, stream=None) -> None:
+    """``tensor_t[j] += float(q[off_t + j]) * scale`` on the bucket's own fp32 tensors."""
+    if bucket.dtype != torch.float32:
+        raise ValueError("dequant_accumulate_bucket expects a bucket of fp32 accumulators")
+    for t in (q, scales):
+        _torch.require_contiguous(t)
+    if q.numel() != bucket.total or scales.numel() != (bucket.total + BLOCK - 1) // BLOCK:
+        raise ValueError("size mismatch between the bucket, q and scales")
+    check(lib().mhip_fp8_dequant_accumulate_bucket(bucket.d_ptrs.data_ptr(), q.data_ptr(), scales.data_ptr(),
+                                                   bucket.d_offsets.data_ptr(), len(bucket.sizes), bucket.total, BLOCK,
+                                                   _torch.stream_handle(stream)))
+
+
 def quantize(flat_bf16: torch.Tensor, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None):
     """Returns ``(q uint8[numel], scales f32[ceil(numel/1024)])``."""
     _torch.require_contiguous(flat_bf16)

@@ -109,6 +109,83 @@ def test_quantize_dequant_accumulate_ragged():
         assert np.array_equal(o.cpu().numpy(), w)
 
 
+def test_fused_bucket_forms_equal_two_step_pipeline():
+    # ragged sizes around block boundaries, empty tensors, odd element alignment, NaN/Inf blocks
+    g = torch.Generator().manual_seed(77)
+    sizes = [1500, 0, 1024, 7, 3, 2048, 1, 1023, 1025, 4096 + 5, 0, 9, 8 * 1024, 333]
+    tensors = []
+    for i, n in enumerate(sizes):
+        t = _c5_like(n, seed=700 + i)
+        if i == 5:
+            t[100] = float("nan"); t[1500] = float("inf")
+        tensors.append(t)
+    store = [torch.zeros(n + 6, dtype=torch.bfloat16, device=DEV) for n in sizes]
+    dev = []
+    for i, (t, st) in enumerate(zip(tensors, store)):
+        v = st[i % 4: i % 4 + t.numel()]  # 2-byte aligned only
+        v.copy_(t)
+        dev.append(v)
+    bucket = fp8.FlatBucket(dev)
+    q2, s2 = fp8.quantize(bucket.pack())
+    q1, s1 = fp8.quantize_bucket(bucket)
+    sync()
+    assert torch.equal(q1, q2) and torch.equal(s1.view(torch.int32), s2.view(torch.int32))
+    wq, ws = oracle.fp8_quantize(oracle.flat_pack([bits(t) for t in tensors], bucket.offsets), 1024)
+    nan = (wq & 0x7F) == 0x7F
+    assert np.array_equal(q1.cpu().numpy()[~nan], wq[~nan]) and np.array_equal(s1.cpu().numpy(), ws)
+    # receive side: accumulate twice into per-tensor fp32 buffers vs flat accumulate + unpack
+    rng = np.random.default_rng(3)
+    acc_h = rng.normal(size=bucket.total).astype(np.float32)
+    outs_store = [torch.zeros(n + 3, dtype=torch.float32, device=DEV) for n in sizes]
+    outs = [st[i % 3: i % 3 + n] for i, (st, n) in enumerate(zip(outs_store, sizes))]
+    offs = bucket.offsets
+    for o, lo, hi in zip(outs, offs[:-1], offs[1:]):
+        o.copy_(torch.from_numpy(acc_h[lo:hi]))
+    abucket = fp8.FlatBucket(outs)
+    qf = q1.clone()
+    qf[(qf & 0x7F) == 0x7F] = 0x11  # keep the comparison free of NaN
+    wq2 = qf.cpu().numpy()
+    for _ in range(2):
+        fp8.dequant_accumulate_bucket(abucket, qf, s1)
+        oracle.fp8_dequant_accumulate(acc_h, wq2, ws, 1024)
+    sync()
+    want = oracle.flat_unpack(acc_h, offs)
+    for o, w, st, i, n in zip(outs, want, outs_store, range(len(sizes)), sizes):
+        assert np.array_equal(o.cpu().numpy().view(np.uint32), w.view(np.uint32))
+        assert st[: i % 3].abs().sum() == 0 and st[i % 3 + n:].abs().sum() == 0  # neighbours untouched
+
+
+@pytest.mark.parametrize("ntensors", [1, 2, 64, 65, 66, 67, 130, 4225, 4226, 9000])
+def test_many_small_tensors_table_search(ntensors):
+    # exercises the cooperative table search at its range boundaries (65-ary steps) with empty tensors mixed in
+    g = torch.Generator().manual_seed(ntensors)
+    sizes = torch.randint(0, 4, (ntensors,), generator=g).tolist()
+    sizes[ntensors // 2] = 3000
+    if sum(sizes) == 0:
+        sizes[0] = 5
+    total = sum(sizes)
+    big = _c5_like(total, seed=ntensors)
+    offs = np.concatenate([[0], np.cumsum(sizes)]).tolist()
+    dbig = big.to(DEV)
+    dev = [dbig[offs[i]: offs[i + 1]].clone() if sizes[i] else dbig[:0] for i in range(ntensors)]
+    bucket = fp8.FlatBucket(dev)
+    flat = bucket.pack()
+    sync()
+    assert torch.equal(flat.view(torch.int16), dbig.view(torch.int16))
+    q1, s1 = fp8.quantize_bucket(bucket)
+    q2, s2 = fp8.quantize(flat)
+    sync()
+    assert torch.equal(q1, q2) and torch.equal(s1, s2)
+    accs = [torch.zeros(n, dtype=torch.float32, device=DEV) for n in sizes]
+    fp8.dequant_accumulate_bucket(fp8.FlatBucket(accs), q1, s1)
+    acc = torch.zeros(total, dtype=torch.float32, device=DEV)
+    fp8.dequant_accumulate(acc, q1, s1)
+    outs = [torch.empty(n, dtype=torch.float32, device=DEV) for n in sizes]
+    bucket.unpack(acc, outs)
+    sync()
+    assert torch.equal(torch.cat(accs), acc) and torch.equal(torch.cat(outs), acc)
+
+
 def test_flat_pack_alignment_and_empty_tensors():
     g = torch.Generator().manual_seed(3)
     for dtype, sizes in ((torch.uint8, [3, 0, 17, 1, 4096, 0, 5]), (torch.bfloat16, [1, 3, 0, 8, 1025, 7]),
@@ -179,3 +256,13 @@ def test_config5_full_size_properties():
     for i in (0, 1, 749, 1498, 1499):
         assert torch.equal(outs[i], acc[offs[i]: offs[i + 1]])
     assert torch.equal(torch.cat(outs), acc)
+    # fused forms give the same bits as the staged pipeline at full size
+    qb, sb = fp8.quantize_bucket(bucket)
+    sync()
+    assert torch.equal(qb, q) and torch.equal(sb, s)
+    accs = [torch.zeros(n, dtype=torch.float32, device=DEV) for n in sizes]
+    ab = fp8.FlatBucket(accs)
+    fp8.dequant_accumulate_bucket(ab, q, s)
+    fp8.dequant_accumulate_bucket(ab, q, s)
+    sync()
+    assert torch.equal(torch.cat(accs), acc)
