@@ -85,6 +85,51 @@ class Events:
 # workloads: each returns (name, algorithmic_bytes_per_step, launch(i), cpu_baseline(), kernel_name)
 # ---------------------------------------------------------------------------
 
+def wl_c1(torch, stage="pack"):
+    """Config 1, the reference's CPU-runnable shape: launch-latency-bound on a GPU (reported, not a target)."""
+    import numpy as np
+    from monarch_amd import Slice, _lib, staging
+    from monarch_amd._lib import ptr_array
+    s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
+    xs = [torch.from_numpy(np.random.default_rng(1000 + k).uniform(-1, 1, size=(4, 256, 256)).astype(np.float32)).to("cuda:0")
+          for k in range(8)]
+    chunks = [staging.pack(x, s) for x in xs]
+    out = torch.empty_like(chunks[0])
+    back = torch.zeros_like(xs[0])
+    n = chunks[0].numel()
+    if stage == "pack":
+        nbytes, kern = 2 * n * 4, "slice_copy_kernel<16>"
+        launch = prepared("mhip_slice_pack", chunks[0].data_ptr(), xs[0].data_ptr(), C.byref(s.c), 4, STREAM())
+    elif stage == "unpack":
+        nbytes, kern = 2 * n * 4, "slice_copy_kernel<16>"
+        launch = prepared("mhip_slice_unpack", back.data_ptr(), chunks[0].data_ptr(), C.byref(s.c), 4, STREAM())
+    else:
+        nbytes, kern = 9 * n * 4, "reduce_kernel<f32,8,sum>"
+        launch = prepared("mhip_reduce", out.data_ptr(), ptr_array([c.data_ptr() for c in chunks]), 8, n, _lib.DTYPE_F32,
+                          _lib.OP_SUM, STREAM())
+    launch.keep = (xs, chunks, out, back, s)
+
+    def cpu():
+        import oracle
+        os_ = oracle.OSlice(s.offset, s.sizes, s.strides)
+        hx = xs[0].cpu().numpy().reshape(-1)
+        hc = [c.cpu().numpy() for c in chunks]
+        reps, t0 = 0, time.perf_counter()
+        while reps < 20 or time.perf_counter() - t0 < 2.0:
+            if stage == "pack":
+                oracle.pack(hx, os_)
+            elif stage == "unpack":
+                oracle.unpack(hx, hc[0], os_)
+            else:
+                oracle.reduce(hc, oracle.SUM)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"full workload, {reps} passes of the oracle"}
+
+    return f"c1_f32_every_other_row_{stage}", nbytes, launch, cpu, kern, "f32" if stage == "reduce" else "u8"
+
+
 def wl_c2(torch, in_place=False, sets=3):
     from monarch_amd import _lib
     from monarch_amd import reduce as R
@@ -345,6 +390,9 @@ def wl_c5(torch, stage="quantize"):
 
 
 WORKLOADS = {
+    "c1_pack": lambda t: wl_c1(t, "pack"),
+    "c1_unpack": lambda t: wl_c1(t, "unpack"),
+    "c1_reduce": lambda t: wl_c1(t, "reduce"),
     "c2": lambda t: wl_c2(t, False),
     "c2_inplace": lambda t: wl_c2(t, True),
     "c2p_pack": lambda t: wl_c2p(t, False),

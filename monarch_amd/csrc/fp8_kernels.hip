@@ -104,24 +104,20 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float*
                                                                           uint64_t numel, uint64_t ntiles) {
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const uint64_t b0 = tile * kDeqSteps;
+        const uint64_t i0 = b0 * kBlock + threadIdx.x * 4;
         uint32_t codes[kDeqSteps];
         uint4 a[kDeqSteps];
         float s[kDeqSteps];
-        bool full[kDeqSteps];
+        if ((b0 + kDeqSteps) * kBlock <= numel) {
+            // interior tile (workgroup-uniform): no per-step predicates, all loads first
 #pragma unroll
-        for (int j = 0; j < kDeqSteps; ++j) {
-            const uint64_t i = (b0 + j) * kBlock + threadIdx.x * 4;
-            full[j] = i + 4 <= numel;
-            if (full[j]) {
-                codes[j] = load4_unaligned(q + i);
-                a[j] = load16_unaligned(acc + i);
+            for (int j = 0; j < kDeqSteps; ++j) {
+                codes[j] = load4_unaligned(q + i0 + j * kBlock);
+                a[j] = load16_unaligned(acc + i0 + j * kBlock);
                 s[j] = scales[b0 + j];
             }
-        }
 #pragma unroll
-        for (int j = 0; j < kDeqSteps; ++j) {
-            const uint64_t i = (b0 + j) * kBlock + threadIdx.x * 4;
-            if (full[j]) {
+            for (int j = 0; j < kDeqSteps; ++j) {
                 const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], false);
                 const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], true);
                 // product rounded to fp32, then added: two roundings (contraction is off)
@@ -130,6 +126,24 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float*
                 r.y = __float_as_uint(__uint_as_float(a[j].y) + p01[1] * s[j]);
                 r.z = __float_as_uint(__uint_as_float(a[j].z) + p23[0] * s[j]);
                 r.w = __float_as_uint(__uint_as_float(a[j].w) + p23[1] * s[j]);
+                store16_unaligned(acc + i0 + j * kBlock, r);
+            }
+            continue;
+        }
+        // last tile: per-step bounds, single elements at the ragged end
+        for (int j = 0; j < kDeqSteps; ++j) {
+            const uint64_t i = i0 + (uint64_t)j * kBlock;
+            if (i + 4 <= numel) {
+                const uint32_t c = load4_unaligned(q + i);
+                const uint4 v = load16_unaligned(acc + i);
+                const float sc = scales[b0 + j];
+                const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, false);
+                const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, true);
+                uint4 r;
+                r.x = __float_as_uint(__uint_as_float(v.x) + p01[0] * sc);
+                r.y = __float_as_uint(__uint_as_float(v.y) + p01[1] * sc);
+                r.z = __float_as_uint(__uint_as_float(v.z) + p23[0] * sc);
+                r.w = __float_as_uint(__uint_as_float(v.w) + p23[1] * sc);
                 store16_unaligned(acc + i, r);
             } else {
                 for (uint64_t e = i; e < numel && e < i + 4; ++e) {
