@@ -265,6 +265,24 @@ int mhip_memcpy_htod(void* dst, const void* src, size_t bytes, mhip_stream_t str
 int mhip_memcpy_dtoh(void* dst, const void* src, size_t bytes, mhip_stream_t stream);
 int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream);
 
+
+/* ====================================================================== */
+/* Staging-buffer lifecycle (GPU memory an RdmaBuffer can register)         */
+/* ====================================================================== */
+/* The VMM recipe of monarch_rdma/src/test_utils.rs:370-444 (cuMemCreate / cuMemAddressReserve /
+ * cuMemMap / cuMemSetAccess with a pinned device allocation): bytes are rounded up to the
+ * allocation granularity, *padded_bytes receives the mapped size.  This is the one place
+ * where the library allocates, and only when asked to. */
+int mhip_staging_alloc(void** ptr, size_t* padded_bytes, size_t bytes, int device);
+int mhip_staging_free(void* ptr, size_t padded_bytes);
+/* RdmaDomain::register_mr's first question (monarch_rdma/src/rdma_components.rs:370-377,
+ * cuPointerGetAttribute(MEMORY_TYPE)): is this address device memory? */
+int mhip_pointer_is_device(const void* ptr, int* is_device);
+/* register_mr's second step (rdma_components.rs:386-394, cuMemGetHandleForAddressRange with
+ * DMA_BUF_FD): a dma-buf file descriptor for [ptr, ptr+bytes), to hand to ibv_reg_dmabuf_mr.
+ * The caller closes the descriptor. */
+int mhip_export_dmabuf(int* fd, const void* ptr, size_t bytes);
+
 #ifdef __cplusplus
 }
 #endif

@@ -87,4 +87,84 @@ int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream) {
     return (int)hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream));
 }
 
+// ---- staging-buffer lifecycle -------------------------------------------------------
+// The recipe of the reference's RDMA test environment (monarch_rdma/src/test_utils.rs:370-444)
+// and of RdmaDomain::register_mr (monarch_rdma/src/rdma_components.rs:364-419) on the HIP
+// virtual-memory API: a physical allocation pinned on the device, mapped at a reserved
+// address with read/write access, exportable as a dma-buf for ibv_reg_dmabuf_mr.
+
+int mhip_staging_alloc(void** ptr, size_t* padded_bytes, size_t bytes, int device) {
+    if (!ptr || !padded_bytes || bytes == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    hipMemAllocationProp prop = {};
+    prop.type = hipMemAllocationTypePinned;
+    prop.location.type = hipMemLocationTypeDevice;
+    prop.location.id = device;
+    prop.requestedHandleTypes = hipMemHandleTypePosixFileDescriptor;
+    size_t granularity = 0;
+    hipError_t e = hipMemGetAllocationGranularity(&granularity, &prop, hipMemAllocationGranularityMinimum);
+    if (e != hipSuccess) return (int)e;
+    if (granularity == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    const size_t padded = ((bytes - 1) / granularity + 1) * granularity;
+    hipMemGenericAllocationHandle_t handle;
+    e = hipMemCreate(&handle, padded, &prop, 0);
+    if (e != hipSuccess) return (int)e;
+    void* va = nullptr;
+    e = hipMemAddressReserve(&va, padded, granularity, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipMemRelease(handle);
+        return (int)e;
+    }
+    e = hipMemMap(va, padded, 0, handle, 0);
+    if (e != hipSuccess) {
+        (void)hipMemAddressFree(va, padded);
+        (void)hipMemRelease(handle);
+        return (int)e;
+    }
+    // the mapping keeps the physical memory alive; the creation reference can go now
+    (void)hipMemRelease(handle);
+    hipMemAccessDesc access = {};
+    access.location.type = hipMemLocationTypeDevice;
+    access.location.id = device;
+    access.flags = hipMemAccessFlagsProtReadWrite;
+    e = hipMemSetAccess(va, padded, &access, 1);
+    if (e != hipSuccess) {
+        (void)hipMemUnmap(va, padded);
+        (void)hipMemAddressFree(va, padded);
+        return (int)e;
+    }
+    *ptr = va;
+    *padded_bytes = padded;
+    return MHIP_SUCCESS;
+}
+
+int mhip_staging_free(void* ptr, size_t padded_bytes) {
+    if (!ptr || padded_bytes == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    hipError_t e = hipMemUnmap(ptr, padded_bytes);
+    if (e != hipSuccess) return (int)e;
+    return (int)hipMemAddressFree(ptr, padded_bytes);
+}
+
+int mhip_pointer_is_device(const void* ptr, int* is_device) {
+    if (!is_device) return MHIP_ERR_INVALID_ARGUMENT;
+    // register_mr's test: the attribute query succeeds only for device memory the runtime knows
+    hipPointerAttribute_t attr = {};
+    const hipError_t e = hipPointerGetAttributes(&attr, ptr);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();  // an unknown host pointer is an answer, not a sticky error
+        *is_device = 0;
+        return MHIP_SUCCESS;
+    }
+    *is_device = attr.type == hipMemoryTypeDevice ? 1 : 0;
+    return MHIP_SUCCESS;
+}
+
+int mhip_export_dmabuf(int* fd, const void* ptr, size_t bytes) {
+    if (!fd || !ptr || bytes == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    int out = -1;
+    const hipError_t e = hipMemGetHandleForAddressRange(&out, const_cast<void*>(ptr), bytes, hipMemRangeHandleTypeDmaBufFd, 0);
+    if (e != hipSuccess) return (int)e;
+    *fd = out;
+    return MHIP_SUCCESS;
+}
+
 }  // extern "C"

@@ -272,3 +272,26 @@ def test_transpose_large_square():
     staging.unpack(back, s, out)
     sync()
     assert torch.equal(back.view(torch.int16), x.view(torch.int16))
+
+
+def test_stream_send_tensor_semantics():
+    from monarch_amd.reduce import Factory
+    from monarch_amd.send_tensor import route, stream_send_tensor
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(6, 10, generator=g).to(DEV)
+    view = base.t()[1:9:2]                      # non-contiguous sender tensor, shape [4, 6]
+    world = {0: view, 1: None, 2: torch.ones(4, 6, device=DEV)}
+    f = Factory.of(view)
+    got = stream_send_tensor(world, 3, from_rank=0, to_rank=None, factory=f)    # receiver
+    sync()
+    assert got.is_contiguous() and torch.equal(got, view) and got.data_ptr() != base.data_ptr()
+    assert stream_send_tensor(world, 0, from_rank=None, to_rank=3, factory=f) is None   # pure sender
+    local = stream_send_tensor(world, 2, from_rank=2, to_rank=2, factory=f)     # defensive copy
+    sync()
+    assert torch.equal(local, world[2]) and local.data_ptr() != world[2].data_ptr()
+    zeros = stream_send_tensor(world, 3, from_rank=1, to_rank=None, factory=f)  # errored input -> zeros
+    assert torch.count_nonzero(zeros) == 0 and zeros.shape == (4, 6)
+    with pytest.raises(ValueError, match="without a to/from rank"):
+        stream_send_tensor(world, 0, None, None, f)
+    fr, to = Slice(offset=0, sizes=[2], strides=[1]), Slice(offset=2, sizes=[2], strides=[1])
+    assert route(fr, to, 3) == (1, None)

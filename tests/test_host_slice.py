@@ -289,3 +289,28 @@ def test_reduce_argument_validation_messages():
         check_reduce_args(names, sizes, (2, 6), "host", "sum", scatter=True, out_shape=(2, 4))
     assert Reduction.from_str("stack").is_stack and Reduction.from_str("avg").op == ReduceOp.Avg
     assert int(ReduceOp.Sum) == 0 and int(ReduceOp.Avg) == 4  # nccl.rs:285-292
+
+
+def test_send_tensor_routing_and_to_mesh_checks():
+    # monarch_tensor_worker/src/lib.rs:722-731: the i-th rank of from_ranks sends to the i-th of to_ranks
+    from monarch_amd.send_tensor import check_to_mesh, route
+    from_ranks = Slice(offset=0, sizes=[2, 2], strides=[4, 1])   # ranks 0, 1, 4, 5
+    to_ranks = Slice(offset=2, sizes=[2, 2], strides=[4, 1])     # ranks 2, 3, 6, 7
+    assert route(from_ranks, to_ranks, 0) == (None, 2)
+    assert route(from_ranks, to_ranks, 5) == (None, 7)
+    assert route(from_ranks, to_ranks, 6) == (4, None)
+    assert route(from_ranks, to_ranks, 8) == (None, None)
+    same = Slice(offset=0, sizes=[4], strides=[1])
+    assert route(same, same, 3) == (3, 3)                         # local: from == to
+    shifted = Slice(offset=1, sizes=[3], strides=[1])
+    assert route(Slice(offset=0, sizes=[3], strides=[1]), shifted, 1) == (0, 2)   # both sender and receiver
+    # python/monarch/common/tensor.py:417-438
+    slicing = Slice(offset=0, sizes=[2, 8], strides=[8, 1])
+    fr, bc = check_to_mesh(["host", "gpu"], slicing, ["host", "gpu"], [2, 8])
+    assert fr == slicing and bc == []
+    fr, bc = check_to_mesh(["gpu"], Slice(offset=8, sizes=[8], strides=[1]), ["replica", "gpu"], [3, 8])
+    assert fr == Slice(offset=8, sizes=[8], strides=[1]) and bc == ["replica"]
+    with pytest.raises(ValueError, match="dimension gpu of destination device_mesh has a different length"):
+        check_to_mesh(["host", "gpu"], slicing, ["host", "gpu"], [2, 4])
+    with pytest.raises(ValueError, match="destination mesh does not have dimensions"):
+        check_to_mesh(["host", "gpu"], slicing, ["gpu"], [8])
