@@ -183,6 +183,30 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     const uint32_t t_lo = s_range[0], t_hi = s_range[1] + 1;
     const uint32_t upe = a.units_per_elem;
 
+    {
+        // Workgroup-uniform fast path: the whole 32 KiB tile lies inside one tensor (most of a
+        // bucket's bytes are in tensors much larger than a tile) and inside the flat buffer.
+        const uint64_t tile_first = block_c0 * VU;
+        const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
+        if (s_range[0] == s_range[1] && tile_first >= a.shift && tile_end - a.shift <= a.total) {
+            const uint64_t first = (block_c0 + threadIdx.x) * VU - a.shift;
+            char* __restrict__ f = a.flat + first * U;
+            char* __restrict__ t = a.tensors[t_lo] + (first - a.offsets[t_lo] * upe) * U;
+            uint4 d[kUnroll];
+#pragma unroll
+            for (int i = 0; i < kUnroll; ++i) {
+                if constexpr (PACK) d[i] = load16_unaligned(t + (size_t)i * kThreads * 16);
+                else d[i] = load16_aligned(f + (size_t)i * kThreads * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < kUnroll; ++i) {
+                if constexpr (PACK) store16_aligned(f + (size_t)i * kThreads * 16, d[i]);
+                else store16_unaligned(t + (size_t)i * kThreads * 16, d[i]);
+            }
+            return;
+        }
+    }
+
     // phase 1: resolve every chunk of this lane to (tensor address, flat address)
     char* tptr[kUnroll];
     char* fptr[kUnroll];
