@@ -163,8 +163,15 @@ def wl_c2(torch, in_place=False, sets=3):
             oracle.reduce(hosts, oracle.AVG, out=out)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
+        # the same reduction through torch's CPU kernels on all host threads (a library path, for scale)
+        hts = [torch.from_numpy(h.view(np.int16)).view(torch.bfloat16) for h in hosts]
+        t1 = time.perf_counter()
+        (torch.stack(hts).float().sum(0) / n).bfloat16()
+        dt_torch = time.perf_counter() - t1
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": f"full workload, {reps} passes of the oracle's scalar fp32-accumulate loop"}
+                "sample": f"full workload, {reps} passes of the oracle's scalar fp32-accumulate loop",
+                "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                              "sample": "one pass of torch.stack(xs).float().sum(0)/8 -> bf16"}}
 
     name = "c2_bf16_bucket_reduce_avg8_inplace" if in_place else "c2_bf16_bucket_reduce_avg8"
     return name, nbytes, launch, cpu, "reduce_kernel<bf16,8,avg>", "bf16"

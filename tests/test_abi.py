@@ -103,3 +103,19 @@ def test_rust_extern_block_names_match_header():
     header = open(os.path.join(ROOT, "include", "monarch_hip.h")).read()
     for name, value in re.findall(r"MHIP_ERR_([A-Z0-9_]+) = (\d+)", header):
         assert re.search(rf"pub const {name}: i32 = {value};", text), name
+
+
+def test_product_never_touches_the_oracle_and_fails_loudly_without_the_library(monkeypatch, tmp_path):
+    import monarch_amd
+    pkg = os.path.dirname(monarch_amd.__file__)
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+    # no CPU fallback: a missing shared library is an error at the first call
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libmonarch_hip.so"))
+    import pytest
+    with pytest.raises(_lib.MonarchHipNotBuilt):
+        monarch_amd.Slice(offset=0, sizes=[2], strides=[1])
