@@ -9,6 +9,7 @@ namespace mhip {
 
 int validate_slice(const uint64_t* sizes, uint32_t nsizes, const uint64_t* strides, uint32_t nstrides);
 uint64_t slice_len(const mhip_slice_t& s);
+bool slice_fits_address_space(const mhip_slice_t& s, uint32_t elem_size);
 
 // A Slice reduced to what a copy kernel needs.  Units are `unit` bytes.  Dimensions
 // are in iteration order (outermost first); size-1 dimensions are dropped and

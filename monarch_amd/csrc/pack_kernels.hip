@@ -378,6 +378,7 @@ static int slice_copy_entry(char* base, char* const* packed, const mhip_slice_t*
         const mhip_slice_t& s = views[k];
         if (s.ndim > MHIP_MAX_DIMS || (s.ndim && (!s.sizes || !s.strides))) return MHIP_ERR_INVALID_ARGUMENT;
         if (int rc = validate_slice(s.sizes, s.ndim, s.strides, s.ndim)) return rc;
+        if (!slice_fits_address_space(s, elem_size)) return MHIP_ERR_INVALID_ARGUMENT;
         if (slice_len(s) != 0 && (!base || !packed[k])) return MHIP_ERR_UNDEFINED_TENSOR;
     }
     hipStream_t hs = static_cast<hipStream_t>(stream);

@@ -394,6 +394,7 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
     const mhip_slice_t& iv = in_view ? *in_view : dense;
     if (iv.ndim > MHIP_MAX_DIMS || (iv.ndim && (!iv.sizes || !iv.strides))) return MHIP_ERR_INVALID_ARGUMENT;
     if (int rc = validate_slice(iv.sizes, iv.ndim, iv.strides, iv.ndim)) return rc;
+    if (!slice_fits_address_space(iv, esize)) return MHIP_ERR_INVALID_ARGUMENT;
     const uint64_t reduced_len = slice_len(iv);
 
     uintptr_t in_align = 0;
@@ -407,6 +408,7 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         const mhip_slice_t& ov = out_views[k];
         if (ov.ndim > MHIP_MAX_DIMS || (ov.ndim && (!ov.sizes || !ov.strides))) return MHIP_ERR_INVALID_ARGUMENT;
         if (int rc = validate_slice(ov.sizes, ov.ndim, ov.strides, ov.ndim)) return rc;
+        if (!slice_fits_address_space(ov, esize)) return MHIP_ERR_INVALID_ARGUMENT;
         const uint64_t len = slice_len(ov);
         if (len == 0) continue;
         if (!outs[k]) return MHIP_ERR_UNDEFINED_TENSOR;

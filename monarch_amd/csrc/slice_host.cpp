@@ -26,9 +26,33 @@ int validate_slice(const uint64_t* sizes, uint32_t nsizes, const uint64_t* strid
             if (stride == pstride && size != 1 && psize != 1) return MHIP_ERR_NONUNIQUE_STRIDES;
         }
         if (space > stride) return MHIP_ERR_STRIDE_TOO_SMALL;
-        space = stride * size;
+        // The reference computes stride * size in usize (wrapping in release builds, panicking in
+        // debug builds); a product that does not fit cannot describe addressable memory, so it is
+        // refused here.
+        if (__builtin_mul_overflow(stride, size, &space)) return MHIP_ERR_INVALID_ARGUMENT;
     }
     return MHIP_SUCCESS;
+}
+
+// True when offset + sum((size-1)*stride) + 1, times elem_size, fits in 63 bits: every byte
+// address the slice can produce is then representable.
+bool slice_fits_address_space(const mhip_slice_t& s, uint32_t elem_size) {
+    uint64_t hi = s.offset;
+    for (uint32_t k = 0; k < s.ndim; ++k) {
+        if (s.sizes[k] == 0) return true;  // empty: nothing is addressed
+        uint64_t ext;
+        if (__builtin_mul_overflow(s.sizes[k] - 1, s.strides[k], &ext)) return false;
+        if (__builtin_add_overflow(hi, ext, &hi)) return false;
+    }
+    uint64_t bytes;
+    if (__builtin_add_overflow(hi, (uint64_t)1, &hi)) return false;
+    if (__builtin_mul_overflow(hi, (uint64_t)elem_size, &bytes)) return false;
+    uint64_t len = 1;
+    for (uint32_t k = 0; k < s.ndim; ++k)
+        if (__builtin_mul_overflow(len, s.sizes[k], &len)) return false;
+    uint64_t packed;
+    if (__builtin_mul_overflow(len, (uint64_t)elem_size, &packed)) return false;
+    return bytes < (1ull << 63) && packed < (1ull << 63);
 }
 
 static inline bool bad(const mhip_slice_t* s) {

@@ -119,3 +119,14 @@ def test_product_never_touches_the_oracle_and_fails_loudly_without_the_library(m
     import pytest
     with pytest.raises(_lib.MonarchHipNotBuilt):
         monarch_amd.Slice(offset=0, sizes=[2], strides=[1])
+
+
+def test_overflowing_slices_are_refused_on_the_host():
+    from monarch_amd import Slice
+    lib = _lib.lib()
+    big = 1 << 62
+    assert lib.mhip_slice_validate(0, _lib.u64_array([8, 2]), 2, _lib.u64_array([big, 1]), 2) == _lib.ERR_INVALID_ARGUMENT
+    s = Slice(offset=1 << 62, sizes=[4], strides=[1])           # valid as a Slice, not addressable at 8 bytes/element
+    assert lib.mhip_slice_pack(16, 16, C.byref(s.c), 8, None) == _lib.ERR_INVALID_ARGUMENT
+    t = Slice(offset=0, sizes=[1 << 40, 1 << 30], strides=[1 << 30, 1], _validate=False)
+    assert lib.mhip_slice_pack(16, 16, C.byref(t.c), 1, None) == _lib.ERR_INVALID_ARGUMENT
