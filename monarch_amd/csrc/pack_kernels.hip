@@ -145,6 +145,16 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     }
 }
 
+// Plain contiguous copy of 16-byte units, both sides 16-byte aligned (a contiguous view, the
+// "transfer" of a staging buffer): one chunk per lane, non-temporal load, write-through
+// store.  For a 50/50 read/write stream this shape beats the 8-deep tile above by ~5%
+// (16.6 vs 17.4 us for 48 MiB).
+__global__ __launch_bounds__(kThreads) void contiguous_copy_kernel(char* __restrict__ dst, const char* __restrict__ src,
+                                                                   uint64_t nchunks) {
+    const uint64_t c = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (c < nchunks) store16_writethrough(dst + c * 16, load16_aligned(src + c * 16));
+}
+
 // ---------------- flat bucket <-> ragged tensors ----------------
 
 struct FlatArgs {
@@ -319,6 +329,16 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         uint32_t unit = 0;
         const uint64_t mask0 = (uint64_t)(uintptr_t)base | (uint64_t)(uintptr_t)packed[k];
         if (!canonicalize(views[k], elem_size, mask0, 16, &first, &unit)) {  // empty view: nothing to move
+            ++k;
+            continue;
+        }
+        if (first.ndim == 0 && unit == 16 && (first.total + kThreads - 1) / kThreads <= 0x7fffffffull) {
+            char* strided = base + first.offset * 16;
+            char* dst = PACK ? packed[k] : strided;
+            const char* src = PACK ? strided : packed[k];
+            hipLaunchKernelGGL(contiguous_copy_kernel, dim3((uint32_t)((first.total + kThreads - 1) / kThreads)),
+                               dim3(kThreads), 0, stream, dst, src, first.total);
+            if (int rc = launch_status()) return rc;
             ++k;
             continue;
         }

@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
         }
 #pragma unroll
         for (int k = 0; k < V; ++k) acc[k] = finish(acc[k], AVG, a.scale, a.divisor);
-        store16_unaligned(static_cast<char*>(a.out) + v * 16, VT::narrow(acc));
+        store16_writethrough(static_cast<char*>(a.out) + v * 16, VT::narrow(acc));
     }
     // ragged tail: fewer than V elements, one lane each
     if (blockIdx.x == 0) {
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
             }
 #pragma unroll
             for (int e = 0; e < V; ++e) acc[e] = finish(acc[e], AVG, a.scale, a.divisor);
-            store16_unaligned(static_cast<char*>(a.outs[k]) + t * 16, VT::narrow(acc));
+            store16_writethrough(static_cast<char*>(a.outs[k]) + t * 16, VT::narrow(acc));
         } else {
             acc_t acc = VT::widen1(a.in[0], loc);
             for (uint32_t g = 1; g < a.n_in; ++g) acc += VT::widen1(a.in[g], loc);
