@@ -168,9 +168,14 @@ struct FlatArgs {
     uint32_t units_per_elem;
 };
 
+// Chunks per lane: 8 when gathering tensors into the flat buffer, 2 when scattering the flat
+// buffer back (measured: unpack 5.74 vs 5.28 TB/s, pack 5.65 vs 5.50 TB/s the other way round).
+template <bool PACK> struct FlatUnroll { static constexpr int value = PACK ? 8 : 2; };
+
 template <int U, bool PACK>
 __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     constexpr int VU = 16 / U;
+    constexpr int kUnroll = FlatUnroll<PACK>::value;
     __shared__ uint32_t s_range[2];
     const uint64_t block_c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll);
     if (threadIdx.x < 64) {
@@ -426,7 +431,7 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
     a.shift = (uint32_t)(((uintptr_t)flat & 15u) / unit);
     const uint32_t vu = 16 / unit;
     a.nchunks = (a.total + a.shift + vu - 1) / vu;
-    const uint64_t per_block = (uint64_t)kThreads * kUnroll;
+    const uint64_t per_block = (uint64_t)kThreads * FlatUnroll<PACK>::value;
     const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
     if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
     hipStream_t hs = static_cast<hipStream_t>(stream);
