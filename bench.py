@@ -163,6 +163,12 @@ def wl_c2(torch, in_place=False, sets=3):
             oracle.reduce(hosts, oracle.AVG, out=out)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
+        # the same loop spread over every host core
+        oracle.reduce(hosts, oracle.AVG, out=out, threads=True)
+        t1 = time.perf_counter()
+        for _ in range(3):
+            oracle.reduce(hosts, oracle.AVG, out=out, threads=True)
+        dt_mt = (time.perf_counter() - t1) / 3
         # the same reduction through torch's CPU kernels on all host threads (a library path, for scale)
         hts = [torch.from_numpy(h.view(np.int16)).view(torch.bfloat16) for h in hosts]
         t1 = time.perf_counter()
@@ -170,6 +176,8 @@ def wl_c2(torch, in_place=False, sets=3):
         dt_torch = time.perf_counter() - t1
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": f"full workload, {reps} passes of the oracle's scalar fp32-accumulate loop",
+                "all_cores": {"value": nbytes / dt_mt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                              "sample": "3 passes of the same loop under OpenMP"},
                 "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                               "sample": "one pass of torch.stack(xs).float().sum(0)/8 -> bf16"}}
 
@@ -204,8 +212,15 @@ def wl_c2p(torch, unpack=False, sets=6):
         t0 = time.perf_counter()
         oracle.pack(h, os_)
         dt = time.perf_counter() - t0
+        oracle.pack(h, os_, threads=True)
+        t1 = time.perf_counter()
+        for _ in range(5):
+            oracle.pack(h, os_, threads=True)
+        dt_mt = (time.perf_counter() - t1) / 5
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "full workload, 1 pass of the per-element Slice::get walk"}
+                "sample": "full workload, 1 pass of the per-element Slice::get walk",
+                "all_cores": {"value": nbytes / dt_mt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                              "sample": "5 passes of one memcpy per contiguous run (here: the whole buffer)"}}
 
     return ("c2p_contiguous_unpack" if unpack else "c2p_contiguous_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 
@@ -243,8 +258,17 @@ def wl_c3(torch, unpack=False, sets=3):
         for v in ov[:2]:
             oracle.pack(h, v)
         dt = (time.perf_counter() - t0) * 4
+        for v in ov:
+            oracle.pack(h, v, threads=True)
+        t1 = time.perf_counter()
+        for _ in range(3):
+            for v in ov:
+                oracle.pack(h, v, threads=True)
+        dt_mt = (time.perf_counter() - t1) / 3
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "2 of the 8 column blocks through the per-element Slice::get walk, scaled x4"}
+                "sample": "2 of the 8 column blocks through the per-element Slice::get walk, scaled x4",
+                "all_cores": {"value": nbytes / dt_mt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
+                              "sample": "3 passes over all 8 blocks, one memcpy per 3584-byte row, rows under OpenMP"}}
 
     return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 

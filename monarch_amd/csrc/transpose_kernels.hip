@@ -143,6 +143,181 @@ __global__ __launch_bounds__(kThreads) void slice_transpose_kernel(TransArgs a) 
     }
 }
 
+// ---- 16-byte-per-lane variant for elements of 1, 2, 4 and 8 bytes ----
+// A tile is TQ x TC elements with TQ * sizeof(T) == TC * sizeof(T) == 256 bytes, so that every
+// row of the tile is a 256-byte run on BOTH HBM sides and every lane moves 16 bytes
+// (E = 16 / sizeof(T) elements) per global access.  The tile sits in LDS as [q][c] with the
+// 16-byte groups of a row permuted by XOR with (q / E) % 16:
+//   * the side whose vectors run along c moves whole groups (ds_read/write_b128); the 16 lanes
+//     that share a row cover its 16 groups, i.e. all banks, whatever the permutation;
+//   * the side whose vectors run along q gathers / scatters E scalars per lane.  The 16 lanes
+//     that share a column c touch rows q = E*qv + j, whose groups are displaced by qv: 16
+//     different displacements, so together with the 4 neighbouring columns of a wavefront the
+//     64 lanes fall into 64 different banks (4-byte elements; narrower ones share words in
+//     pairs, which is a broadcast, not a conflict).
+// Tiles are handed to workgroups so that each XCD (workgroup index mod 8) owns a contiguous
+// range of the blocked walk: tiles whose 256-byte rows share a cache line when rows are not
+// 256-byte aligned are then combined in one L2 instead of being written as partial lines from
+// eight of them.
+template <typename T, int THREADS, bool PACK>
+__global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs a) {
+    constexpr int E = 16 / sizeof(T);
+    constexpr int TQ = 256 / sizeof(T), TC = TQ;
+    constexpr int G = TC / E;  // 16 groups of 16 bytes per LDS row
+    static_assert(G == 16, "a tile row is 256 bytes");
+    __shared__ __attribute__((aligned(16))) T tile[TQ * TC];
+    __shared__ uint64_t s_off[TQ];
+    union Vec {
+        u32x4 v;
+        T e[E];
+    };
+    // LDS position of element (q, c)
+    auto at = [](int q, int c) { return q * TC + (c ^ (E * ((q / E) % G))); };
+
+    T* __restrict__ mem = reinterpret_cast<T*>(a.base) + a.offset;
+    T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
+    const uint64_t per_batch = (uint64_t)a.cgroups * ((a.qtiles + a.group - 1) / a.group) * a.group * a.group;
+
+    // XCD-contiguous tile ranges: workgroup w runs on XCD w % 8
+    const uint64_t per_xcd = (a.ntiles + 7) / 8;
+    const uint64_t tile_id = (uint64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile_id >= a.ntiles) return;
+
+    const uint64_t b = tile_id / per_batch;
+    const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
+    const uint32_t gsz = a.group * a.group;
+    const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
+    const uint32_t gq = grp / a.cgroups, gc = grp - gq * a.cgroups;
+    const uint32_t qt = gq * a.group + within / a.group, ct = gc * a.group + within % a.group;
+    if (qt >= a.qtiles || ct >= a.ctiles) return;  // padding of the blocked walk (uniform per workgroup)
+    // A tile that would hang over the edge is moved back inside when the extent allows it: it
+    // then overlaps its neighbour, and both write the same bytes to the overlap.
+    uint32_t q0 = qt * TQ, c0 = ct * TC;
+    if (q0 + TQ > a.Q && a.Q >= (uint32_t)TQ) q0 = a.Q - TQ;
+    if (c0 + TC > a.Sc && a.Sc >= (uint32_t)TC) c0 = a.Sc - TC;
+    uint64_t batch_off = 0;
+    {
+        uint64_t rem = b;
+        for (int k = a.n_outer - 1; k >= 0; --k) {
+            const uint64_t qd = rem / a.outer_size[k];
+            batch_off += (rem - qd * a.outer_size[k]) * a.outer_stride[k];
+            rem = qd;
+        }
+    }
+    if (threadIdx.x < TQ) {
+        uint32_t q = q0 + threadIdx.x;
+        uint64_t off = 0;
+        if (q < a.Q) {
+            for (int k = a.n_inner - 1; k > 0; --k) {
+                uint32_t qd, r;
+                a.inner_div[k].divmod(q, qd, r);
+                off += (uint64_t)r * a.inner_stride[k];
+                q = qd;
+            }
+            off += (uint64_t)q * a.inner_stride[0];
+        }
+        s_off[threadIdx.x] = off;
+    }
+    __syncthreads();
+    T* mem_tile = mem + batch_off + c0;                                        // + s_off[q] + c
+    T* packed_tile = packed + (b * a.Sc + c0) * (uint64_t)a.Q + q0;            // + c * Q + q
+    const bool full = q0 + TQ <= a.Q && c0 + TC <= a.Sc;
+    const int v16 = threadIdx.x % 16;  // which 16-byte vector of a 256-byte row
+    const int r16 = threadIdx.x / 16;  // which row of a pass of ROWS rows
+    constexpr int ROWS = THREADS / 16;
+    if (full) {
+        constexpr int PASSES = TQ / ROWS;
+        Vec d[PASSES];
+        if constexpr (PACK) {
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int q = r16 + ROWS * p;
+                d[p].v = *reinterpret_cast<const u32x4_unaligned*>(mem_tile + s_off[q] + v16 * E);
+            }
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int q = r16 + ROWS * p;
+                *reinterpret_cast<u32x4*>(&tile[at(q, v16 * E)]) = d[p].v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int cc = r16 + ROWS * p;
+                Vec o;
+#pragma unroll
+                for (int j = 0; j < E; ++j) o.e[j] = tile[at(v16 * E + j, cc)];
+                *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E) = o.v;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int cc = r16 + ROWS * p;
+                d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E);
+            }
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int cc = r16 + ROWS * p;
+#pragma unroll
+                for (int j = 0; j < E; ++j) tile[at(v16 * E + j, cc)] = d[p].e[j];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int q = r16 + ROWS * p;
+                const u32x4 o = *reinterpret_cast<const u32x4*>(&tile[at(q, v16 * E)]);
+                *reinterpret_cast<u32x4_unaligned*>(mem_tile + s_off[q] + v16 * E) = o;
+            }
+        }
+        return;
+    }
+    // Narrow extent (fewer than a tile's worth of q or of c): element by element through the same
+    // LDS layout.  Loads are unconditional, from a clamped address, so that a batch of them is
+    // in flight at once; only the stores are predicated.
+    constexpr int BATCH = TQ * TC / THREADS < 8 ? TQ * TC / THREADS : 8;
+    static_assert((TQ * TC) % (THREADS * BATCH) == 0, "whole batches");
+    if constexpr (PACK) {
+        for (int i0 = threadIdx.x; i0 < TQ * TC; i0 += THREADS * BATCH) {
+            T v[BATCH];
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int i = i0 + k * THREADS, q = i / TC, c = i % TC;
+                const bool ok = q0 + q < a.Q && c0 + c < a.Sc;
+                v[k] = mem_tile[ok ? s_off[q] + c : s_off[0]];
+            }
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int i = i0 + k * THREADS;
+                tile[at(i / TC, i % TC)] = v[k];
+            }
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < TQ * TC; i += THREADS) {
+            const int c = i / TQ, q = i % TQ;
+            if (q0 + q < a.Q && c0 + c < a.Sc) packed_tile[(uint64_t)c * a.Q + q] = tile[at(q, c)];
+        }
+    } else {
+        for (int i0 = threadIdx.x; i0 < TQ * TC; i0 += THREADS * BATCH) {
+            T v[BATCH];
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int i = i0 + k * THREADS, c = i / TQ, q = i % TQ;
+                const bool ok = q0 + q < a.Q && c0 + c < a.Sc;
+                v[k] = packed_tile[ok ? (uint64_t)c * a.Q + q : 0];
+            }
+#pragma unroll
+            for (int k = 0; k < BATCH; ++k) {
+                const int i = i0 + k * THREADS;
+                tile[at(i % TQ, i / TQ)] = v[k];
+            }
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < TQ * TC; i += THREADS) {
+            const int q = i / TC, c = i % TC;
+            if (q0 + q < a.Q && c0 + c < a.Sc) mem_tile[s_off[q] + c] = tile[at(q, c)];
+        }
+    }
+}
+
 template <bool PACK>
 bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t unit, hipStream_t stream, int* rc) {
     if (c.run != 1 || c.ndim < 2 || c.ndim > kMaxCanonDims) return false;
@@ -172,7 +347,8 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     const uint64_t Sc = c.dims[cd].size;
     // worth it only when both sides have something to coalesce
     if (Sc < 8 || Q < 8 || Sc >= kFastDivLimit) return false;
-    const uint32_t tile = unit >= 8 ? 32 : 64;
+    const bool vec = unit <= 8;  // 16-byte elements already move 16 bytes per lane in the scalar kernel
+    const uint32_t tile = vec ? 256 / unit : 32;
     a.base = base;
     a.packed = packed;
     a.offset = c.offset;
@@ -180,19 +356,31 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     a.Q = (uint32_t)Q;
     a.ctiles = (uint32_t)((Sc + tile - 1) / tile);
     a.qtiles = (uint32_t)((Q + tile - 1) / tile);
-    a.group = 4;  // 4 x 4 tiles per block of the walk: +7% over a plain row-major walk at 8192^2 fp32
+    // Tiles are walked in group x group blocks, and a block is about what one XCD runs at a time
+    // (8 workgroups per CU of 4-byte tiles, 4 of 2-byte tiles), so that the eight XCDs each stream
+    // runs of group * 256 bytes on both sides.  Measured at 8192^2 fp32 pack: group 1 0.47, 4 0.52,
+    // 16 0.65 of peak; 2-byte elements do best at 8.
+    a.group = (unit == 4 || unit == 8) ? 16 : vec ? 8 : 4;
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
     const uint64_t qgroups = (a.qtiles + a.group - 1) / a.group;
     a.ntiles = nbatch * a.cgroups * qgroups * a.group * a.group;
     const uint64_t cap = 0x7fffffffull;
-    const dim3 grid((uint32_t)(a.ntiles < cap ? a.ntiles : cap)), block(kThreads);
-    switch (unit) {
-        case 1: hipLaunchKernelGGL((slice_transpose_kernel<uint8_t, 64, PACK>), grid, block, 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((slice_transpose_kernel<uint16_t, 64, PACK>), grid, block, 0, stream, a); break;
-        case 4: hipLaunchKernelGGL((slice_transpose_kernel<uint32_t, 64, PACK>), grid, block, 0, stream, a); break;
-        case 8: hipLaunchKernelGGL((slice_transpose_kernel<uint64_t, 32, PACK>), grid, block, 0, stream, a); break;
-        case 16: hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), grid, block, 0, stream, a); break;
-        default: return false;
+    const dim3 block(kThreads);
+    if (vec) {
+        const uint64_t nblocks = 8 * ((a.ntiles + 7) / 8);  // one tile per workgroup, eight XCD ranges
+        if (nblocks > cap) return false;
+        const dim3 grid((uint32_t)nblocks);
+        switch (unit) {
+            case 1: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+            case 8: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+            default: return false;
+        }
+    } else {
+        const dim3 grid((uint32_t)(a.ntiles < cap ? a.ntiles : cap));
+        if (unit != 16) return false;
+        hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), grid, block, 0, stream, a);
     }
     *rc = launch_status();
     return true;

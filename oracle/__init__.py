@@ -196,11 +196,12 @@ def _ptr(a: np.ndarray):
     return a.ctypes.data_as(C.c_void_p)
 
 
-def pack(src_base: np.ndarray, s: OSlice, runs: bool = False) -> np.ndarray:
-    """dst[i] = src_base.flat[s.get(i)]; ``src_base`` is the flat storage."""
+def pack(src_base: np.ndarray, s: OSlice, runs: bool = False, threads: bool = False) -> np.ndarray:
+    """dst[i] = src_base.flat[s.get(i)]; ``src_base`` is the flat storage.  ``runs`` copies one
+    contiguous run per memcpy; ``threads`` also spreads the runs over every host core."""
     src_base = np.ascontiguousarray(src_base).reshape(-1)
     dst = np.empty(len(s), dtype=src_base.dtype)
-    fn = lib().o_pack_runs if runs else lib().o_slice_pack
+    fn = lib().o_pack_runs_mt if threads else lib().o_pack_runs if runs else lib().o_slice_pack
     fn(_ptr(dst), _ptr(src_base), C.byref(s.c), C.c_uint32(src_base.itemsize))
     return dst
 
@@ -217,9 +218,16 @@ _REDUCE = {"float32": "o_reduce_f32", "float64": "o_reduce_f64", "uint16": "o_re
 SUM, AVG = 0, 4
 
 
-def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = None, half: bool = False) -> np.ndarray:
+def num_threads() -> int:
+    """Host threads the ``threads=True`` variants use."""
+    return int(lib().o_num_threads())
+
+
+def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = None, half: bool = False,
+           threads: bool = False) -> np.ndarray:
     """Elementwise Sum/Avg over ``ins``.  bf16 data is passed as uint16 bit patterns
-    (``half=True``: the uint16 patterns are IEEE binary16 instead)."""
+    (``half=True``: the uint16 patterns are IEEE binary16 instead).  ``threads`` runs the same
+    loop on every host core (fp32 and bf16 only)."""
     ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
     dt = ins[0].dtype
     if half:
@@ -233,6 +241,9 @@ def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = No
         out = np.empty_like(ins[0])
     ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
     name = _REDUCE[dt.name]
+    if threads:
+        assert dt.name in ("float32", "uint16")
+        name += "_mt"
     args = [_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint64(ins[0].size)]
     if dt.name in ("float32", "float64", "uint16"):
         args.append(C.c_int(op))

@@ -23,6 +23,9 @@
  *     refused, torch-sys-cuda/src/nccl.rs:474-476): PARITY UNPINNED in the reference; the encode/decode
  *     tables are pinned against the OCP format via torch's CPU cast over all 65536 bf16 patterns.
  */
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <math.h>
 #include <float.h>
 #include <stdint.h>
@@ -641,4 +644,54 @@ void o_pack_runs(void* dst, const void* src_base, const o_slice_t* s, uint32_t e
         memcpy((char*)dst + i * elem_size, (const char*)src_base + loc * elem_size,
                run * elem_size);
     }
+}
+
+/* ---- the same two loops on every host core (OpenMP): the "fair" CPU figures that
+ * bench.py reports beside the single-thread restatement, so that the GPU is not only
+ * compared with a scalar loop.  Results are identical to the single-thread functions:
+ * rows (pack) and elements (reduce) are independent. */
+void o_pack_runs_mt(void* dst, const void* src_base, const o_slice_t* s, uint32_t elem_size) {
+    if (s->ndim == 0 || s->strides[s->ndim - 1] != 1) {
+        o_slice_pack(dst, src_base, s, elem_size);
+        return;
+    }
+    const uint64_t run = s->sizes[s->ndim - 1];
+    const uint64_t len = o_slice_len(s);
+    if (run == 0 || len == 0) return;
+    const int64_t rows = (int64_t)(len / run);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < rows; r++) {
+        uint64_t loc;
+        o_slice_get(s, (uint64_t)r * run, &loc);
+        memcpy((char*)dst + (uint64_t)r * run * elem_size, (const char*)src_base + loc * elem_size,
+               run * elem_size);
+    }
+}
+
+void o_reduce_bf16_mt(uint16_t* out, const uint16_t* const* in, uint32_t n, uint64_t numel, int op) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)numel; i++) {
+        float acc = bf16_to_f32(in[0][i]);
+        for (uint32_t r = 1; r < n; r++) acc += bf16_to_f32(in[r][i]);
+        if (op == 4) acc = acc / (float)n;
+        out[i] = f32_to_bf16_rne(acc);
+    }
+}
+
+void o_reduce_f32_mt(float* out, const float* const* in, uint32_t n, uint64_t numel, int op) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)numel; i++) {
+        float acc = in[0][i];
+        for (uint32_t r = 1; r < n; r++) acc += in[r][i];
+        if (op == 4) acc = acc / (float)n;
+        out[i] = acc;
+    }
+}
+
+int o_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
 }

@@ -261,6 +261,31 @@ def test_transposing_views_lds_path(dtype):
             assert np.array_equal(out.cpu().numpy(), oracle.pack(hb, oslice(s)))
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+def test_transposing_views_interior_and_edge_tiles(dtype):
+    # large enough for whole 256-byte x 256-byte tiles at every element size, with rows that are
+    # not 16-byte aligned (odd pitch, odd offset), ragged edges on both sides, and a packed-side
+    # index that spans two iteration dimensions
+    g = torch.Generator().manual_seed(13)
+    info = torch.iinfo(dtype)
+    for shape, view_of in [((523, 777), lambda t: t[3:, 5:].t()),
+                           ((4, 300, 261), lambda t: t.permute(2, 0, 1)),
+                           ((2, 270, 2, 259), lambda t: t.permute(0, 3, 2, 1)[:, 1:])]:
+        host = torch.randint(info.min, info.max, shape, dtype=dtype, generator=g)
+        dev = host.to(DEV)
+        view, hview = view_of(dev), view_of(host)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.cpu(), hview.contiguous().flatten()), (shape, dtype)
+        back = torch.full_like(dev, 7)
+        staging.unpack(back, s, out)
+        sync()
+        ref = torch.full_like(host, 7)
+        view_of(ref).copy_(hview)
+        assert torch.equal(back.cpu(), ref), (shape, dtype)
+
+
 def test_transpose_large_square():
     g = torch.Generator(device=DEV).manual_seed(12)
     x = (torch.randn(4096, 4096, generator=g, device=DEV)).bfloat16()

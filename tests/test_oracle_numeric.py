@@ -119,6 +119,7 @@ def test_reduce_f32_vs_torch(n):
         acc = acc + x
     assert np.array_equal(oracle.reduce(ins, SUM), acc)
     assert np.array_equal(oracle.reduce(ins, AVG), acc / np.float32(n))
+    assert np.array_equal(oracle.reduce(ins, AVG, threads=True), acc / np.float32(n))
     # in place on input 0
     first = ins[0].copy()
     oracle.reduce([first] + ins[1:], SUM, out=first)
@@ -143,6 +144,7 @@ def test_reduce_bf16_vs_torch(n):
         for t in ts[1:]:
             acc = acc + t.float()
         assert np.array_equal(got, bits((acc / div).bfloat16()))
+        assert np.array_equal(oracle.reduce(ins, op, threads=True), got)  # the all-cores loop is the same loop
 
 
 def test_reduce_integer_wraps():

@@ -265,6 +265,7 @@ def test_pack_unpack_against_as_strided():
             want = torch.as_strided(torch.from_numpy(base), s.sizes, s.strides, s.offset).contiguous().flatten().numpy()
             assert np.array_equal(got, want)
             assert np.array_equal(oracle.pack(base, s, runs=True), want)
+            assert np.array_equal(oracle.pack(base, s, threads=True), want)
             # unpack: round trip on the view, untouched elsewhere
             dst = np.full_like(base, 7)
             oracle.unpack(dst, got, s)
