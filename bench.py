@@ -29,10 +29,11 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_659_750, "c2_inplace": 452_659_692, "c2p_pack": 100_663_296, "c2p_unpack": 100_661_715,
-    "c3_pack": 234_810_402, "c3_unpack": 234_815_974, "c4": 603_524_872,
-    "c5_flat_pack": 3_210_331_152, "c5_quantize": 2_361_569_907, "c5_dequant": 7_100_632_520,
-    "c5_flat_unpack": 6_100_598_486, "tr_f32_pack": 536_653_207, "tr_bf16_pack": 268_365_014,
+    "c2": 452_884_129, "c2_inplace": 452_884_140, "c2p_pack": 100_663_296, "c2p_unpack": 100_663_296,
+    "c3_pack": 234_902_749, "c3_unpack": 234_904_867, "c4": 603_819_707,
+    "c5_flat_pack": 3_187_684_377, "c5_quantize": 2_362_572_636, "c5_dequant": 7_103_230_055,
+    "c5_flat_unpack": 6_017_507_751, "c5_quantize_bucket": 2_378_462_487, "c5_dequant_bucket": 7_178_455_286,
+    "tr_f32_pack": 536_838_397, "tr_f32_unpack": 536_848_703, "tr_bf16_pack": 268_470_512,
 }
 
 
@@ -222,7 +223,7 @@ def wl_c2p(torch, unpack=False, sets=6):
                 "all_cores": {"value": nbytes / dt_mt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(),
                               "sample": "5 passes of one memcpy per contiguous run (here: the whole buffer)"}}
 
-    return ("c2p_contiguous_unpack" if unpack else "c2p_contiguous_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
+    return ("c2p_contiguous_unpack" if unpack else "c2p_contiguous_pack"), nbytes, launch, cpu, "contiguous_copy_kernel", "u8"
 
 
 def wl_c3(torch, unpack=False, sets=3):
@@ -304,7 +305,7 @@ def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
                 "sample": f"{m}x{m} corner through the per-element Slice::get walk, scaled to {n}x{n}"}
 
     name = f"transpose_{dtype_name}_{n}x{n}_" + ("unpack" if unpack else "pack")
-    return name, nbytes, launch, cpu, "slice_transpose_kernel", "u8"
+    return name, nbytes, launch, cpu, "slice_transpose_vec_kernel", "u8"
 
 
 def wl_c4(torch, sets=2):

@@ -659,12 +659,17 @@ void o_pack_runs_mt(void* dst, const void* src_base, const o_slice_t* s, uint32_
     const uint64_t len = o_slice_len(s);
     if (run == 0 || len == 0) return;
     const int64_t rows = (int64_t)(len / run);
+    /* long runs are cut into 1 MiB pieces so that a slice of few rows still uses every core */
+    const uint64_t piece = (1u << 20) / elem_size ? (1u << 20) / elem_size : 1;
+    const int64_t per_row = (int64_t)((run + piece - 1) / piece);
 #pragma omp parallel for schedule(static)
-    for (int64_t r = 0; r < rows; r++) {
+    for (int64_t t = 0; t < rows * per_row; t++) {
+        const uint64_t r = (uint64_t)(t / per_row), first = (uint64_t)(t % per_row) * piece;
+        const uint64_t n = run - first < piece ? run - first : piece;
         uint64_t loc;
-        o_slice_get(s, (uint64_t)r * run, &loc);
-        memcpy((char*)dst + (uint64_t)r * run * elem_size, (const char*)src_base + loc * elem_size,
-               run * elem_size);
+        o_slice_get(s, r * run, &loc);
+        memcpy((char*)dst + (r * run + first) * elem_size,
+               (const char*)src_base + (loc + first) * elem_size, n * elem_size);
     }
 }
 
