@@ -76,8 +76,8 @@ __global__ __launch_bounds__(kThreads) void fp8_quantize_bucket_kernel(uint8_t* 
         const uint64_t span_begin = b0 * kBlock;
         const uint64_t span_end = span_begin + (uint64_t)kBucketBlocks * kBlock < a.total
                                       ? span_begin + (uint64_t)kBucketBlocks * kBlock : a.total;
-        const uint32_t t_first = wave_find_tensor(a.offsets, 1, 0, a.ntensors, span_begin);
-        const uint32_t t_last = wave_find_tensor(a.offsets, 1, t_first, a.ntensors, span_end - 1);
+        uint32_t t_first, t_last;
+        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, span_begin, span_end - 1, &t_first, &t_last);
         uint4 lo[kBucketBlocks], hi[kBucketBlocks];
         const bool one_tensor = t_first == t_last && span_end - span_begin == (uint64_t)kBucketBlocks * kBlock;
         if (one_tensor) {  // wave-uniform
@@ -142,8 +142,8 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_bucket_kernel
     for (uint64_t b = wave; b < a.nblocks; b += nwaves) {
         const uint64_t begin = b * kBlock;
         const uint64_t end = begin + kBlock < a.total ? begin + kBlock : a.total;
-        const uint32_t t_lo = wave_find_tensor(a.offsets, 1, 0, a.ntensors, begin);
-        const uint32_t t_hi = wave_find_tensor(a.offsets, 1, t_lo, a.ntensors, end - 1);
+        uint32_t t_lo, t_hi;
+        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, &t_lo, &t_hi);
         const float s = scales[b];
         if (t_lo == t_hi && end - begin == kBlock) {
             // the whole block lies in one tensor: 4 steps of 256 elements, all loads first

@@ -87,4 +87,40 @@ __device__ __forceinline__ uint32_t wave_find_tensor(const uint64_t* __restrict_
     return lo;
 }
 
+// Two positions u1 <= u2 in one descent: the probes of a step are loaded once and compared with
+// both, and the searches only part ways (rarely: the positions are a few thousand elements
+// apart) when they fall into different sub-ranges.
+__device__ __forceinline__ void wave_find_tensor_pair(const uint64_t* __restrict__ offsets, uint32_t upe, uint32_t lo,
+                                                      uint32_t hi, uint64_t u1, uint64_t u2, uint32_t* t1,
+                                                      uint32_t* t2) {
+    const uint32_t lane = threadIdx.x & 63;
+    while (hi - lo > 1) {
+        const uint32_t span = hi - lo;
+        if (span <= 65) {
+            const uint32_t pos = lo + 1 + lane;
+            const uint64_t off = pos < hi ? offsets[pos] * upe : ~0ull;
+            *t1 = lo + (uint32_t)__popcll(__ballot(pos < hi && off <= u1));
+            *t2 = lo + (uint32_t)__popcll(__ballot(pos < hi && off <= u2));
+            return;
+        }
+        const uint32_t pos = lo + (uint32_t)(((uint64_t)(lane + 1) * span) / 65);
+        const uint64_t off = offsets[pos] * upe;
+        const uint32_t c1 = (uint32_t)__popcll(__ballot(off <= u1));
+        const uint32_t c2 = (uint32_t)__popcll(__ballot(off <= u2));
+        const uint32_t lo1 = c1 ? lo + (uint32_t)(((uint64_t)c1 * span) / 65) : lo;
+        const uint32_t hi1 = c1 < 64 ? lo + (uint32_t)(((uint64_t)(c1 + 1) * span) / 65) : hi;
+        if (c1 != c2) {
+            const uint32_t lo2 = lo + (uint32_t)(((uint64_t)c2 * span) / 65);
+            const uint32_t hi2 = c2 < 64 ? lo + (uint32_t)(((uint64_t)(c2 + 1) * span) / 65) : hi;
+            *t1 = wave_find_tensor(offsets, upe, lo1, hi1, u1);
+            *t2 = wave_find_tensor(offsets, upe, lo2, hi2, u2);
+            return;
+        }
+        lo = lo1;
+        hi = hi1;
+    }
+    *t1 = lo;
+    *t2 = lo;
+}
+
 }  // namespace mhip
