@@ -131,15 +131,24 @@ def wl_c1(torch, stage="pack"):
     return f"c1_f32_every_other_row_{stage}", nbytes, launch, cpu, kern, "f32" if stage == "reduce" else "u8"
 
 
-def wl_c2(torch, in_place=False, sets=3):
-    from monarch_amd import _lib
+def wl_c2(torch, in_place=False, sets=3, separate=False):
+    """8 bf16 chunks of one gradient bucket -> their average.  By default the chunks are the slots of
+    one staging area laid out by the library (`mhip_staging_slot_pitch`); `separate` allocates them
+    as eight independent torch tensors instead (which end up a multiple of 16 KiB apart)."""
+    from monarch_amd import _lib, staging
     from monarch_amd import reduce as R
     from monarch_amd._lib import ptr_array
     n, numel = 8, 25_165_824
     g = torch.Generator(device="cuda:0").manual_seed(2000)
     bufs = []
     for _ in range(sets):  # rotate buffer sets so that no pass is served from the 256 MB Infinity Cache
-        ins = [(torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16() for _ in range(n)]
+        if separate:
+            ins = [(torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16() for _ in range(n)]
+        else:
+            area = staging.StagingArea(n, numel * 2)
+            ins = area.slots(torch.bfloat16)
+            for t in ins:
+                t.copy_((torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16())
         out = ins[0] if in_place else torch.empty_like(ins[0])
         bufs.append((ins, out))
     nbytes = (n + 1) * numel * 2
@@ -182,7 +191,7 @@ def wl_c2(torch, in_place=False, sets=3):
                 "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                               "sample": "one pass of torch.stack(xs).float().sum(0)/8 -> bf16"}}
 
-    name = "c2_bf16_bucket_reduce_avg8_inplace" if in_place else "c2_bf16_bucket_reduce_avg8"
+    name = "c2_bf16_bucket_reduce_avg8" + ("_inplace" if in_place else "") + ("_separate_allocations" if separate else "")
     return name, nbytes, launch, cpu, "reduce_kernel<bf16,8,avg>", "bf16"
 
 
@@ -308,19 +317,29 @@ def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
     return name, nbytes, launch, cpu, "slice_transpose_vec_kernel", "u8"
 
 
-def wl_c4(torch, sets=2):
-    from monarch_amd import Slice, _lib
+def wl_c4(torch, sets=2, slots=False):
+    """Mesh [2 hosts, 8 gpus] x [2048, 4096] fp32, summed over gpus, last dim scattered 8 ways.  By default
+    the 16 slabs are one dense tensor, as the configuration states it; `slots` places them in the slots of a
+    staging area instead (pitch 32 MiB + 8 KiB), which is where peers' slabs would land on a real mesh."""
+    from monarch_amd import Slice, _lib, staging
     from monarch_amd._lib import ptr_array
     from monarch_amd.ndslice import slice_array
     H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
     g = torch.Generator(device="cuda:0").manual_seed(4000)
     slab, w = Rr * Cc, Cc // K
-    in_view = Slice(offset=0, sizes=[H, Rr, Cc], strides=[G * slab, Cc, 1])
+    pitch = staging.slot_pitch(slab * 4) // 4 if slots else slab
+    in_view = Slice(offset=0, sizes=[H, Rr, Cc], strides=[G * pitch, Cc, 1])
     out_views = [Slice(offset=k * w, sizes=[H, Rr, w], strides=[Rr * Cc, Cc, 1]) for k in range(K)]
     bufs = []
     for _ in range(sets):
-        x = torch.rand(H, G, Rr, Cc, generator=g, device="cuda:0") * 2 - 1
-        group = [x.view(-1)[gi * slab:] for gi in range(G)]
+        if slots:
+            area = staging.StagingArea(H * G, slab * 4)
+            x = area.storage.view(torch.float32)
+            for t in area.slots(torch.float32):
+                t.copy_(torch.rand(slab, generator=g, device="cuda:0") * 2 - 1)
+        else:
+            x = (torch.rand(H, G, Rr, Cc, generator=g, device="cuda:0") * 2 - 1).view(-1)
+        group = [x[gi * pitch:] for gi in range(G)]
         outs = [torch.empty(H * Rr * w, device="cuda:0") for _ in range(K)]
         bufs.append((x, group, outs))
     nbytes = H * G * slab * 4 + H * slab * 4
@@ -339,12 +358,13 @@ def wl_c4(torch, sets=2):
         ov = oracle.OSlice(in_view.offset, in_view.sizes, in_view.strides)
         o0 = oracle.OSlice(out_views[0].offset, out_views[0].sizes, out_views[0].strides)
         t0 = time.perf_counter()
-        oracle.reduce_scatter([hx[gi * slab:] for gi in range(G)], ov, [o0], oracle.SUM)
+        oracle.reduce_scatter([hx[gi * pitch:] for gi in range(G)], ov, [o0], oracle.SUM)
         dt = (time.perf_counter() - t0) * K
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "1 of the 8 scatter outputs through the oracle, scaled x8"}
 
-    return "c4_mesh_dim_reduce_scatter_f32", nbytes, launch, cpu, "reduce_scatter_kernel<f32,vec>", "f32"
+    name = "c4_mesh_dim_reduce_scatter_f32" + ("_staging_slots" if slots else "")
+    return name, nbytes, launch, cpu, "reduce_scatter_kernel<f32,vec>", "f32"
 
 
 def _c5_setup(torch):
@@ -431,17 +451,29 @@ def wl_c5(torch, stage="quantize"):
     return f"c5_fp8_{stage}", nbytes, launch, cpu, kern, "bf16->f8e4m3fn"
 
 
+LAYOUT = {  # where a workload's inputs live, when that is the library's choice
+    "c2": "8 slots of one staging area, pitch mhip_staging_slot_pitch(48 MiB) = 48 MiB + 8 KiB",
+    "c2_inplace": "8 slots of one staging area, pitch 48 MiB + 8 KiB; output = slot 0",
+    "c2_separate": "8 separate torch allocations",
+    "c2_inplace_separate": "8 separate torch allocations; output = input 0",
+    "c4": "one dense [2,8,2048,4096] tensor (slab pitch 32 MiB)",
+    "c4_slots": "16 slots of one staging area, pitch 32 MiB + 8 KiB",
+}
+
 WORKLOADS = {
     "c1_pack": lambda t: wl_c1(t, "pack"),
     "c1_unpack": lambda t: wl_c1(t, "unpack"),
     "c1_reduce": lambda t: wl_c1(t, "reduce"),
     "c2": lambda t: wl_c2(t, False),
     "c2_inplace": lambda t: wl_c2(t, True),
+    "c2_separate": lambda t: wl_c2(t, False, separate=True),
+    "c2_inplace_separate": lambda t: wl_c2(t, True, separate=True),
     "c2p_pack": lambda t: wl_c2p(t, False),
     "c2p_unpack": lambda t: wl_c2p(t, True),
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
     "c4": wl_c4,
+    "c4_slots": lambda t: wl_c4(t, slots=True),
     "tr_f32_pack": lambda t: wl_transpose(t, "f32", False),
     "tr_f32_unpack": lambda t: wl_transpose(t, "f32", True),
     "tr_bf16_pack": lambda t: wl_transpose(t, "bf16", False),
@@ -478,7 +510,8 @@ def run(workload: str, steps: int, warmup: int, cpu_baseline: bool):
         "metric": METRIC, "value": nbytes / (wall_ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
         "steps": steps, "warmup": warmup, "ms_per_step": wall_ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name, "algorithmic_bytes_per_step": nbytes, "kernel": kernel},
+        "config": {"workload": name, "algorithmic_bytes_per_step": nbytes, "kernel": kernel,
+                   **({"layout": LAYOUT[workload]} if workload in LAYOUT else {})},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(workload)},
     }

@@ -132,6 +132,7 @@ extern "C" {
     pub fn mhip_memset(dst: *mut c_void, value: c_int, bytes: usize, stream: *mut c_void) -> c_int;
     pub fn mhip_staging_alloc(ptr: *mut *mut c_void, padded_bytes: *mut usize, bytes: usize, device: c_int) -> c_int;
     pub fn mhip_staging_free(ptr: *mut c_void, padded_bytes: usize) -> c_int;
+    pub fn mhip_staging_slot_pitch(slot_bytes: usize, pitch_bytes: *mut usize) -> c_int;
     pub fn mhip_pointer_is_device(ptr: *const c_void, is_device: *mut c_int) -> c_int;
     pub fn mhip_export_dmabuf(fd: *mut c_int, ptr: *const c_void, bytes: usize) -> c_int;
 }

@@ -275,6 +275,13 @@ int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream);
  * where the library allocates, and only when asked to. */
 int mhip_staging_alloc(void** ptr, size_t* padded_bytes, size_t bytes, int device);
 int mhip_staging_free(void* ptr, size_t padded_bytes);
+/* Distance in bytes between consecutive slots of one staging area whose slots are read side by
+ * side by mhip_reduce / mhip_reduce_scatter (slot r = what peer r wrote: the per-worker chunks of
+ * monarch_rdma/examples/parameter_server/parameter_server.rs:193-210).  No counterpart in the
+ * reference: it is a layout rule of this part's memory system.  Streams that start a multiple of
+ * 16 KiB apart collide in HBM; a pitch of (slot_bytes rounded up to 16 KiB) + 8 KiB keeps them
+ * apart (bf16 reduce of 8 x 48 MiB: 74.8 us at a 48 MiB pitch, 70.6 us at 48 MiB + 8 KiB). */
+int mhip_staging_slot_pitch(size_t slot_bytes, size_t* pitch_bytes);
 /* RdmaDomain::register_mr's first question (monarch_rdma/src/rdma_components.rs:370-377,
  * cuPointerGetAttribute(MEMORY_TYPE)): is this address device memory? */
 int mhip_pointer_is_device(const void* ptr, int* is_device);

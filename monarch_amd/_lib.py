@@ -139,6 +139,7 @@ SIGNATURES = {
     "mhip_memset": (C.c_int, [_vp, C.c_int, C.c_size_t, _vp]),
     "mhip_staging_alloc": (C.c_int, [_vpp, C.POINTER(C.c_size_t), C.c_size_t, C.c_int]),
     "mhip_staging_free": (C.c_int, [_vp, C.c_size_t]),
+    "mhip_staging_slot_pitch": (C.c_int, [C.c_size_t, C.POINTER(C.c_size_t)]),
     "mhip_pointer_is_device": (C.c_int, [_vp, C.POINTER(C.c_int)]),
     "mhip_export_dmabuf": (C.c_int, [C.POINTER(C.c_int), _vp, C.c_size_t]),
 }

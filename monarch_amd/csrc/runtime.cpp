@@ -1,5 +1,6 @@
 // Runtime pass-through and error text: the small part of the HIP runtime that the
 // data path's callers reach through this library instead of through cuda-sys/nccl-sys.
+#include <cstdint>
 #include <hip/hip_runtime.h>
 
 #include "mhip_internal.h"
@@ -92,6 +93,14 @@ int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream) {
 // and of RdmaDomain::register_mr (monarch_rdma/src/rdma_components.rs:364-419) on the HIP
 // virtual-memory API: a physical allocation pinned on the device, mapped at a reserved
 // address with read/write access, exportable as a dma-buf for ibv_reg_dmabuf_mr.
+
+int mhip_staging_slot_pitch(size_t slot_bytes, size_t* pitch_bytes) {
+    if (!pitch_bytes || slot_bytes == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    constexpr size_t kPeriod = 16384, kSkew = 8192;
+    if (slot_bytes > SIZE_MAX - kPeriod - kSkew) return MHIP_ERR_INVALID_ARGUMENT;
+    *pitch_bytes = (slot_bytes + kPeriod - 1) / kPeriod * kPeriod + kSkew;
+    return MHIP_SUCCESS;
+}
 
 int mhip_staging_alloc(void** ptr, size_t* padded_bytes, size_t bytes, int device) {
     if (!ptr || !padded_bytes || bytes == 0) return MHIP_ERR_INVALID_ARGUMENT;

@@ -153,3 +153,39 @@ class TensorBuffer:
     def commit(self, stream=None) -> None:
         """Scatter the staging bytes back into the view (call after ``buffer.write_from``)."""
         unpack(self.view, self.slice, self.buffer.data, stream=stream)
+
+
+def slot_pitch(slot_bytes: int) -> int:
+    """Byte distance between consecutive slots of a staging area (``mhip_staging_slot_pitch``)."""
+    pitch = C.c_size_t()
+    check(lib().mhip_staging_slot_pitch(slot_bytes, C.byref(pitch)))
+    return pitch.value
+
+
+class StagingArea:
+    """``n_slots`` equally sized staging buffers carved from one allocation: slot *r* is where
+    peer *r*'s chunk lands before the local combine, the per-worker chunks of the reference's
+    parameter server (monarch_rdma/examples/parameter_server/parameter_server.rs:193-210).
+    Slots are ``slot_pitch(slot_bytes)`` apart rather than back to back: reduce kernels read all
+    slots side by side, and streams that start a multiple of 16 KiB apart collide in HBM."""
+
+    def __init__(self, n_slots: int, slot_bytes: int, device="cuda:0") -> None:
+        if n_slots <= 0 or slot_bytes <= 0:
+            raise ValueError("a staging area needs at least one slot of at least one byte")
+        self.n_slots, self.slot_bytes = n_slots, slot_bytes
+        self.pitch = slot_pitch(slot_bytes)
+        self.storage = torch.empty((n_slots - 1) * self.pitch + slot_bytes, dtype=torch.uint8, device=device)
+        _torch.require_device(self.storage)
+
+    def slot(self, r: int, dtype: torch.dtype = torch.uint8) -> torch.Tensor:
+        """Slot ``r`` as a 1-D tensor of ``dtype`` (a view: no copy)."""
+        if not 0 <= r < self.n_slots:
+            raise IndexError(f"slot {r} of {self.n_slots}")
+        return self.storage[r * self.pitch: r * self.pitch + self.slot_bytes].view(dtype)
+
+    def slots(self, dtype: torch.dtype = torch.uint8) -> List[torch.Tensor]:
+        return [self.slot(r, dtype) for r in range(self.n_slots)]
+
+    def buffer(self, r: int) -> RDMABuffer:
+        """Slot ``r`` as the 1-D uint8 buffer an RDMA transfer targets."""
+        return RDMABuffer(self.slot(r))

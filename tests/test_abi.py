@@ -58,6 +58,13 @@ def test_status_text_and_host_only_calls():
     assert lib.mhip_slice_pack(16, 16, C.byref(bad.c), 4, None) == _lib.ERR_NONUNIQUE_STRIDES
     empty = Slice(offset=0, sizes=[0], strides=[1])
     assert lib.mhip_slice_pack(None, None, C.byref(empty.c), 4, None) == 0
+    # staging slots are never a multiple of 16 KiB apart, and always at least a slot apart
+    pitch = C.c_size_t()
+    for nbytes in (1, 8191, 8192, 16384, 16385, 50331648, 33554432, 3 * 16384 + 8192):
+        assert lib.mhip_staging_slot_pitch(nbytes, C.byref(pitch)) == 0
+        assert pitch.value >= nbytes and pitch.value % 16384 == 8192 and pitch.value - nbytes < 16384 + 8192
+    assert lib.mhip_staging_slot_pitch(0, C.byref(pitch)) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.mhip_staging_slot_pitch(2**64 - 1, C.byref(pitch)) == _lib.ERR_INVALID_ARGUMENT
 
 
 def test_fastdiv_exhaustive_on_host(tmp_path):

@@ -175,6 +175,32 @@ def test_config2_bf16_bucket_full_size():
     assert torch.equal(out.view(torch.int16), (first.float() * 8).bfloat16().view(torch.int16))
 
 
+def test_reduce_over_staging_area_slots():
+    # the chunks of peers sit in the slots of one staging area (skewed pitch); slot 0 doubles as the output
+    from monarch_amd import staging
+    n, numel = 8, 300_001
+    area = staging.StagingArea(n, numel * 2)
+    assert area.pitch % 16384 == 8192 and area.pitch >= numel * 2
+    hosts = [_rand(torch.bfloat16, numel, 700 + r) for r in range(n)]
+    area.storage.fill_(0x5a)
+    for r, h in enumerate(hosts):
+        area.slot(r, torch.bfloat16).copy_(h)
+        assert area.buffer(r).size == numel * 2
+    want = _oracle_reduce(hosts, AVG, torch.bfloat16)
+    out = torch.empty(numel, dtype=torch.bfloat16, device=DEV)
+    R.all_reduce(out, area.slots(torch.bfloat16), R.ReduceOp.Avg)
+    sync()
+    assert np.array_equal(bits(out.cpu()), want)
+    R.all_reduce(area.slot(0, torch.bfloat16), area.slots(torch.bfloat16), R.ReduceOp.Avg)   # in place on slot 0
+    sync()
+    assert np.array_equal(bits(area.slot(0, torch.bfloat16).cpu()), want)
+    # the gaps between slots are never written
+    gap = area.storage[numel * 2: area.pitch].cpu()
+    assert bool((gap == 0x5a).all())
+    with pytest.raises(IndexError):
+        area.slot(n)
+
+
 def test_config1_sum_of_8_packed_chunks():
     from monarch_amd import staging
     s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
