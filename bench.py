@@ -29,11 +29,12 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_884_129, "c2_inplace": 452_884_140, "c2p_pack": 100_663_296, "c2p_unpack": 100_663_296,
-    "c3_pack": 234_902_749, "c3_unpack": 234_904_867, "c4": 603_819_707,
-    "c5_flat_pack": 3_187_684_377, "c5_quantize": 2_362_572_636, "c5_dequant": 7_103_230_055,
-    "c5_flat_unpack": 6_017_507_751, "c5_quantize_bucket": 2_378_462_487, "c5_dequant_bucket": 7_178_455_286,
-    "tr_f32_pack": 536_838_397, "tr_f32_unpack": 536_848_703, "tr_bf16_pack": 268_470_512,
+    "c2": 452_885_315, "c2_inplace": 452_885_711, "c2_separate": 452_884_036, "c2p_pack": 100_663_296,
+    "c2p_unpack": 100_663_296, "c3_pack": 234_902_749, "c3_unpack": 234_904_867, "c4": 603_819_563,
+    "c4_slots": 603_820_299, "c5_flat_pack": 3_187_684_377, "c5_quantize": 2_362_572_636,
+    "c5_dequant": 7_103_230_055, "c5_flat_unpack": 6_017_507_751, "c5_quantize_bucket": 2_379_634_019,
+    "c5_dequant_bucket": 7_178_104_765, "tr_f32_pack": 536_838_397, "tr_f32_unpack": 536_848_703,
+    "tr_bf16_pack": 268_470_512,
 }
 
 
