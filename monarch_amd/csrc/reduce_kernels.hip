@@ -21,6 +21,7 @@ struct ReduceArgs {
     uint32_t n;
     float scale;   // 1/n when n is a power of two and op is Avg (exact), else 0
     float divisor; // n as a float
+    uint32_t xcd_contiguous;  // see inputs_alias()
 };
 
 // ---- per-type vector traits: 16 bytes <-> accumulator lanes ----
@@ -128,6 +129,28 @@ template <typename A> __device__ __forceinline__ A finish(A acc, bool avg, float
 // persistent grid-stride loop (5.99 vs 5.56 TB/s for 8 bf16 inputs of 48 MiB).
 constexpr int kReduceThreads = 128;
 
+// Workgroup i runs on XCD i mod 8, and a workgroup covers 2 KiB of every input, so with the
+// plain mapping one XCD only ever touches addresses that agree modulo 16 KiB.  That is the
+// fastest arrangement when the inputs themselves sit at different 4 KiB phases of 16 KiB (what
+// mhip_staging_slot_pitch arranges): 8 x 48 MiB bf16 at 70.6 us.  When more than half of the
+// inputs share a phase (slots packed back to back, power-of-two slabs of one tensor) it is the
+// slowest (75.6 us), and handing each XCD one contiguous eighth of the index space instead is
+// better (73.1 us; the fp32 mesh-dim reduce+scatter over 32 MiB slabs 105 -> 96 us).  The host
+// looks at the input addresses and picks the mapping per launch.
+static bool inputs_alias(const void* const* in, uint32_t n) {
+    if (n < 4) return false;
+    uint32_t count[4] = {0, 0, 0, 0};
+    for (uint32_t r = 0; r < n; ++r) ++count[((uintptr_t)in[r] >> 12) & 3u];
+    uint32_t most = 0;
+    for (uint32_t c : count) most = c > most ? c : most;
+    return most * 2 > n;
+}
+
+__device__ __forceinline__ uint32_t xcd_contiguous_block() {
+    const uint32_t per = gridDim.x / 8;  // blocks past the last whole group of 8 keep their index
+    return blockIdx.x < per * 8 ? (blockIdx.x & 7u) * per + (blockIdx.x >> 3) : blockIdx.x;
+}
+
 template <typename T, int N, bool AVG>
 __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
     using VT = Vec<T>;
@@ -135,7 +158,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
     constexpr int V = VT::V;
     const uint64_t nvec = a.numel / V;
     const uint64_t stride = (uint64_t)gridDim.x * kReduceThreads;
-    for (uint64_t v = (uint64_t)blockIdx.x * kReduceThreads + threadIdx.x; v < nvec; v += stride) {
+    const uint32_t bid = a.xcd_contiguous ? xcd_contiguous_block() : blockIdx.x;
+    for (uint64_t v = (uint64_t)bid * kReduceThreads + threadIdx.x; v < nvec; v += stride) {
         acc_t acc[V];
         if constexpr (N > 0) {
             uint4 raw[N];
@@ -198,6 +222,7 @@ struct ScatterArgs {
     uint32_t n_out;                    // outputs handled by this launch
     float scale;
     float divisor;
+    uint32_t xcd_contiguous;           // see inputs_alias()
     DimsArg out_dims;                  // packed output index -> reduced-tensor index
     DimsArg in_dims;                   // reduced-tensor index -> input memory
 };
@@ -216,8 +241,9 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
     // (Rotating k by the tile number, so that an output is not pinned to one XCD, was
     // measured and does not help: -6% on flat chunks, +0.5% on column blocks.)
     const uint32_t nk = a.n_out;
-    const uint64_t tile0 = blockIdx.x / nk;
-    const uint32_t k = blockIdx.x % nk;
+    const uint32_t bid = a.xcd_contiguous ? xcd_contiguous_block() : blockIdx.x;
+    const uint64_t tile0 = bid / nk;
+    const uint32_t k = bid % nk;
     const uint64_t stride = (uint64_t)(gridDim.x / nk) * kReduceThreads;
     for (uint64_t t = tile0 * kReduceThreads + threadIdx.x; t < a.total; t += stride) {
         uint64_t col;
@@ -364,6 +390,7 @@ int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, in
     a.numel = numel;
     a.n = n;
     avg_factors(n, op, &a.scale, &a.divisor);
+    a.xcd_contiguous = inputs_alias(in, n);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     switch (dtype) {
@@ -444,6 +471,7 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         // whole units too, which canonicalize guarantees by folding offset into the mask.
         const bool vec = max_unit == V;
         ScatterArgs a{};
+        a.xcd_contiguous = inputs_alias(in, n_in);
         bool o32 = false, i32 = false;
         const int nd = oc.ndim > ic.ndim ? oc.ndim : ic.ndim;
         const int d = nd <= 2 ? 2 : (nd <= 4 ? 4 : -1);  // compiled decode depths

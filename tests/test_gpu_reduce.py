@@ -201,6 +201,27 @@ def test_reduce_over_staging_area_slots():
         area.slot(n)
 
 
+@pytest.mark.parametrize("numel", [1, 1023, 128 * 8 * 8 * 3, 128 * 8 * 61 + 777, 1_000_003])
+def test_reduce_both_block_mappings(numel):
+    # inputs that share a 16 KiB phase take the XCD-contiguous block mapping, inputs at different
+    # phases the plain one; both must cover every element exactly once, for grids that are and
+    # are not a multiple of 8 workgroups
+    n = 8
+    hosts = [_rand(torch.float32, numel, 900 + r) for r in range(n)]
+    want = oracle.reduce([h.numpy() for h in hosts], SUM)
+    for pitch_bytes in (((numel * 4 + 16383) // 16384) * 16384, ((numel * 4 + 16383) // 16384) * 16384 + 4096):
+        store = torch.zeros((n - 1) * pitch_bytes + numel * 4, dtype=torch.uint8, device=DEV)
+        ins = [store[r * pitch_bytes: r * pitch_bytes + numel * 4].view(torch.float32) for r in range(n)]
+        assert len({(t.data_ptr() >> 12) & 3 for t in ins}) == (1 if pitch_bytes % 16384 == 0 else 4)
+        for t, h in zip(ins, hosts):
+            t.copy_(h)
+        out = torch.full((numel + 2,), 7.0, device=DEV)
+        R.all_reduce(out[1:-1], ins, R.ReduceOp.Sum)
+        sync()
+        assert np.array_equal(out[1:-1].cpu().numpy(), want)
+        assert out[0].item() == 7.0 and out[-1].item() == 7.0
+
+
 def test_config1_sum_of_8_packed_chunks():
     from monarch_amd import staging
     s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
@@ -244,6 +265,31 @@ def test_reduce_scatter_mesh_dim_small(dtype, shape):
                                      [oslice(v) for v in out_views], code)
         for k in range(K):
             assert np.array_equal(bits(outs[k]), want[k]), (shape, k, op)
+
+
+@pytest.mark.parametrize("pad", [0, 1024])
+def test_reduce_scatter_both_block_mappings(pad):
+    # slabs of 3 x 16 KiB: back to back they share a 16 KiB phase (XCD-contiguous block mapping),
+    # 4 KiB further apart they do not (plain mapping); 2*24*8 = 384 + ... workgroups, and a second
+    # shape whose workgroup count is not a multiple of 8
+    for H, G, Rr, Cc, K in ((2, 8, 24, 512, 8), (1, 8, 37, 512, 4)):
+        slab = Rr * Cc
+        pitch = slab + pad + (0 if (slab * 4) % 16384 == 0 else (16384 - (slab * 4) % 16384) // 4)
+        g = torch.Generator(device=DEV).manual_seed(77 + pad)
+        x = torch.rand(H * G * pitch, generator=g, device=DEV) * 2 - 1
+        group = [x[gi * pitch:] for gi in range(G)]
+        assert len({(t.data_ptr() >> 12) & 3 for t in group}) == (1 if pad == 0 else 4)
+        in_view = Slice(offset=0, sizes=[H, Rr, Cc], strides=[G * pitch, Cc, 1])
+        w = Cc // K
+        out_views = [Slice(offset=k * w, sizes=[H, Rr, w], strides=[Rr * Cc, Cc, 1]) for k in range(K)]
+        outs = [torch.empty(H * Rr * w, device=DEV) for _ in range(K)]
+        R.reduce_scatter_views(outs, out_views, group, in_view, R.ReduceOp.Sum)
+        sync()
+        hx = x.cpu().numpy()
+        want = oracle.reduce_scatter([hx[gi * pitch:] for gi in range(G)], oslice(in_view),
+                                     [oslice(v) for v in out_views], SUM)
+        for k in range(K):
+            assert np.array_equal(outs[k].cpu().numpy(), want[k]), (H, G, Rr, Cc, K, k)
 
 
 def test_config4_mesh_dim_reduce_scatter_full_size():
