@@ -132,6 +132,91 @@ def wl_c1(torch, stage="pack"):
     return f"c1_f32_every_other_row_{stage}", nbytes, launch, cpu, kern, "f32" if stage == "reduce" else "u8"
 
 
+def wl_c1_pipeline(torch, mode="eager"):
+    """Config 1 end to end: 8 every-other-row views -> their elementwise sum -> unpacked into a view.
+    eager: 8 packs + reduce + unpack (10 launches); graph: the same 10 kernels replayed as one HIP graph;
+    fused: mhip_reduce_scatter reads the 8 strided views directly (2 launches); fused_graph: those two as a graph.
+    GB/s counts the fused pipeline's bytes for every mode, so the modes compare by time."""
+    import numpy as np
+    from monarch_amd import Slice, staging
+    from monarch_amd import reduce as R
+    s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
+    n = 8
+    xs = [torch.from_numpy(np.random.default_rng(1000 + k).uniform(-1, 1, size=(4, 256, 256)).astype(np.float32)).to("cuda:0")
+          for k in range(n)]
+    chunks = [torch.empty(len(s), device="cuda:0") for _ in range(n)]
+    total = torch.empty(len(s), device="cuda:0")
+    back = torch.zeros(4, 256, 256, device="cuda:0")
+    whole = Slice.new_row_major([len(s)])
+    nbytes = (n + 1) * len(s) * 4 + 2 * len(s) * 4
+
+    from monarch_amd import _lib
+    from monarch_amd._lib import ptr_array
+    from monarch_amd.ndslice import slice_array
+
+    def calls(stream):  # prepared C-ABI calls on `stream`: the timed loop pays no Python wrapper cost
+        packs = [prepared("mhip_slice_pack", c.data_ptr(), x.data_ptr(), C.byref(s.c), 4, stream) for x, c in zip(xs, chunks)]
+        red = prepared("mhip_reduce", total.data_ptr(), ptr_array([c.data_ptr() for c in chunks]), n, len(s),
+                       _lib.DTYPE_F32, _lib.OP_SUM, stream)
+        unp = prepared("mhip_slice_unpack", back.data_ptr(), total.data_ptr(), C.byref(s.c), 4, stream)
+        fus = prepared("mhip_reduce_scatter", ptr_array([total.data_ptr()]), slice_array([whole]), 1,
+                       ptr_array([x.data_ptr() for x in xs]), C.byref(s.c), 0, n, _lib.DTYPE_F32, _lib.OP_SUM, stream)
+        return packs + [red, unp], [fus, unp]
+
+    def run(seq):
+        rc = 0
+        for f in seq:
+            rc |= f()
+        return rc
+
+    def eager():
+        for x, c in zip(xs, chunks):
+            staging.pack(x, s, out=c)
+        R.all_reduce(total, chunks, R.ReduceOp.Sum)
+        staging.unpack(back, s, total)
+
+    def fused():
+        R.reduce_scatter_views([total], [whole], xs, s, R.ReduceOp.Sum)
+        staging.unpack(back, s, total)
+
+    body = eager if mode in ("eager", "graph") else fused
+    body()  # once through the checked host API
+    torch.cuda.synchronize()
+    if mode.endswith("graph"):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            seq_e, seq_f = calls(STREAM())  # the capture stream is current here
+            assert run(seq_e if mode == "graph" else seq_f) == 0
+
+        def launch(_i=0):
+            graph.replay()
+            return 0
+    else:
+        seq_e, seq_f = calls(STREAM())
+        seq = seq_e if mode == "eager" else seq_f
+
+        def launch(_i=0):
+            return run(seq)
+    launch.keep = (xs, chunks, total, back)
+
+    def cpu():
+        import oracle
+        os_ = oracle.OSlice(s.offset, s.sizes, s.strides)
+        hx = [x.cpu().numpy().reshape(-1) for x in xs]
+        hb = np.zeros(4 * 256 * 256, dtype=np.float32)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 5 or time.perf_counter() - t0 < 2.0:
+            oracle.unpack(hb, oracle.reduce([oracle.pack(h, os_) for h in hx], oracle.SUM), os_)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": f"full pipeline, {reps} passes of the oracle (per-element Slice::get walk, scalar sum)"}
+
+    kern = {"eager": "10 launches", "graph": "10 kernels, one graph launch", "fused": "reduce_scatter_kernel + slice_copy_kernel",
+            "fused_graph": "2 kernels, one graph launch"}[mode]
+    return f"c1_pipeline_{mode}", nbytes, launch, cpu, kern, "f32"
+
+
 def wl_c2(torch, in_place=False, sets=3, separate=False):
     """8 bf16 chunks of one gradient bucket -> their average.  By default the chunks are the slots of
     one staging area laid out by the library (`mhip_staging_slot_pitch`); `separate` allocates them
@@ -465,6 +550,10 @@ WORKLOADS = {
     "c1_pack": lambda t: wl_c1(t, "pack"),
     "c1_unpack": lambda t: wl_c1(t, "unpack"),
     "c1_reduce": lambda t: wl_c1(t, "reduce"),
+    "c1_pipeline": lambda t: wl_c1_pipeline(t, "eager"),
+    "c1_pipeline_graph": lambda t: wl_c1_pipeline(t, "graph"),
+    "c1_pipeline_fused": lambda t: wl_c1_pipeline(t, "fused"),
+    "c1_pipeline_fused_graph": lambda t: wl_c1_pipeline(t, "fused_graph"),
     "c2": lambda t: wl_c2(t, False),
     "c2_inplace": lambda t: wl_c2(t, True),
     "c2_separate": lambda t: wl_c2(t, False, separate=True),

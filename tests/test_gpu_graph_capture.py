@@ -1,0 +1,100 @@
+"""The device entry points only enqueue kernels on the caller's stream (no allocation, no
+synchronisation, no memset), so a caller can record them into a HIP graph.  A captured
+pack -> reduce -> unpack pipeline and a captured fp8 round trip are replayed several times with
+new input data and eager work in between, and every replay is compared with the eager result."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from monarch_amd import Slice, fp8, staging
+from monarch_amd import reduce as R
+from util import oslice, sync
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_pack_reduce_unpack_pipeline_replays():
+    s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])  # every other row
+    n = 8
+    xs = [torch.zeros(4, 256, 256, device=DEV) for _ in range(n)]
+    chunks = [torch.empty(len(s), device=DEV) for _ in range(n)]
+    total = torch.empty(len(s), device=DEV)
+    back = torch.zeros(4, 256, 256, device=DEV)
+
+    def pipeline():
+        for x, c in zip(xs, chunks):
+            staging.pack(x, s, out=c)
+        R.all_reduce(total, chunks, R.ReduceOp.Sum)
+        staging.unpack(back, s, total)
+
+    def fill(seed):
+        hosts = [np.random.default_rng(seed + k).uniform(-1, 1, size=(4, 256, 256)).astype(np.float32) for k in range(n)]
+        for x, h in zip(xs, hosts):
+            x.copy_(torch.from_numpy(h))
+        return hosts
+
+    def expect(hosts):
+        packed = [oracle.pack(h.reshape(-1), oslice(s)) for h in hosts]
+        want = np.zeros(4 * 256 * 256, dtype=np.float32)
+        oracle.unpack(want, oracle.reduce(packed, oracle.SUM), oslice(s))
+        return want
+
+    hosts = fill(100)
+    pipeline()  # eager
+    sync()
+    assert np.array_equal(back.cpu().numpy().reshape(-1), expect(hosts))
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pipeline()  # warm the stream before capture
+    torch.cuda.current_stream().wait_stream(side)
+    sync()
+    with torch.cuda.graph(graph, stream=side):
+        pipeline()
+    for rep in range(4):
+        hosts = fill(200 + 10 * rep)
+        back.zero_()
+        scratch = torch.randn(1 << 20, device=DEV).sum()  # unrelated eager work between replays
+        graph.replay()
+        sync()
+        assert np.array_equal(back.cpu().numpy().reshape(-1), expect(hosts)), rep
+        assert torch.isfinite(scratch)
+
+
+def test_fp8_bucket_round_trip_replays():
+    g = torch.Generator().manual_seed(5)
+    sizes = [1024, 3000, 1, 7777, 2048, 513]
+    tensors = [torch.zeros(k, dtype=torch.bfloat16, device=DEV) for k in sizes]
+    accs = [torch.zeros(k, dtype=torch.float32, device=DEV) for k in sizes]
+    src, dst = fp8.FlatBucket(tensors), fp8.FlatBucket(accs)
+    total = sum(sizes)
+    q = torch.empty(total, dtype=torch.uint8, device=DEV)
+    scales = torch.empty((total + 1023) // 1024, dtype=torch.float32, device=DEV)
+
+    def pipeline():
+        fp8.quantize_bucket(src, q, scales)
+        fp8.dequant_accumulate_bucket(dst, q, scales)
+
+    pipeline()
+    sync()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pipeline()
+    for rep in range(3):
+        hosts = [(torch.randn(k, generator=g) * (rep + 1)).bfloat16() for k in sizes]
+        for t, h in zip(tensors, hosts):
+            t.copy_(h)
+        for a in accs:
+            a.fill_(float(rep))
+        graph.replay()
+        sync()
+        flat = torch.cat(hosts).view(torch.uint16).numpy()
+        hq, hs = oracle.fp8_quantize(flat, 1024)
+        want = np.full(total, float(rep), dtype=np.float32)
+        oracle.fp8_dequant_accumulate(want, hq, hs, 1024)
+        assert np.array_equal(q.cpu().numpy(), hq) and np.array_equal(scales.cpu().numpy(), hs)
+        assert np.array_equal(torch.cat(accs).cpu().numpy(), want), rep

@@ -225,17 +225,23 @@ def test_reduce_both_block_mappings(numel):
 def test_config1_sum_of_8_packed_chunks():
     from monarch_amd import staging
     s = Slice(offset=0, sizes=[4, 128, 256], strides=[65536, 512, 1])
-    chunks, hosts = [], []
+    chunks, hosts, devs = [], [], []
     for k in range(8):
         rng = np.random.default_rng(1000 + k)
         x = rng.uniform(-1, 1, size=(4, 256, 256)).astype(np.float32)
-        chunks.append(staging.pack(torch.from_numpy(x).to(DEV), s))
+        devs.append(torch.from_numpy(x).to(DEV))
+        chunks.append(staging.pack(devs[-1], s))
         hosts.append(oracle.pack(x.reshape(-1), oslice(s)))
     out = torch.empty_like(chunks[0])
     R.all_reduce(out, chunks, R.ReduceOp.Sum)
     sync()
     assert np.array_equal(out.cpu().numpy(), oracle.reduce(hosts, SUM))
     np.testing.assert_allclose(out.cpu().numpy(), np.sum(np.stack(hosts).astype(np.float64), 0), rtol=1e-6, atol=1e-6)
+    # the fused form reads the eight strided views directly: same bits, no staging chunks
+    fused = torch.empty_like(out)
+    R.reduce_scatter_views([fused], [Slice.new_row_major([len(s)])], devs, s, R.ReduceOp.Sum)
+    sync()
+    assert torch.equal(fused, out)
 
 
 def _c4(H, G, Rr, Cc, K, seed, dtype=torch.float32):
