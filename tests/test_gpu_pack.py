@@ -84,6 +84,19 @@ def test_odd_byte_alignment():
     _roundtrip(Slice(offset=3, sizes=[40, 300], strides=[301, 1]), 2, seed=2, misalign=2, dst_misalign=6)
 
 
+@pytest.mark.parametrize("elem_size", [1, 2, 4, 8, 3, 6])
+def test_rows_that_are_not_whole_chunks(elem_size):
+    # rows at least 16 bytes long whose length is not a multiple of 16 bytes, and staging addresses
+    # that are not 16-byte aligned: chunks straddling a row boundary move as two overlapping vectors
+    cases = [Slice(offset=1, sizes=[300, 1791], strides=[2047, 1]), Slice(offset=0, sizes=[1200, 17], strides=[19, 1]),
+             Slice(offset=5, sizes=[7, 50, 129], strides=[52 * 131, 131, 1]), Slice(offset=0, sizes=[2500, 33], strides=[40, 1]),
+             Slice(offset=2, sizes=[3, 2, 40, 100], strides=[2 * 40 * 128 * 2, 40 * 128, 128, 1]),
+             Slice(offset=0, sizes=[1000, 128], strides=[136, 1])]   # whole chunks, but the staging address is shifted
+    for i, s in enumerate(cases):
+        for dst_misalign in (0, elem_size, 5 * elem_size):
+            _roundtrip(s, elem_size, seed=i, misalign=(i % 3) * elem_size, dst_misalign=dst_misalign)
+
+
 def test_many_dims_peels_on_host():
     # 10 dims that cannot merge (every stride leaves a gap): more than the kernel decodes at once
     sizes = [2] * 10
