@@ -298,6 +298,60 @@ def test_reduce_scatter_both_block_mappings(pad):
             assert np.array_equal(outs[k].cpu().numpy(), want[k]), (H, G, Rr, Cc, K, k)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float64, torch.int32])
+def test_reduce_scatter_rows_that_are_not_whole_vectors(dtype):
+    # rows of at least one 16-byte vector whose length or offset is not a multiple of one: chunks that
+    # straddle an output row are computed as two overlapping vectors
+    for shape in [(2, 4, 9, 77, 7), (1, 3, 50, 1022, 2), (2, 8, 5, 129, 3), (1, 2, 300, 45, 1)]:
+        H, G, Rr, Cc, K = shape
+        x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=sum(shape), dtype=torch.float32)
+        if dtype == torch.int32:
+            x = (x * 1e6).to(torch.int32)
+        else:
+            x = x.to(dtype)
+        slab = Rr * Cc
+        group = [x.view(-1)[gi * slab:] for gi in range(G)]
+        ops = ((R.ReduceOp.Sum, SUM),) if dtype == torch.int32 else ((R.ReduceOp.Sum, SUM), (R.ReduceOp.Avg, AVG))
+        for op, code in ops:
+            store = torch.full((K, H * Rr * w + 8), 7, dtype=dtype, device=DEV)
+            outs = [store[k, 3: 3 + H * Rr * w] for k in range(K)]          # element-aligned only
+            R.reduce_scatter_views(outs, out_views, group, in_view, op)
+            sync()
+            hx = bits(x).reshape(-1)
+            want = oracle.reduce_scatter([hx[g * slab:] for g in range(G)], oslice(in_view),
+                                         [oslice(v) for v in out_views], code) if dtype in (torch.float32, torch.bfloat16) else None
+            for k in range(K):
+                if want is not None:
+                    assert np.array_equal(bits(outs[k]), want[k]), (shape, k, op)
+                else:  # f64 / i32: torch on the host, same order
+                    hv = x.cpu().view(H, G, Rr, Cc)
+                    acc = hv[:, 0].clone()
+                    for g in range(1, G):
+                        acc = acc + hv[:, g]
+                    if code == AVG:
+                        acc = acc / G
+                    assert torch.equal(outs[k].cpu().view(H, Rr, w), acc[:, :, k * w:(k + 1) * w]), (shape, k, op)
+                assert bool((store[k, :3] == 7).all()) and bool((store[k, 3 + H * Rr * w:] == 7).all())
+
+
+def test_reduce_scatter_vectors_crossing_input_rows():
+    # outputs are flat chunks of the reduced tensor while the inputs are read through a view with padded
+    # rows: output vectors that cross an input row fall back to single elements
+    Rr, Cc, G, K = 40, 45, 3, 4
+    pitch = Cc + 3
+    g = torch.Generator(device=DEV).manual_seed(31)
+    xs = [torch.rand(Rr * pitch, generator=g, device=DEV) * 2 - 1 for _ in range(G)]
+    in_view = Slice(offset=0, sizes=[Rr, Cc], strides=[pitch, 1])
+    c = Rr * Cc // K
+    out_views = [Slice(offset=k * c, sizes=[c], strides=[1]) for k in range(K)]
+    outs = [torch.empty(c, device=DEV) for _ in range(K)]
+    R.reduce_scatter_views(outs, out_views, xs, in_view, R.ReduceOp.Sum)
+    sync()
+    want = oracle.reduce_scatter([t.cpu().numpy() for t in xs], oslice(in_view), [oslice(v) for v in out_views], SUM)
+    for k in range(K):
+        assert np.array_equal(outs[k].cpu().numpy(), want[k]), k
+
+
 def test_config4_mesh_dim_reduce_scatter_full_size():
     H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
     x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=4000)
