@@ -231,6 +231,117 @@ __global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a)
     }
 }
 
+// Views whose contiguous runs are shorter than a chunk (element-strided selections such as
+// x[:, ::2], rows of a few bytes): a lane still owns whole 16-byte chunks of the packed side,
+// which it moves with one aligned 128-bit access, and gathers (pack) or scatters (unpack) the
+// chunk's units one by one on the strided side.  All unit loads of a lane are issued before
+// the first use and none is predicated.  Unit addresses come from one full decode per chunk
+// followed by an odometer over the run and the innermost dimension outside it; a full decode
+// is repeated only when that dimension wraps.  Strided-side accesses are NOT non-temporal:
+// the lanes of a wavefront return to the same cache lines for every unit of their chunks.
+constexpr int kGatherUnroll = 2;
+
+template <int U, bool PACK, bool WIDE, int NDIM>
+__global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
+    using T = typename UnitType<U>::type;
+    constexpr int VU = 16 / U;
+    constexpr int UN = kGatherUnroll;
+    const uint64_t tile = blockIdx.x / a.nviews;
+    const uint32_t v = blockIdx.x % a.nviews;
+    char* __restrict__ packed = a.packed[v];
+    T* __restrict__ strided = reinterpret_cast<T*>(a.base) + a.offset[v];
+    const uint64_t c0 = tile * (kThreads * UN) + threadIdx.x;
+    const int nd = NDIM >= 0 ? NDIM : a.dims.ndim;
+    const uint64_t run = a.dims.run;
+    const uint64_t size_last = a.dims.size[nd - 1];
+    const uint64_t step_last = a.dims.stride[nd - 1] - run;  // from one past a run's end to the start of the next run
+    const uint64_t safe_first = a.shift ? VU - a.shift : 0;  // first unit of the view's first whole chunk (the host checks there is one)
+
+    uint64_t off[UN][VU];
+    bool full[UN], edge[UN];
+#pragma unroll
+    for (int i = 0; i < UN; ++i) {
+        const uint64_t c = c0 + (uint64_t)i * kThreads;
+        const uint64_t tb = c * VU;
+        const uint64_t first = tb - a.shift;
+        full[i] = c < a.nchunks && tb >= a.shift && first + VU <= a.total;
+        edge[i] = c < a.nchunks && !full[i];
+        if (full[i]) {
+            uint64_t col;
+            uint64_t loc = decode<WIDE, NDIM>(a.dims, first, &col);
+            uint64_t ilast;  // index along the innermost dimension outside the run
+            if constexpr (WIDE) {
+                ilast = ((first - col) / run) % size_last;
+            } else {
+                uint32_t r32, c32, q32, i32;
+                a.dims.run_div.divmod((uint32_t)first, r32, c32);
+                a.dims.size_div[nd - 1].divmod(r32, q32, i32);
+                ilast = i32;
+            }
+            off[i][0] = loc;
+#pragma unroll
+            for (int j = 1; j < VU; ++j) {
+                ++col;
+                ++loc;
+                if (col == run) {
+                    col = 0;
+                    ++ilast;
+                    loc += step_last;
+                    if (ilast == size_last) {
+                        loc = decode<WIDE, NDIM>(a.dims, first + j, &col);
+                        ilast = 0;
+                    }
+                }
+                off[i][j] = loc;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < VU; ++j) off[i][j] = 0;  // a valid unit: the view is not empty
+        }
+    }
+    union Chunk {
+        uint4 v;
+        T e[VU];
+    };
+    Chunk d[UN];
+    if constexpr (PACK) {
+#pragma unroll
+        for (int i = 0; i < UN; ++i)
+#pragma unroll
+            for (int j = 0; j < VU; ++j) d[i].e[j] = strided[off[i][j]];
+#pragma unroll
+        for (int i = 0; i < UN; ++i)
+            if (full[i]) store16_aligned(packed + ((c0 + (uint64_t)i * kThreads) * VU - a.shift) * U, d[i].v);
+    } else {
+#pragma unroll
+        for (int i = 0; i < UN; ++i) {
+            const uint64_t first = (c0 + (uint64_t)i * kThreads) * VU - a.shift;
+            d[i].v = load16_aligned(packed + (full[i] ? first : safe_first) * U);
+        }
+#pragma unroll
+        for (int i = 0; i < UN; ++i)
+            if (full[i]) {
+#pragma unroll
+                for (int j = 0; j < VU; ++j) strided[off[i][j]] = d[i].e[j];
+            }
+    }
+    // ragged first and last chunk of the view: unit by unit
+#pragma unroll
+    for (int i = 0; i < UN; ++i) {
+        if (edge[i]) {
+            const uint64_t tb = (c0 + (uint64_t)i * kThreads) * VU;
+            for (int j = 0; j < VU; ++j) {
+                const uint64_t t = tb + j - a.shift;
+                if (tb + j >= a.shift && t < a.total) {
+                    uint64_t col;
+                    const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
+                    move_unit<U, PACK>(reinterpret_cast<char*>(strided + l), packed + t * U);
+                }
+            }
+        }
+    }
+}
+
 // Plain contiguous copy of 16-byte units, both sides 16-byte aligned (a contiguous view, the
 // "transfer" of a staging buffer): one chunk per lane, non-temporal load, write-through
 // store.  For a 50/50 read/write stream this shape beats the 8-deep tile above by ~5%
@@ -366,11 +477,25 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
 
 // ---------------- host side ----------------
 
+enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns };
+
 template <int U, bool PACK>
-static void launch_slice_copy_u(bool wide, bool ragged, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
+static void launch_slice_copy_u(bool wide, CopyForm form, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
     const dim3 block(kThreads);
     if constexpr (U < 16) {
-        if (ragged) {
+        if (form == kShortRuns) {
+            if (wide) {
+                hipLaunchKernelGGL((slice_gather_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
+                return;
+            }
+            switch (ndim) {
+                case 1: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
+                case 2: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
+                default: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
+            }
+            return;
+        }
+        if (form == kRaggedRows) {
             if (wide) {
                 hipLaunchKernelGGL((slice_copy_ragged_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
                 return;
@@ -396,13 +521,13 @@ static void launch_slice_copy_u(bool wide, bool ragged, int ndim, dim3 grid, hip
 }
 
 template <bool PACK>
-static void launch_slice_copy(uint32_t unit, bool wide, bool ragged, dim3 grid, hipStream_t stream, const PackArgs& a) {
+static void launch_slice_copy(uint32_t unit, bool wide, CopyForm form, dim3 grid, hipStream_t stream, const PackArgs& a) {
     switch (unit) {
-        case 1: launch_slice_copy_u<1, PACK>(wide, ragged, a.dims.ndim, grid, stream, a); break;
-        case 2: launch_slice_copy_u<2, PACK>(wide, ragged, a.dims.ndim, grid, stream, a); break;
-        case 4: launch_slice_copy_u<4, PACK>(wide, ragged, a.dims.ndim, grid, stream, a); break;
-        case 8: launch_slice_copy_u<8, PACK>(wide, ragged, a.dims.ndim, grid, stream, a); break;
-        default: launch_slice_copy_u<16, PACK>(wide, false, a.dims.ndim, grid, stream, a); break;
+        case 1: launch_slice_copy_u<1, PACK>(wide, form, a.dims.ndim, grid, stream, a); break;
+        case 2: launch_slice_copy_u<2, PACK>(wide, form, a.dims.ndim, grid, stream, a); break;
+        case 4: launch_slice_copy_u<4, PACK>(wide, form, a.dims.ndim, grid, stream, a); break;
+        case 8: launch_slice_copy_u<8, PACK>(wide, form, a.dims.ndim, grid, stream, a); break;
+        default: launch_slice_copy_u<16, PACK>(wide, kWholeChunks, a.dims.ndim, grid, stream, a); break;
     }
 }
 
@@ -483,14 +608,25 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             a.offset[nbatch] = next.offset;
             ++nbatch;
         }
-        // rows that are not whole chunks (and are at least one chunk long) take the two-vector form
-        const bool ragged = unit < 16 && first.ndim >= 1 && first.run >= vu && (first.run % vu != 0 || a.shift != 0);
-        const uint64_t per_block = (uint64_t)kThreads * (ragged ? kRaggedUnroll : kUnroll);
+        CopyForm form = kWholeChunks;
+        if (unit < 16 && first.ndim >= 1 && (first.run % vu != 0 || a.shift != 0)) {
+            // Rows that are not whole chunks.  Measured on 8192^2 matrices with rows of r-1 of r elements:
+            // gathering 4-byte units into a chunk streams at 0.77 of peak whatever the row length (the
+            // two-vector form reaches 0.64-0.75), gathering 2-byte units at 0.50 (two-vector form: 0.50 at
+            // 254-byte rows, 0.58 at 510, 0.69 at 2046); scattering units is slower than either beyond
+            // 256-byte rows (fp32: 0.46-0.49 against 0.61-0.73).
+            uint64_t gather_below = 16 * vu;                 // row length in units
+            if (unit == 1) gather_below = 4 * vu;
+            if (PACK && unit >= 4) gather_below = 256 * vu;  // rows under 4 KiB; longer ones: 0.72-0.75 two-vector vs 0.69-0.74
+            if (first.run < gather_below && first.total >= 2 * vu) form = kShortRuns;
+            else if (first.run >= vu) form = kRaggedRows;
+        }
+        const uint64_t per_block = (uint64_t)kThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : kUnroll);
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
         if (blocks * nbatch > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
         a.nviews = nbatch;
         dim3 grid((uint32_t)(blocks * nbatch));
-        launch_slice_copy<PACK>(unit, !fits32, ragged, grid, stream, a);
+        launch_slice_copy<PACK>(unit, !fits32, form, grid, stream, a);
         if (int rc = launch_status()) return rc;
         k += nbatch;
     }

@@ -97,6 +97,21 @@ def test_rows_that_are_not_whole_chunks(elem_size):
             _roundtrip(s, elem_size, seed=i, misalign=(i % 3) * elem_size, dst_misalign=dst_misalign)
 
 
+@pytest.mark.parametrize("elem_size", [1, 2, 4, 8, 6])
+def test_runs_shorter_than_a_chunk(elem_size):
+    # element-strided selections and rows of a few bytes: packed chunks are gathered / scattered unit by
+    # unit, with the unit addresses stepped by an odometer that re-decodes when the inner dimension wraps
+    cases = [Slice(offset=0, sizes=[500, 333], strides=[700, 2]),              # x[:, ::2]
+             Slice(offset=3, sizes=[5, 7, 9], strides=[7 * 9 * 4 * 2, 9 * 4, 4]),
+             Slice(offset=1, sizes=[4000, 3], strides=[5, 1]),                  # rows of 3 elements
+             Slice(offset=0, sizes=[3, 2, 50, 2], strides=[2 * 50 * 8 * 2, 50 * 8, 8, 4]),
+             Slice(offset=2, sizes=[20000], strides=[3]),
+             Slice(offset=0, sizes=[9, 100, 5], strides=[5, 45 * 2, 1])]          # non-monotone strides, short runs
+    for i, s in enumerate(cases):
+        for dst_misalign in (0, 3 * elem_size):
+            _roundtrip(s, elem_size, seed=40 + i, misalign=(i % 2) * elem_size, dst_misalign=dst_misalign)
+
+
 def test_many_dims_peels_on_host():
     # 10 dims that cannot merge (every stride leaves a gap): more than the kernel decodes at once
     sizes = [2] * 10
