@@ -1,11 +1,17 @@
 // Slice pack/unpack and flat-bucket pack/unpack kernels for gfx950.
 //
 // Every copy is HBM-bound byte movement.  The packed (staging) side is contiguous, so
-// work is cut into 16-byte chunks aligned on the packed address; a thread moves a chunk
-// with one 128-bit access on each side whenever the chunk lies inside one contiguous
-// run of the strided tensor, and unit by unit otherwise (run boundaries, ragged head
-// and tail).  Consecutive lanes take consecutive chunks, so each wavefront instruction
-// touches 1 KiB of contiguous staging memory.
+// work is cut into 16-byte chunks aligned on the packed address, consecutive lanes take
+// consecutive chunks, and each wavefront instruction touches 1 KiB of contiguous staging
+// memory.  What happens on the strided side depends on the view's contiguous runs:
+//   slice_copy_kernel         rows are whole chunks: one 128-bit access per chunk and side
+//   slice_copy_ragged_kernel  rows of at least a chunk that are not whole chunks: a chunk
+//                             straddling a row boundary moves as two overlapping vectors
+//   slice_gather_kernel       runs shorter than (a few) chunks: the chunk's units are
+//                             gathered / scattered one by one
+//   contiguous_copy_kernel    one run: plain copy
+// (views whose memory-contiguous dimension is not the innermost one go to the LDS-tiled
+// transposing kernels instead).  The host picks the form per launch from the canonical slice.
 #include "mhip_device.h"
 #include "fp8_common.h"
 #include "pack_internal.h"
