@@ -111,6 +111,7 @@ extern "C" {
     pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *mut c_void, in_view: *const mhip_slice_t, in_numel: usize, n_in: u32, dtype: c_int, op: c_int, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_quantize(q: *mut c_void, scales: *mut c_void, x_bf16: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_dequant_accumulate(acc: *mut c_void, q: *mut c_void, scales: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_many(acc: *mut c_void, q: *const *mut c_void, scales: *const *mut c_void, n: u32, numel: usize, block: u32, overwrite: c_int, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_quantize_bucket(q: *mut c_void, scales: *mut c_void, d_tensors: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *mut c_void, q: *mut c_void, scales: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
     pub fn mhip_device_count(count: *mut c_int) -> c_int;

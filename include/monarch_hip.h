@@ -226,6 +226,15 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
 int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scales, uint64_t numel,
                                 uint32_t block, mhip_stream_t stream);
 
+/* The receive side of an fp8 exchange with n peers in one pass:
+ *   acc[i] = (overwrite ? 0 : acc[i]) + q[0][i]*scales[0][b] + q[1][i]*scales[1][b] + ...   (b = i / block)
+ * peers in order, each product rounded before its add: bit-identical to n calls of
+ * mhip_fp8_dequant_accumulate (on a zeroed accumulator when overwrite != 0), with the fp32
+ * accumulator crossing HBM once.  q and scales are host tables of n device pointers, n <= 64. */
+int mhip_fp8_dequant_accumulate_many(float* acc, const uint8_t* const* q, const float* const* scales,
+                                     uint32_t n, uint64_t numel, uint32_t block, int overwrite,
+                                     mhip_stream_t stream);
+
 /* Fused forms on a tensor bucket (device tables as for mhip_flat_pack): bit-identical to
  * mhip_flat_pack (bf16) + mhip_fp8_quantize, resp. to mhip_fp8_dequant_accumulate on a flat
  * fp32 accumulator + mhip_flat_unpack, without materialising the flat buffers.  Blocks are

@@ -155,6 +155,90 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float*
     }
 }
 
+// acc[i] (+)= sum over r of float(q_r[i]) * scales_r[i / 1024], peers in order, every product
+// rounded before its add: the same bits as n calls of the kernel above, but the fp32
+// accumulator crosses HBM once instead of n times (n + 8 bytes per element instead of 9n;
+// n + 4 when `overwrite` starts from zero instead of reading acc).
+constexpr int kMaxPeers = 64;
+constexpr int kManySteps = 2;
+
+struct DequantManyArgs {
+    float* acc;
+    const uint8_t* q[kMaxPeers];
+    const float* scales[kMaxPeers];
+    uint64_t numel;
+    uint64_t ntiles;
+    uint32_t n;
+    uint32_t overwrite;
+};
+
+template <int N>  // N > 0: peers known at compile time; N == 0: a.n peers, eight at a time
+__global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_many_kernel(DequantManyArgs a) {
+    float* __restrict__ acc = a.acc;
+    const uint32_t n = N > 0 ? N : a.n;
+    for (uint64_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+        const uint64_t b0 = tile * kManySteps;
+        const uint64_t i0 = b0 * kBlock + threadIdx.x * 4;
+        if ((b0 + kManySteps) * kBlock <= a.numel) {  // interior tile, workgroup-uniform
+            float v[kManySteps][4];
+#pragma unroll
+            for (int j = 0; j < kManySteps; ++j) {
+                if (a.overwrite) {
+                    v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.0f;
+                } else {
+                    const uint4 r = load16_unaligned(acc + i0 + j * kBlock);
+                    v[j][0] = __uint_as_float(r.x); v[j][1] = __uint_as_float(r.y);
+                    v[j][2] = __uint_as_float(r.z); v[j][3] = __uint_as_float(r.w);
+                }
+            }
+            for (uint32_t r0 = 0; r0 < n; r0 += 8) {
+                constexpr int G = N > 0 && N < 8 ? N : 8;
+                uint32_t codes[kManySteps][G];
+                float s[kManySteps][G];
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const uint32_t r = r0 + g < n ? r0 + g : n - 1;  // clamped: the extra loads of a short last group are unused
+#pragma unroll
+                    for (int j = 0; j < kManySteps; ++j) {
+                        codes[j][g] = load4_unaligned(a.q[r] + i0 + j * kBlock);
+                        s[j][g] = a.scales[r][b0 + j];
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    if (r0 + g < n) {
+#pragma unroll
+                        for (int j = 0; j < kManySteps; ++j) {
+                            const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j][g], false);
+                            const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j][g], true);
+                            v[j][0] = v[j][0] + p01[0] * s[j][g];
+                            v[j][1] = v[j][1] + p01[1] * s[j][g];
+                            v[j][2] = v[j][2] + p23[0] * s[j][g];
+                            v[j][3] = v[j][3] + p23[1] * s[j][g];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kManySteps; ++j)
+                store16_unaligned(acc + i0 + j * kBlock, make_uint4(__float_as_uint(v[j][0]), __float_as_uint(v[j][1]),
+                                                                     __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
+            continue;
+        }
+        // last tile: element by element
+        for (int j = 0; j < kManySteps; ++j) {
+            for (uint64_t e = i0 + (uint64_t)j * kBlock; e < a.numel && e < i0 + (uint64_t)j * kBlock + 4; ++e) {
+                float x = a.overwrite ? 0.0f : acc[e];
+                for (uint32_t r = 0; r < n; ++r) {
+                    const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)a.q[r][e], false);
+                    x = x + p[0] * a.scales[r][e / kBlock];
+                }
+                acc[e] = x;
+            }
+        }
+    }
+}
+
 }  // namespace mhip
 
 using namespace mhip;
@@ -191,6 +275,40 @@ int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scale
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kThreads), 0,
                        hs, acc, q, scales, numel, ntiles);
+    return launch_status();
+}
+
+int mhip_fp8_dequant_accumulate_many(float* acc, const uint8_t* const* q, const float* const* scales, uint32_t n,
+                                     uint64_t numel, uint32_t block, int overwrite, mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (!q || !scales || n == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    if (n > (uint32_t)kMaxPeers) return MHIP_ERR_TOO_MANY_INPUTS;
+    if (numel == 0) return MHIP_SUCCESS;
+    if (!acc) return MHIP_ERR_UNDEFINED_TENSOR;
+    if ((uintptr_t)acc & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+    DequantManyArgs a{};
+    for (uint32_t r = 0; r < n; ++r) {
+        if (!q[r] || !scales[r]) return MHIP_ERR_UNDEFINED_TENSOR;
+        if ((uintptr_t)scales[r] & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+        a.q[r] = q[r];
+        a.scales[r] = scales[r];
+    }
+    a.acc = acc;
+    a.numel = numel;
+    a.n = n;
+    a.overwrite = overwrite ? 1u : 0u;
+    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
+    a.ntiles = (nblocks + kManySteps - 1) / kManySteps;
+    const uint64_t cap = 0x7fffffffull;
+    const dim3 grid((uint32_t)(a.ntiles > cap ? cap : a.ntiles)), blockdim(kThreads);
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    switch (n) {
+        case 2: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<2>, grid, blockdim, 0, hs, a); break;
+        case 4: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<4>, grid, blockdim, 0, hs, a); break;
+        case 8: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<8>, grid, blockdim, 0, hs, a); break;
+        default: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<0>, grid, blockdim, 0, hs, a); break;
+    }
     return launch_status();
 }
 

@@ -15,7 +15,7 @@ from typing import List, Sequence
 import torch
 
 from . import _torch
-from ._lib import check, lib
+from ._lib import check, lib, ptr_array
 
 BLOCK = 1024
 FP8_MAX = 448.0
@@ -124,3 +124,26 @@ def dequant_accumulate(acc: torch.Tensor, q: torch.Tensor, scales: torch.Tensor,
         raise ValueError("size mismatch between acc, q and scales")
     check(lib().mhip_fp8_dequant_accumulate(acc.data_ptr(), q.data_ptr(), scales.data_ptr(), q.numel(), BLOCK,
                                             _torch.stream_handle(stream)))
+
+
+def dequant_accumulate_many(acc: torch.Tensor, qs: Sequence[torch.Tensor], scales: Sequence[torch.Tensor],
+                            overwrite: bool = False, stream=None) -> None:
+    """The receive side of an exchange with ``len(qs)`` peers in one pass:
+    ``acc = (0 if overwrite else acc) + sum_r float(qs[r]) * scales[r][i // 1024]``, peers in order,
+    bit-identical to calling ``dequant_accumulate`` once per peer."""
+    if len(qs) == 0 or len(qs) != len(scales):
+        raise ValueError("one scales tensor per code tensor, at least one peer")
+    _torch.require_contiguous(acc)
+    if acc.dtype != torch.float32:
+        raise ValueError("acc must be fp32")
+    n = acc.numel()
+    for q, s in zip(qs, scales):
+        _torch.require_contiguous(q)
+        _torch.require_contiguous(s)
+        if q.element_size() != 1 or s.dtype != torch.float32:
+            raise ValueError("codes must be one byte per element and scales fp32")
+        if q.numel() != n or s.numel() != (n + BLOCK - 1) // BLOCK:
+            raise ValueError("size mismatch between acc, q and scales")
+    check(lib().mhip_fp8_dequant_accumulate_many(acc.data_ptr(), ptr_array([q.data_ptr() for q in qs]),
+                                                 ptr_array([s.data_ptr() for s in scales]), len(qs), n, BLOCK,
+                                                 1 if overwrite else 0, _torch.stream_handle(stream)))

@@ -109,6 +109,38 @@ def test_quantize_dequant_accumulate_ragged():
         assert np.array_equal(o.cpu().numpy(), w)
 
 
+@pytest.mark.parametrize("npeers", [1, 2, 3, 4, 8, 9, 17])
+def test_dequant_accumulate_from_many_peers(npeers):
+    # one pass over n peers' payloads == n single-peer passes, bit for bit, also when starting from zero
+    for numel in (1, 1023, 2048, 2 * 1024 * 7 + 5, 300_000):
+        payloads = []
+        for r in range(npeers):
+            x = _c5_like(numel, seed=31 * npeers + r) * float(1 + r % 3)
+            wq, ws = oracle.fp8_quantize(bits(x), 1024)
+            payloads.append((wq, ws))
+        rng = np.random.default_rng(numel)
+        acc_h = rng.normal(size=numel).astype(np.float32)
+        qs = [torch.from_numpy(wq).to(DEV) for wq, _ in payloads]
+        ss = [torch.from_numpy(ws).to(DEV) for _, ws in payloads]
+        for overwrite in (False, True):
+            want = np.zeros(numel, dtype=np.float32) if overwrite else acc_h.copy()
+            for wq, ws in payloads:
+                oracle.fp8_dequant_accumulate(want, wq, ws, 1024)
+            store = torch.full((numel + 2,), 7.0, device=DEV)
+            acc = store[1:-1]
+            acc.copy_(torch.from_numpy(acc_h))
+            fp8.dequant_accumulate_many(acc, qs, ss, overwrite=overwrite)
+            sync()
+            assert np.array_equal(acc.cpu().numpy().view(np.uint32), want.view(np.uint32)), (npeers, numel, overwrite)
+            assert store[0].item() == 7.0 and store[-1].item() == 7.0
+            if not overwrite:   # and the same as the single-peer entry point called n times
+                seq = torch.from_numpy(acc_h.copy()).to(DEV)
+                for q, s_ in zip(qs, ss):
+                    fp8.dequant_accumulate(seq, q, s_)
+                sync()
+                assert torch.equal(seq, acc)
+
+
 def test_fused_bucket_forms_equal_two_step_pipeline():
     # ragged sizes around block boundaries, empty tensors, odd element alignment, NaN/Inf blocks
     g = torch.Generator().manual_seed(77)
