@@ -240,25 +240,69 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
                 *reinterpret_cast<u32x4*>(&tile[at(q, v16 * E)]) = d[p].v;
             }
             __syncthreads();
+            if constexpr (sizeof(T) == 2) {
+                // Two neighbouring columns at once: eight 32-bit LDS reads fetch (q, c) and (q, c+1) for
+                // eight rows, and a 2x2 transpose in registers turns them into the two output vectors.
+                // Half the LDS instructions of the element-wise form, and no sub-dword accesses.
 #pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                const int cc = r16 + ROWS * p;
-                Vec o;
+                for (int p = 0; p < PASSES / 2; ++p) {
+                    const int c = 2 * (r16 + ROWS * p);
+                    uint32_t w[E];
 #pragma unroll
-                for (int j = 0; j < E; ++j) o.e[j] = tile[at(v16 * E + j, cc)];
-                *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E) = o.v;
+                    for (int j = 0; j < E; ++j) w[j] = *reinterpret_cast<const uint32_t*>(&tile[at(v16 * E + j, c)]);
+                    u32x4 lo, hi;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        lo[k] = (w[2 * k] & 0xffffu) | (w[2 * k + 1] << 16);
+                        hi[k] = (w[2 * k] >> 16) | (w[2 * k + 1] & 0xffff0000u);
+                    }
+                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)c * a.Q + v16 * E) = lo;
+                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E) = hi;
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p) {
+                    const int cc = r16 + ROWS * p;
+                    Vec o;
+#pragma unroll
+                    for (int j = 0; j < E; ++j) o.e[j] = tile[at(v16 * E + j, cc)];
+                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E) = o.v;
+                }
             }
         } else {
+            if constexpr (sizeof(T) == 2) {
+                // the mirror image: rows c and c+1 of the packed side are loaded together and their
+                // halves interleaved into eight 32-bit LDS writes
 #pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                const int cc = r16 + ROWS * p;
-                d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E);
-            }
+                for (int p = 0; p < PASSES / 2; ++p) {
+                    const int c = 2 * (r16 + ROWS * p);
+                    d[2 * p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)c * a.Q + v16 * E);
+                    d[2 * p + 1].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E);
+                }
 #pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                const int cc = r16 + ROWS * p;
+                for (int p = 0; p < PASSES / 2; ++p) {
+                    const int c = 2 * (r16 + ROWS * p);
+                    const u32x4 lo = d[2 * p].v, hi = d[2 * p + 1].v;
 #pragma unroll
-                for (int j = 0; j < E; ++j) tile[at(v16 * E + j, cc)] = d[p].e[j];
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t w0 = (lo[k] & 0xffffu) | (hi[k] << 16);
+                        const uint32_t w1 = (lo[k] >> 16) | (hi[k] & 0xffff0000u);
+                        *reinterpret_cast<uint32_t*>(&tile[at(v16 * E + 2 * k, c)]) = w0;
+                        *reinterpret_cast<uint32_t*>(&tile[at(v16 * E + 2 * k + 1, c)]) = w1;
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p) {
+                    const int cc = r16 + ROWS * p;
+                    d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E);
+                }
+#pragma unroll
+                for (int p = 0; p < PASSES; ++p) {
+                    const int cc = r16 + ROWS * p;
+#pragma unroll
+                    for (int j = 0; j < E; ++j) tile[at(v16 * E + j, cc)] = d[p].e[j];
+                }
             }
             __syncthreads();
 #pragma unroll
