@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a)
 // followed by an odometer over the run and the innermost dimension outside it; a full decode
 // is repeated only when that dimension wraps.  Strided-side accesses are NOT non-temporal:
 // the lanes of a wavefront return to the same cache lines for every unit of their chunks.
-constexpr int kGatherUnroll = 2;
+constexpr int kGatherUnroll = 1;
 
 template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
