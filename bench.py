@@ -29,12 +29,12 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_885_315, "c2_inplace": 452_885_711, "c2_separate": 452_884_036, "c2p_pack": 100_663_296,
-    "c2p_unpack": 100_663_296, "c3_pack": 234_902_749, "c3_unpack": 234_904_867, "c4": 603_819_563,
-    "c4_slots": 603_820_299, "c5_flat_pack": 3_187_684_377, "c5_quantize": 2_362_572_636,
-    "c5_dequant": 7_103_230_055, "c5_flat_unpack": 6_017_507_751, "c5_quantize_bucket": 2_379_634_019,
-    "c5_dequant_bucket": 7_178_104_765, "tr_f32_pack": 536_838_397, "tr_f32_unpack": 536_848_703,
-    "tr_bf16_pack": 268_470_512,
+    "c2": 452_980_098, "c2_inplace": 452_980_226, "c2_separate": 452_979_098, "c2p_pack": 100_663_296,
+    "c2p_unpack": 100_663_241, "c3_pack": 234_977_377, "c3_unpack": 234_958_725, "c4": 603_968_237,
+    "c4_slots": 603_969_709, "c5_flat_pack": 3_174_782_136, "c5_quantize": 2_366_058_518,
+    "c5_dequant": 7_129_890_652, "c5_flat_unpack": 6_016_924_093, "c5_dequant_many8": 12_782_544_690,
+    "c5_quantize_bucket": 2_380_058_974, "c5_dequant_bucket": 7_179_240_731, "tr_f32_pack": 536_911_930,
+    "tr_f32_unpack": 536_922_367, "tr_bf16_pack": 268_505_286,
 }
 
 
