@@ -417,7 +417,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         switch (unit) {
             case 1: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
             case 2: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-            case 4: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
             case 8: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
             default: return false;
         }
