@@ -494,6 +494,17 @@ def wl_c5(torch, stage="quantize"):
         launch = prepared("mhip_fp8_dequant_accumulate_bucket", aptrs.data_ptr(), q.data_ptr(), s.data_ptr(),
                           bucket.d_offsets.data_ptr(), len(sizes), total, 1024, STREAM())
         launch.keep = accs
+    elif stage == "dequant_bucket_many8":
+        qs = [q] + [(q ^ (r + 1)).contiguous() for r in range(1, 8)]
+        ss = [s] + [(s * (1.0 + 0.125 * r)).contiguous() for r in range(1, 8)]
+        nbytes, kern = (8 + 8) * total + 8 * 4 * nblk, "fp8_dequant_accumulate_bucket_many_kernel"
+        accs = [torch.zeros(n, device="cuda:0") for n in sizes]
+        aptrs = bucket.pointer_table(accs)
+        from monarch_amd._lib import ptr_array
+        launch = prepared("mhip_fp8_dequant_accumulate_bucket_many", aptrs.data_ptr(), ptr_array([t.data_ptr() for t in qs]),
+                          ptr_array([t.data_ptr() for t in ss]), 8, bucket.d_offsets.data_ptr(), len(sizes), total, 1024,
+                          STREAM())
+        launch.keep = (accs, qs, ss)
     elif stage in ("dequant_many8", "dequant_many8_overwrite"):
         # 8 peers' payloads (the same codes perturbed per peer) into one accumulator in one pass
         over = stage.endswith("overwrite")
@@ -523,11 +534,11 @@ def wl_c5(torch, stage="quantize"):
         t0 = time.perf_counter()
         if stage in ("quantize", "quantize_bucket"):
             oracle.fp8_quantize(h, 1024)
-        elif stage in ("dequant_accumulate", "dequant_bucket", "dequant_many8", "dequant_many8_overwrite"):
+        elif stage.startswith("dequant"):
             hq, hs = q[:sample].cpu().numpy(), s[: (sample + 1023) // 1024].cpu().numpy()
             ha = np.zeros(sample, dtype=np.float32)
             t0 = time.perf_counter()
-            for _ in range(8 if stage.startswith("dequant_many8") else 1):  # one oracle pass per peer
+            for _ in range(8 if "many8" in stage else 1):  # one oracle pass per peer
                 oracle.fp8_dequant_accumulate(ha, hq, hs, 1024)
         else:
             # the oracle's flat pack / unpack (one memcpy per tensor) over the leading tensors of the bucket
@@ -586,6 +597,7 @@ WORKLOADS = {
     "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
     "c5_dequant_many8": lambda t: wl_c5(t, "dequant_many8"),
     "c5_dequant_many8_overwrite": lambda t: wl_c5(t, "dequant_many8_overwrite"),
+    "c5_dequant_bucket_many8": lambda t: wl_c5(t, "dequant_bucket_many8"),
 }
 
 

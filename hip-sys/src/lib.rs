@@ -114,6 +114,7 @@ extern "C" {
     pub fn mhip_fp8_dequant_accumulate_many(acc: *mut c_void, q: *const *mut c_void, scales: *const *mut c_void, n: u32, numel: usize, block: u32, overwrite: c_int, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_quantize_bucket(q: *mut c_void, scales: *mut c_void, d_tensors: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *mut c_void, q: *mut c_void, scales: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *mut c_void, q: *const *mut c_void, scales: *const *mut c_void, n: u32, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
     pub fn mhip_device_count(count: *mut c_int) -> c_int;
     pub fn mhip_set_device(device: c_int) -> c_int;
     pub fn mhip_device_synchronize() -> c_int;

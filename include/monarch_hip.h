@@ -248,6 +248,14 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
                                        uint32_t ntensors, uint64_t total, uint32_t block,
                                        mhip_stream_t stream);
 
+/* mhip_fp8_dequant_accumulate_bucket for n peers in one pass (q and scales: host tables of n device
+ * pointers, n <= 64): bit-identical to n single-peer calls in peer order, the accumulators cross
+ * HBM once. */
+int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const uint8_t* const* q,
+                                            const float* const* scales, uint32_t n,
+                                            const uint64_t* d_offsets, uint32_t ntensors, uint64_t total,
+                                            uint32_t block, mhip_stream_t stream);
+
 /* ====================================================================== */
 /* Runtime pass-through (the cuda-sys / nccl-sys symbols this path uses)   */
 /* ====================================================================== */

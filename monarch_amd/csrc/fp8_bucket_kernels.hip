@@ -178,6 +178,81 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_bucket_kernel
     }
 }
 
+// The same with n peers' payloads in one pass: every accumulator element crosses HBM once
+// (n + 8 bytes per element instead of 9n).  Peers are added in order, product rounded before
+// each add, so the result has the bits of n single-peer passes.
+constexpr int kMaxBucketPeers = 64;
+
+struct BucketPeersArgs {
+    BucketArgs b;
+    const uint8_t* q[kMaxBucketPeers];
+    const float* scales[kMaxBucketPeers];
+    uint32_t n;
+};
+
+__global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_bucket_many_kernel(BucketPeersArgs p) {
+    const BucketArgs& a = p.b;
+    const int lane = threadIdx.x & 63;
+    const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t nwaves = (uint64_t)gridDim.x * (kThreads / 64);
+    for (uint64_t b = wave; b < a.nblocks; b += nwaves) {
+        const uint64_t begin = b * kBlock;
+        const uint64_t end = begin + kBlock < a.total ? begin + kBlock : a.total;
+        uint32_t t_lo, t_hi;
+        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, &t_lo, &t_hi);
+        if (t_lo == t_hi && end - begin == kBlock) {
+            float* dst = reinterpret_cast<float*>(a.tensors[t_lo]) + (begin - a.offsets[t_lo]);
+            float v[4][4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint4 r = load16_unaligned(dst + j * 256 + lane * 4);
+                v[j][0] = __uint_as_float(r.x); v[j][1] = __uint_as_float(r.y);
+                v[j][2] = __uint_as_float(r.z); v[j][3] = __uint_as_float(r.w);
+            }
+            for (uint32_t r0 = 0; r0 < p.n; r0 += 4) {
+                uint32_t codes[4][4];
+                float s[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t r = r0 + g < p.n ? r0 + g : p.n - 1;  // clamped: surplus loads are unused
+                    s[g] = p.scales[r][b];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) codes[g][j] = load4_unaligned(p.q[r] + begin + j * 256 + lane * 4);
+                }
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if (r0 + g < p.n) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], false);
+                            const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], true);
+                            v[j][0] = v[j][0] + p01[0] * s[g];
+                            v[j][1] = v[j][1] + p01[1] * s[g];
+                            v[j][2] = v[j][2] + p23[0] * s[g];
+                            v[j][3] = v[j][3] + p23[1] * s[g];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                store16_unaligned(dst + j * 256 + lane * 4, make_uint4(__float_as_uint(v[j][0]), __float_as_uint(v[j][1]),
+                                                                      __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
+            continue;
+        }
+        for (uint64_t e = begin + lane; e < end; e += 64) {
+            const uint32_t t = find_tensor(a.offsets, 1, t_lo, t_hi + 1, e);
+            float* ptr = reinterpret_cast<float*>(a.tensors[t]) + (e - a.offsets[t]);
+            float x = *ptr;
+            for (uint32_t r = 0; r < p.n; ++r) {
+                const auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)p.q[r][e], false);
+                x = x + c[0] * p.scales[r][b];
+            }
+            *ptr = x;
+        }
+    }
+}
+
 }  // namespace mhip
 
 using namespace mhip;
@@ -225,6 +300,36 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads), 0,
                        hs, q, scales, a);
+    return launch_status();
+}
+
+int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const uint8_t* const* q,
+                                            const float* const* scales, uint32_t n, const uint64_t* d_offsets,
+                                            uint32_t ntensors, uint64_t total, uint32_t block, mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (!q || !scales || n == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    if (n > (uint32_t)kMaxBucketPeers) return MHIP_ERR_TOO_MANY_INPUTS;
+    if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
+    if (!d_acc_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
+    BucketPeersArgs p{};
+    for (uint32_t r = 0; r < n; ++r) {
+        if (!q[r] || !scales[r]) return MHIP_ERR_UNDEFINED_TENSOR;
+        if ((uintptr_t)scales[r] & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+        p.q[r] = q[r];
+        p.scales[r] = scales[r];
+    }
+    p.n = n;
+    p.b.tensors = reinterpret_cast<char* const*>(d_acc_tensors);
+    p.b.offsets = d_offsets;
+    p.b.total = total;
+    p.b.nblocks = (total + kBlock - 1) / kBlock;
+    p.b.ntensors = ntensors;
+    const uint64_t wgs = (p.b.nblocks + 3) / 4;
+    const uint64_t cap = 0x7fffffffull;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_many_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads),
+                       0, hs, p);
     return launch_status();
 }
 

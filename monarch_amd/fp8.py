@@ -147,3 +147,22 @@ def dequant_accumulate_many(acc: torch.Tensor, qs: Sequence[torch.Tensor], scale
     check(lib().mhip_fp8_dequant_accumulate_many(acc.data_ptr(), ptr_array([q.data_ptr() for q in qs]),
                                                  ptr_array([s.data_ptr() for s in scales]), len(qs), n, BLOCK,
                                                  1 if overwrite else 0, _torch.stream_handle(stream)))
+
+
+def dequant_accumulate_bucket_many(bucket: FlatBucket, qs: Sequence[torch.Tensor], scales: Sequence[torch.Tensor],
+                                   stream=None) -> None:
+    """``dequant_accumulate_bucket`` for all peers' payloads in one pass (peers added in order)."""
+    if bucket.dtype != torch.float32:
+        raise ValueError("dequant_accumulate_bucket_many expects a bucket of fp32 accumulators")
+    if len(qs) == 0 or len(qs) != len(scales):
+        raise ValueError("one scales tensor per code tensor, at least one peer")
+    for q, s in zip(qs, scales):
+        _torch.require_contiguous(q)
+        _torch.require_contiguous(s)
+        if q.element_size() != 1 or s.dtype != torch.float32:
+            raise ValueError("codes must be one byte per element and scales fp32")
+        if q.numel() != bucket.total or s.numel() != (bucket.total + BLOCK - 1) // BLOCK:
+            raise ValueError("size mismatch between the bucket, q and scales")
+    check(lib().mhip_fp8_dequant_accumulate_bucket_many(
+        bucket.d_ptrs.data_ptr(), ptr_array([q.data_ptr() for q in qs]), ptr_array([s.data_ptr() for s in scales]),
+        len(qs), bucket.d_offsets.data_ptr(), len(bucket.sizes), bucket.total, BLOCK, _torch.stream_handle(stream)))

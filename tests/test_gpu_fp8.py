@@ -141,6 +141,30 @@ def test_dequant_accumulate_from_many_peers(npeers):
                 assert torch.equal(seq, acc)
 
 
+@pytest.mark.parametrize("npeers", [1, 3, 4, 8, 9])
+def test_dequant_accumulate_bucket_from_many_peers(npeers):
+    sizes = [1024, 3000, 1, 7777, 2048, 513, 40_000, 5]
+    total = sum(sizes)
+    payloads = []
+    for r in range(npeers):
+        x = _c5_like(total, seed=77 * npeers + r) * float(1 + r % 4)
+        payloads.append(oracle.fp8_quantize(bits(x), 1024))
+    qs = [torch.from_numpy(wq).to(DEV) for wq, _ in payloads]
+    ss = [torch.from_numpy(ws).to(DEV) for _, ws in payloads]
+    rng = np.random.default_rng(npeers)
+    acc_h = rng.normal(size=total).astype(np.float32)
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    accs = [torch.from_numpy(acc_h[offs[i]: offs[i + 1]].copy()).to(DEV) for i in range(len(sizes))]
+    bucket = fp8.FlatBucket(accs)
+    fp8.dequant_accumulate_bucket_many(bucket, qs, ss)
+    sync()
+    want = acc_h.copy()
+    for wq, ws in payloads:
+        oracle.fp8_dequant_accumulate(want, wq, ws, 1024)
+    got = torch.cat(accs).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), npeers
+
+
 def test_fused_bucket_forms_equal_two_step_pipeline():
     # ragged sizes around block boundaries, empty tensors, odd element alignment, NaN/Inf blocks
     g = torch.Generator().manual_seed(77)
