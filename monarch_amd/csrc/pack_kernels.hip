@@ -45,6 +45,22 @@ __device__ __forceinline__ void move_unit(char* strided, char* packed) {
         *reinterpret_cast<T*>(strided) = *reinterpret_cast<const T*>(packed);
 }
 
+// One chunk moved unit by unit, with every unit tested against the view's extent: the ragged first
+// and last chunk of a view, and chunks that no vector form applies to.
+template <int U, bool PACK, bool WIDE, int NDIM>
+__device__ __forceinline__ void move_chunk_by_units(const PackArgs& a, char* strided, char* packed, uint64_t chunk) {
+    constexpr int VU = 16 / U;
+    const uint64_t tb = chunk * VU;
+    for (int j = 0; j < VU; ++j) {
+        const uint64_t t = tb + j - a.shift;
+        if (tb + j >= a.shift && t < a.total) {
+            uint64_t col;
+            const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
+            move_unit<U, PACK>(strided + l * U, packed + t * U);
+        }
+    }
+}
+
 template <int U, bool PACK, bool WIDE, int NDIM, int kUnroll>
 __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     constexpr int VU = 16 / U;  // units per chunk
@@ -140,17 +156,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     if constexpr (VU > 1) {
 #pragma unroll
         for (int i = 0; i < kUnroll; ++i) {
-            if (live[i] && !vec[i]) {
-                const uint64_t tb = (c0 + (uint64_t)i * kThreads) * VU;
-                for (int j = 0; j < VU; ++j) {
-                    const uint64_t t = tb + j - a.shift;
-                    if (tb + j >= a.shift && t < a.total) {
-                        uint64_t col;
-                        const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
-                        move_unit<U, PACK>(strided + l * U, packed + t * U);
-                    }
-                }
-            }
+            if (live[i] && !vec[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kThreads);
         }
     }
 }
@@ -227,17 +233,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a)
     }
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        if (edge[i]) {
-            const uint64_t tb = (c0 + (uint64_t)i * kThreads) * VU;
-            for (int j = 0; j < VU; ++j) {
-                const uint64_t t = tb + j - a.shift;
-                if (tb + j >= a.shift && t < a.total) {
-                    uint64_t col;
-                    const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
-                    move_unit<U, PACK>(strided + l * U, packed + t * U);
-                }
-            }
-        }
+        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kThreads);
     }
 }
 
@@ -338,17 +334,7 @@ __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
     // ragged first and last chunk of the view: unit by unit
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        if (edge[i]) {
-            const uint64_t tb = (c0 + (uint64_t)i * kThreads) * VU;
-            for (int j = 0; j < VU; ++j) {
-                const uint64_t t = tb + j - a.shift;
-                if (tb + j >= a.shift && t < a.total) {
-                    uint64_t col;
-                    const uint64_t l = decode<WIDE, NDIM>(a.dims, t, &col);
-                    move_unit<U, PACK>(reinterpret_cast<char*>(strided + l), packed + t * U);
-                }
-            }
-        }
+        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, reinterpret_cast<char*>(strided), packed, c0 + (uint64_t)i * kThreads);
     }
 }
 
