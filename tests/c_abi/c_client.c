@@ -1,0 +1,191 @@
+/* A plain-C client of include/monarch_hip.h: the shape of the call sequence a host-language
+ * binding makes (device memory and streams through the runtime pass-through, then the data
+ * path), with nothing but libc around it.  It checks results against loops written here, so
+ * it depends neither on Python nor on the test oracle.  Exit code 0 and "c_client ok" on success.
+ *
+ *   gcc -std=c11 -O1 -I include tests/c_abi/c_client.c -o tests/c_abi/c_client \
+ *       -L monarch_amd -lmonarch_hip -Wl,-rpath,'$ORIGIN/../../monarch_amd' -lm
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "monarch_hip.h"
+
+#define CHECK(call)                                                                      \
+    do {                                                                                 \
+        int rc_ = (call);                                                                \
+        if (rc_ != MHIP_SUCCESS) {                                                       \
+            fprintf(stderr, "%s:%d: %s -> %d (%s)\n", __FILE__, __LINE__, #call, rc_,    \
+                    mhip_error_string(rc_));                                             \
+            return 1;                                                                    \
+        }                                                                                \
+    } while (0)
+
+static uint32_t lcg(uint32_t* s) { return *s = *s * 1664525u + 1013904223u; }
+
+static uint16_t f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+static float bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+int main(void) {
+    int ndev = 0;
+    CHECK(mhip_device_count(&ndev));
+    if (ndev < 1) {
+        fprintf(stderr, "no device\n");
+        return 2;
+    }
+    CHECK(mhip_set_device(0));
+    mhip_stream_t stream = NULL;
+    CHECK(mhip_stream_create(&stream));
+
+    /* 1. every other row of a [4,256,256] f32 tensor, packed and unpacked (configuration 1) */
+    enum { N = 4 * 256 * 256, P = 4 * 128 * 256 };
+    float* x = malloc(N * sizeof(float));
+    float* packed = malloc(P * sizeof(float));
+    float* back = malloc(N * sizeof(float));
+    uint32_t seed = 1;
+    for (int i = 0; i < N; ++i) x[i] = (float)(lcg(&seed) >> 8) / 8388608.0f - 1.0f;
+    void *dx, *dp, *db;
+    CHECK(mhip_malloc(&dx, N * sizeof(float)));
+    CHECK(mhip_malloc(&dp, P * sizeof(float)));
+    CHECK(mhip_malloc(&db, N * sizeof(float)));
+    CHECK(mhip_memcpy_htod(dx, x, N * sizeof(float), stream));
+    CHECK(mhip_memset(db, 0, N * sizeof(float), stream));
+    const uint64_t sizes[3] = {4, 128, 256}, strides[3] = {65536, 512, 1};
+    CHECK(mhip_slice_validate(0, sizes, 3, strides, 3));
+    const mhip_slice_t view = {0, 3, sizes, strides};
+    CHECK(mhip_slice_pack(dp, dx, &view, sizeof(float), stream));
+    CHECK(mhip_slice_unpack(db, dp, &view, sizeof(float), stream));
+    CHECK(mhip_memcpy_dtoh(packed, dp, P * sizeof(float), stream));
+    CHECK(mhip_memcpy_dtoh(back, db, N * sizeof(float), stream));
+    CHECK(mhip_stream_synchronize(stream));
+    for (int a = 0, i = 0; a < 4; ++a)
+        for (int r = 0; r < 128; ++r)
+            for (int c = 0; c < 256; ++c, ++i) {
+                const float want = x[a * 65536 + r * 512 + c];
+                if (packed[i] != want || back[a * 65536 + r * 512 + c] != want) {
+                    fprintf(stderr, "pack/unpack mismatch at %d\n", i);
+                    return 1;
+                }
+            }
+    for (int a = 0; a < 4; ++a)
+        for (int r = 1; r < 256; r += 2)
+            for (int c = 0; c < 256; ++c)
+                if (back[a * 65536 + r * 256 + c] != 0.0f) {
+                    fprintf(stderr, "unpack touched an element outside the view\n");
+                    return 1;
+                }
+
+    /* 2. average of 8 bf16 buffers, fp32 accumulation in member order, one rounding */
+    enum { M = 100003, G = 8 };
+    uint16_t* h[G];
+    void* d[G];
+    const void* dptr[G];
+    for (int g = 0; g < G; ++g) {
+        h[g] = malloc(M * sizeof(uint16_t));
+        for (int i = 0; i < M; ++i) h[g][i] = f32_to_bf16(((float)(lcg(&seed) >> 8) / 8388608.0f - 1.0f) * 0.02f);
+        CHECK(mhip_malloc(&d[g], M * sizeof(uint16_t)));
+        CHECK(mhip_memcpy_htod(d[g], h[g], M * sizeof(uint16_t), stream));
+        dptr[g] = d[g];
+    }
+    void* dout;
+    CHECK(mhip_malloc(&dout, M * sizeof(uint16_t)));
+    mhip_event_t e0, e1;
+    CHECK(mhip_event_create(&e0));
+    CHECK(mhip_event_create(&e1));
+    CHECK(mhip_event_record(e0, stream));
+    CHECK(mhip_reduce(dout, dptr, G, M, MHIP_DTYPE_BF16, MHIP_OP_AVG, stream));
+    CHECK(mhip_event_record(e1, stream));
+    uint16_t* out = malloc(M * sizeof(uint16_t));
+    CHECK(mhip_memcpy_dtoh(out, dout, M * sizeof(uint16_t), stream));
+    CHECK(mhip_event_synchronize(e1));
+    float ms = -1.0f;
+    CHECK(mhip_event_elapsed_ms(&ms, e0, e1));
+    CHECK(mhip_stream_synchronize(stream));
+    for (int i = 0; i < M; ++i) {
+        volatile float acc = bf16_to_f32(h[0][i]);
+        for (int g = 1; g < G; ++g) acc = acc + bf16_to_f32(h[g][i]);
+        acc = acc / 8.0f;
+        if (out[i] != f32_to_bf16(acc)) {
+            fprintf(stderr, "reduce mismatch at %d: %04x vs %04x\n", i, out[i], f32_to_bf16(acc));
+            return 1;
+        }
+    }
+    if (!(ms >= 0.0f)) {
+        fprintf(stderr, "event timing failed\n");
+        return 1;
+    }
+
+    /* 3. refusals come back as status codes, not as aborts */
+    if (mhip_reduce(dout, dptr, G, M, MHIP_DTYPE_F8E4M3FN, MHIP_OP_SUM, stream) != MHIP_ERR_FLOAT8_REDUCTION) {
+        fprintf(stderr, "an fp8 reduce was not refused\n");
+        return 1;
+    }
+    const uint64_t bad_strides[3] = {65536, 128, 1};  /* rows of 256 elements only 128 apart: they overlap */
+    if (mhip_slice_validate(0, sizes, 3, bad_strides, 3) != MHIP_ERR_STRIDE_TOO_SMALL) {
+        fprintf(stderr, "overlapping rows were not refused\n");
+        return 1;
+    }
+
+    /* 4. fp8 round trip: block maxima come back exactly (they encode to +-448) */
+    enum { T = 5000 };
+    uint16_t* t16 = malloc(T * sizeof(uint16_t));
+    for (int i = 0; i < T; ++i) t16[i] = f32_to_bf16((float)(lcg(&seed) >> 8) / 8388608.0f - 1.0f);
+    void *dt, *dq, *dsc, *dacc;
+    const int nblk = (T + 1023) / 1024;
+    CHECK(mhip_malloc(&dt, T * 2));
+    CHECK(mhip_malloc(&dq, T));
+    CHECK(mhip_malloc(&dsc, nblk * sizeof(float)));
+    CHECK(mhip_malloc(&dacc, T * sizeof(float)));
+    CHECK(mhip_memcpy_htod(dt, t16, T * 2, stream));
+    CHECK(mhip_memset(dacc, 0, T * sizeof(float), stream));
+    CHECK(mhip_fp8_quantize(dq, dsc, dt, T, 1024, stream));
+    CHECK(mhip_fp8_dequant_accumulate(dacc, dq, dsc, T, 1024, stream));
+    float* acc = malloc(T * sizeof(float));
+    float* sc = malloc(nblk * sizeof(float));
+    CHECK(mhip_memcpy_dtoh(acc, dacc, T * sizeof(float), stream));
+    CHECK(mhip_memcpy_dtoh(sc, dsc, nblk * sizeof(float), stream));
+    CHECK(mhip_stream_synchronize(stream));
+    for (int b = 0; b < nblk; ++b) {
+        float amax = 0.0f;
+        int at = -1;
+        for (int i = b * 1024; i < T && i < (b + 1) * 1024; ++i)
+            if (fabsf(bf16_to_f32(t16[i])) > amax) {
+                amax = fabsf(bf16_to_f32(t16[i]));
+                at = i;
+            }
+        if (sc[b] != amax / 448.0f) {
+            fprintf(stderr, "scale of block %d: %g vs %g\n", b, sc[b], amax / 448.0f);
+            return 1;
+        }
+        /* float(448) * (amax / 448) is amax again up to one rounding of the product */
+        if (fabsf(fabsf(acc[at]) - amax) > amax * 1.2e-7f) {
+            fprintf(stderr, "block maximum of block %d not recovered: %g vs %g\n", b, acc[at], amax);
+            return 1;
+        }
+        for (int i = b * 1024; i < T && i < (b + 1) * 1024; ++i)
+            if (fabsf(acc[i] - bf16_to_f32(t16[i])) > sc[b] * 16.0f + 1e-30f) { /* half of the widest code spacing (32) */
+                fprintf(stderr, "fp8 error too large at %d\n", i);
+                return 1;
+            }
+    }
+
+    for (int g = 0; g < G; ++g) CHECK(mhip_free(d[g]));
+    CHECK(mhip_free(dx)); CHECK(mhip_free(dp)); CHECK(mhip_free(db)); CHECK(mhip_free(dout));
+    CHECK(mhip_free(dt)); CHECK(mhip_free(dq)); CHECK(mhip_free(dsc)); CHECK(mhip_free(dacc));
+    CHECK(mhip_event_destroy(e0)); CHECK(mhip_event_destroy(e1));
+    CHECK(mhip_stream_destroy(stream));
+    printf("c_client ok (reduce of 8 x %d bf16: %.3f ms)\n", (int)M, ms);
+    return 0;
+}
