@@ -77,6 +77,16 @@ def test_fuzz_slices(elem_size):
         _roundtrip(s, elem_size, seed=i, misalign=(i % 4) * elem_size, dst_misalign=(i % 3) * elem_size)
 
 
+@pytest.mark.parametrize("elem_size", [1, 2, 4])
+def test_fuzz_slices_with_longer_rows(elem_size):
+    # the same generator with sizes up to 39: rows long enough for the two-vector and whole-chunk forms,
+    # at every alignment of the strided and the staging side
+    picked = [s for s in fuzz_slices(400, seed=100 + elem_size, max_size=40) if 0 < len(s) <= 150_000][:60]
+    assert len(picked) >= 40
+    for i, s in enumerate(picked):
+        _roundtrip(s, elem_size, seed=i, misalign=(i % 5) * elem_size, dst_misalign=(i % 7) * elem_size)
+
+
 def test_odd_byte_alignment():
     for i, s in enumerate(fuzz_slices(40, seed=99)):
         _roundtrip(s, 1, seed=i, misalign=1 + (i % 15), dst_misalign=(i * 7) % 16)
