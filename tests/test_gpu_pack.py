@@ -5,7 +5,7 @@ import torch
 
 import oracle
 from monarch_amd import Slice, staging
-from util import bits, fuzz_slices, oslice, span, sync
+from util import valid_slices, bits, fuzz_slices, oslice, span, sync
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -79,10 +79,10 @@ def test_fuzz_slices(elem_size):
 
 @pytest.mark.parametrize("elem_size", [1, 2, 4])
 def test_fuzz_slices_with_longer_rows(elem_size):
-    # the same generator with sizes up to 39: rows long enough for the two-vector and whole-chunk forms,
-    # at every alignment of the strided and the staging side
-    picked = [s for s in fuzz_slices(400, seed=100 + elem_size, max_size=40) if 0 < len(s) <= 150_000][:60]
-    assert len(picked) >= 40
+    # valid-by-construction slices with sizes up to 39 in up to four dimensions: rows long enough for the
+    # two-vector and whole-chunk forms, short-run and transposing views, at every alignment of both sides
+    picked = valid_slices(80, seed=100 + elem_size)
+    assert sum(len(s) > 1000 for s in picked) >= 12
     for i, s in enumerate(picked):
         _roundtrip(s, elem_size, seed=i, misalign=(i % 5) * elem_size, dst_misalign=(i % 7) * elem_size)
 

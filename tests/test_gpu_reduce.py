@@ -352,6 +352,37 @@ def test_reduce_scatter_vectors_crossing_input_rows():
         assert np.array_equal(outs[k].cpu().numpy(), want[k]), k
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reduce_scatter_fuzz(dtype):
+    # random input views and random strided
+    # selections of the reduced index space as outputs
+    import random
+    from util import span, valid_slices
+    gen = random.Random(5)
+    views = [v for v in valid_slices(120, seed=17, max_size=24, max_len=60_000) if len(v) >= 64][:40]
+    assert len(views) >= 25
+    for i, in_view in enumerate(views):
+        L, G = len(in_view), gen.choice([1, 2, 3, 5, 8])
+        n_store = span(in_view) + 4
+        hosts = [_rand(dtype, n_store, 1000 * i + g) for g in range(G)]
+        group = [h.to(DEV) for h in hosts]
+        out_views = []
+        for _ in range(gen.choice([1, 2, 4])):
+            st = gen.choice([1, 1, 1, 2, 3])
+            n = gen.randrange(1, max(2, (L - 1) // st))
+            o = gen.randrange(0, L - (n - 1) * st)
+            out_views.append(Slice(offset=o, sizes=[n], strides=[st]))
+        if L % 4 == 0:   # and a two-dimensional one: column blocks of the index space seen as [L/4, 4]
+            out_views.append(Slice(offset=1, sizes=[L // 4, 3], strides=[4, 1]))
+        op, code = gen.choice([(R.ReduceOp.Sum, SUM), (R.ReduceOp.Avg, AVG)])
+        outs = [torch.empty(len(v), dtype=dtype, device=DEV) for v in out_views]
+        R.reduce_scatter_views(outs, out_views, group, in_view, op)
+        sync()
+        want = oracle.reduce_scatter([bits(h).reshape(-1) for h in hosts], oslice(in_view), [oslice(v) for v in out_views], code)
+        for k in range(len(out_views)):
+            assert np.array_equal(bits(outs[k]), want[k]), (i, in_view, out_views[k], G, op)
+
+
 def test_config4_mesh_dim_reduce_scatter_full_size():
     H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
     x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=4000)

@@ -50,5 +50,33 @@ def fuzz_slices(n, seed, max_size=10, max_offset=10000):
     return out
 
 
+def valid_slices(n, seed, max_size=40, max_len=150_000, max_offset=1000):
+    """Random slices that are valid by construction: each stride is the extent of the dimension below it
+    times a random gap factor, a unit innermost stride two times out of three, dimensions in random order.
+    (The reference's rejection sampler above rarely accepts anything beyond one short dimension.)"""
+    gen = random.Random(seed)
+    out = []
+    while len(out) < n:
+        ndim = gen.choice([1, 2, 2, 3, 3, 4])
+        sizes = [gen.randrange(1, max_size) for _ in range(ndim)]
+        total = 1
+        for z in sizes:
+            total *= z
+        if total > max_len:
+            continue
+        strides, stride = [], gen.choice([1, 1, 2, 3])
+        for z in sizes:
+            strides.append(stride)
+            stride = stride * z * gen.choice([1, 1, 2]) if z > 1 else stride * gen.choice([1, 2])
+        order = list(range(ndim))
+        if gen.random() < 0.5:
+            gen.shuffle(order)
+        else:
+            order.reverse()  # row-major: innermost stride last
+        out.append(Slice(offset=gen.randrange(max_offset), sizes=[sizes[o] for o in order],
+                         strides=[strides[o] for o in order]))
+    return out
+
+
 def sync():
     torch.cuda.synchronize()
