@@ -89,6 +89,24 @@ def unpack_many(base: torch.Tensor, views: Sequence[Slice], srcs: Sequence[torch
                                        len(views), base.element_size(), _torch.stream_handle(stream)))
 
 
+# One RDMA work request carries its length in a 32-bit field of the scatter/gather entry
+# (monarch_rdma/src/rdma_components.rs:1041,1063 cast the size with ``as u32``), so a transfer of
+# 4 GiB or more has to be cut into several requests.  Segments are multiples of 16 bytes.
+MAX_SEGMENT_BYTES = (1 << 32) - 16
+
+
+def transfer_segments(nbytes: int, max_bytes: Optional[int] = None):
+    """``(offset, length)`` pairs that cover ``nbytes`` with every length <= ``max_bytes``."""
+    limit = MAX_SEGMENT_BYTES if max_bytes is None else max_bytes
+    if limit <= 0:
+        raise ValueError("segments must hold at least one byte")
+    done = 0
+    while done < nbytes:
+        step = min(limit, nbytes - done)
+        yield done, step
+        done += step
+
+
 class RDMABuffer:
     """A registered contiguous byte range ``{addr, size}`` (rdma_components.rs:94-102).
 
@@ -109,8 +127,10 @@ class RDMABuffer:
         return self._data
 
     def _copy(self, dst_ptr: int, src_ptr: int, nbytes: int, stream) -> None:
-        flat = Slice.new_row_major([nbytes])
-        check(lib().mhip_slice_pack(dst_ptr, src_ptr, C.byref(flat.c), 1, _torch.stream_handle(stream)))
+        for offset, length in transfer_segments(nbytes):  # one "work request" per segment
+            flat = Slice.new_row_major([length])
+            check(lib().mhip_slice_pack(dst_ptr + offset, src_ptr + offset, C.byref(flat.c), 1,
+                                        _torch.stream_handle(stream)))
 
     def read_into(self, dst: torch.Tensor, offset: int = 0, stream=None) -> int:
         _assert_tensor_is_1d_contiguous_uint8(dst)

@@ -267,6 +267,23 @@ def test_tensor_buffer_round_trip():
         buf.read_into(torch.zeros(buf.size + 1, dtype=torch.uint8, device=DEV))
 
 
+def test_rdma_buffer_transfer_in_segments(monkeypatch):
+    # a transfer longer than one work request can carry goes out as several segments
+    monkeypatch.setattr(staging, "MAX_SEGMENT_BYTES", 1008)
+    g = torch.Generator().manual_seed(3)
+    host = torch.randint(0, 256, (5003,), dtype=torch.uint8, generator=g)
+    buf = staging.RDMABuffer(host.to(DEV))
+    dst = torch.zeros(4000, dtype=torch.uint8, device=DEV)
+    assert buf.read_into(dst, offset=1001) == 4000
+    sync()
+    assert torch.equal(dst.cpu(), host[1001:5001])
+    buf.write_from(torch.full((3000,), 9, dtype=torch.uint8, device=DEV), offset=7)
+    sync()
+    want = host.clone()
+    want[7:3007] = 9
+    assert torch.equal(buf.data.cpu(), want)
+
+
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64, torch.complex128])
 def test_transposing_views_lds_path(dtype):
     # permuted views: the memory-contiguous dimension is not the innermost iteration dimension

@@ -314,3 +314,17 @@ def test_send_tensor_routing_and_to_mesh_checks():
         check_to_mesh(["host", "gpu"], slicing, ["host", "gpu"], [2, 4])
     with pytest.raises(ValueError, match="destination mesh does not have dimensions"):
         check_to_mesh(["host", "gpu"], slicing, ["gpu"], [8])
+
+
+def test_transfer_segments_cover_the_range():
+    # lengths fit the 32-bit field of a scatter/gather entry (rdma_components.rs:1041,1063)
+    from monarch_amd.staging import MAX_SEGMENT_BYTES, transfer_segments
+    assert MAX_SEGMENT_BYTES < 2**32 and MAX_SEGMENT_BYTES % 16 == 0
+    assert list(transfer_segments(0)) == []
+    assert list(transfer_segments(100)) == [(0, 100)]
+    assert list(transfer_segments(10, max_bytes=4)) == [(0, 4), (4, 4), (8, 2)]
+    big = list(transfer_segments(3 * 2**32 + 5))
+    assert [o for o, _ in big] == [0, MAX_SEGMENT_BYTES, 2 * MAX_SEGMENT_BYTES, 3 * MAX_SEGMENT_BYTES]
+    assert sum(n for _, n in big) == 3 * 2**32 + 5 and all(n <= MAX_SEGMENT_BYTES for _, n in big)
+    with pytest.raises(ValueError):
+        list(transfer_segments(1, max_bytes=0))
