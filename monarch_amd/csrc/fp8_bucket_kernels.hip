@@ -10,9 +10,8 @@
 // scales are bit-identical to the two-step pipeline.  A wavefront finds the tensors that
 // hold the first and the last element of its span with two cooperative 65-ary searches over
 // the offsets table; a span inside one tensor (the common case: tensors are >= 1K
-// elements) then costs nothing extra, a block that straddles tensors resolves each
-// 8-element (resp. 4-element) group on its own and falls back to single elements only
-// where a group itself straddles.
+// elements) then costs nothing extra; a block that straddles tensors is walked tensor by
+// tensor, the lanes taking consecutive elements of each segment.
 #include "fp8_common.h"
 
 namespace mhip {
@@ -25,40 +24,35 @@ struct BucketArgs {
     uint32_t ntensors;
 };
 
-__device__ __forceinline__ uint16_t bucket_elem_bf16(const BucketArgs& a, uint32_t t_lo, uint32_t t_hi, uint64_t e) {
-    const uint32_t ti = find_tensor(a.offsets, 1, t_lo, t_hi + 1, e);
-    return reinterpret_cast<const uint16_t*>(a.tensors[ti])[e - a.offsets[ti]];
-}
-
-// 8 consecutive bf16 elements of the bucket starting at flat element e
-__device__ __forceinline__ uint4 bucket_load8_bf16(const BucketArgs& a, uint32_t t_lo, uint32_t t_hi, uint64_t e) {
-    const uint32_t ti = find_tensor(a.offsets, 1, t_lo, t_hi + 1, e);
-    const uint64_t begin = a.offsets[ti], end = a.offsets[ti + 1];
-    if (e + 8 <= end) return load16_unaligned(a.tensors[ti] + (e - begin) * 2);
-    uint32_t w[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const uint32_t lo = bucket_elem_bf16(a, ti, t_hi, e + 2 * k);
-        const uint32_t hi = bucket_elem_bf16(a, ti, t_hi, e + 2 * k + 1);
-        w[k] = lo | (hi << 16);
-    }
-    return make_uint4(w[0], w[1], w[2], w[3]);
-}
-
-__device__ __noinline__ void quantize_bucket_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
-                                                           const BucketArgs& a, uint32_t t_lo, uint32_t t_hi,
-                                                           uint64_t begin, uint32_t count, uint64_t b, int lane) {
+// Careful path for one block that straddles tensors, holds NaN / Inf, or is the short last block of
+// the bucket, whole wavefront.  [t_lo, t_hi] are the tensors of its first and last element.  The block
+// is walked tensor by tensor (a wave-uniform loop whose table reads are scalar loads), so that inside a
+// segment the lanes take consecutive elements from one base pointer and no lane searches the table.
+__device__ void quantize_bucket_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                           char* const* tensors, const uint64_t* offsets, uint32_t t_lo,
+                                                           uint32_t t_hi, uint64_t begin, uint32_t count, uint64_t b,
+                                                           int lane) {
+    const uint64_t end = begin + count;
     uint32_t m = 0;
-    for (uint32_t i = lane; i < count; i += 64) {
-        const uint32_t v = bucket_elem_bf16(a, t_lo, t_hi, begin + i) & 0x7fffu;
-        if (v <= 0x7f80u && v > m) m = v;
+    for (uint32_t t = t_lo; t <= t_hi; ++t) {
+        const uint64_t off = offsets[t], next = offsets[t + 1];
+        const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+        const uint16_t* __restrict__ p = reinterpret_cast<const uint16_t*>(tensors[t]) - off;  // p[e] is bucket element e
+        for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
+            const uint32_t v = p[e] & 0x7fffu;
+            if (v <= 0x7f80u && v > m) m = v;
+        }
     }
     m = wave_max_u32(m);
     float scale, inv;
     block_factors(m, &scale, &inv);
     if (lane == 0) scales[b] = scale;
-    for (uint32_t i = lane; i < count; i += 64)
-        q[begin + i] = quant_one_careful(bucket_elem_bf16(a, t_lo, t_hi, begin + i), inv);
+    for (uint32_t t = t_lo; t <= t_hi; ++t) {
+        const uint64_t off = offsets[t], next = offsets[t + 1];
+        const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+        const uint16_t* __restrict__ p = reinterpret_cast<const uint16_t*>(tensors[t]) - off;
+        for (uint64_t e = seg_b + lane; e < seg_e; e += 64) q[e] = quant_one_careful(p[e], inv);
+    }
 }
 
 // A wavefront handles kBucketBlocks consecutive blocks per step (8 KiB of input): one
@@ -66,6 +60,109 @@ __device__ __noinline__ void quantize_bucket_block_careful(uint8_t* __restrict__
 // whole span; when they coincide (the common case) all 2 * kBucketBlocks loads of a lane
 // are issued back to back from one base pointer.
 constexpr int kBucketBlocks = 4;
+
+// ---- 16-byte-aligned loads of a span that starts at an odd multiple of 2 bytes ----
+// Tensors of a bucket start wherever the previous one ended, so a span's bytes are usually not
+// 16-byte aligned in memory, and unaligned 128-bit loads of 2-byte data cost this kernel 8% (0.70 of
+// peak against 0.76 on the same bucket with every tensor padded to 8 elements).  When the tensor
+// extends far enough on both sides, the wavefront loads the enclosing aligned vectors instead and
+// shifts the bytes into place: lane i needs the tail of its own vector and the head of lane i+1's,
+// which a DPP wavefront shift delivers (lane 63 takes lane 0 of the next 1 KiB row), followed by a
+// 128-bit funnel shift built from v_alignbyte.
+__device__ __forceinline__ uint32_t wave_shl1(uint32_t v, uint32_t fill) {
+    // lane i <- lane i + 1; lane 63 <- fill (wave-uniform)
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)fill, (int)v, 0x130, 0xF, 0xF, false);
+}
+
+// bytes [4 * D + r, 4 * D + r + 16) of the 32 bytes {a, b}
+template <int D>
+__device__ __forceinline__ uint4 funnel16(const uint4& a, const uint4& b, uint32_t r) {
+    const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    return make_uint4(__builtin_amdgcn_alignbyte(w[D + 1], w[D], r), __builtin_amdgcn_alignbyte(w[D + 2], w[D + 1], r),
+                      __builtin_amdgcn_alignbyte(w[D + 3], w[D + 2], r), __builtin_amdgcn_alignbyte(w[D + 4], w[D + 3], r));
+}
+
+// v[k] (k < N) are the lane's aligned vectors of N consecutive 1 KiB rows starting `shift` bytes before
+// the wanted data, tail is the first vector after the last row (the same for all lanes).  Replaces every
+// v[k] by the 16 wanted bytes.
+template <int D, int N>
+__device__ __forceinline__ void shift_rows(uint4 (&v)[N], const uint4& tail, uint32_t r) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) {  // ascending: v[k + 1] is still untouched when row k needs its lane 0
+        const uint4& after = k + 1 < N ? v[k + 1] : tail;
+        uint4 next;
+        next.x = wave_shl1(v[k].x, __builtin_amdgcn_readfirstlane(after.x));
+        next.y = wave_shl1(v[k].y, __builtin_amdgcn_readfirstlane(after.y));
+        next.z = wave_shl1(v[k].z, __builtin_amdgcn_readfirstlane(after.z));
+        next.w = wave_shl1(v[k].w, __builtin_amdgcn_readfirstlane(after.w));
+        v[k] = funnel16<D>(v[k], next, r);
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void shift_rows_into_place(uint4 (&v)[N], const uint4& tail, uint32_t shift) {
+    const uint32_t r = shift & 3u;
+    switch (shift >> 2) {  // wave-uniform
+        case 0: shift_rows<0, N>(v, tail, r); break;
+        case 1: shift_rows<1, N>(v, tail, r); break;
+        case 2: shift_rows<2, N>(v, tail, r); break;
+        default: shift_rows<3, N>(v, tail, r); break;
+    }
+}
+
+// One full block whose 16 elements per lane are already in registers.  Returns false (and does
+// nothing) when the block holds Inf or NaN and has to take the careful path.
+__device__ __forceinline__ bool quantize_loaded_block(uint8_t* __restrict__ q, float* __restrict__ scales, uint4 lo, uint4 hi,
+                                                      uint64_t begin, uint64_t b, int lane) {
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t m = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t v = w[k] & 0x7fff7fffu;
+        const uint32_t v0 = v & 0xffffu, v1 = v >> 16;
+        m = v0 > m ? v0 : m;
+        m = v1 > m ? v1 : m;
+    }
+    m = wave_max_u32(m);
+    if (m >= 0x7f80u) return false;  // wave-uniform
+    float scale, inv;
+    block_factors(m, &scale, &inv);
+    if (lane == 0) scales[b] = scale;
+    int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+    c0 = quant_pair<false>(w[0], inv, c0); c0 = quant_pair<true>(w[1], inv, c0);
+    c1 = quant_pair<false>(w[2], inv, c1); c1 = quant_pair<true>(w[3], inv, c1);
+    c2 = quant_pair<false>(w[4], inv, c2); c2 = quant_pair<true>(w[5], inv, c2);
+    c3 = quant_pair<false>(w[6], inv, c3); c3 = quant_pair<true>(w[7], inv, c3);
+    uint8_t* dst = q + begin;
+    store8_unaligned(dst + lane * 8, (uint32_t)c0, (uint32_t)c1);
+    store8_unaligned(dst + 512 + lane * 8, (uint32_t)c2, (uint32_t)c3);
+    return true;
+}
+
+// The rare span that touches several tensors or holds the short last block: block by block, each
+// block narrowed to its own tensors by a wave-uniform walk over the table.
+__device__ void quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                       char* const* tensors, const uint64_t* offsets, uint64_t total,
+                                                       uint64_t nblocks, uint32_t t_first, uint32_t t_last, uint64_t b0,
+                                                       int lane) {
+    uint32_t tb = t_first;
+    for (int j = 0; j < kBucketBlocks; ++j) {
+        const uint64_t b = b0 + j;
+        if (b >= nblocks) break;
+        const uint64_t begin = b * kBlock;
+        const uint64_t end = begin + kBlock < total ? begin + kBlock : total;
+        while (tb < t_last && offsets[tb + 1] <= begin) ++tb;
+        uint32_t te = tb;
+        while (te < t_last && offsets[te + 1] < end) ++te;
+        if (tb == te && end - begin == kBlock) {
+            const char* src = tensors[tb] + (begin - offsets[tb]) * 2;
+            const uint4 lo = load16_unaligned(src + lane * 16);
+            const uint4 hi = load16_unaligned(src + 1024 + lane * 16);
+            if (quantize_loaded_block(q, scales, lo, hi, begin, b, lane)) continue;
+        }
+        quantize_bucket_block_careful(q, scales, tensors, offsets, tb, te, begin, (uint32_t)(end - begin), b, lane);
+    }
+}
 
 __global__ __launch_bounds__(kThreads) void fp8_quantize_bucket_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                        BucketArgs a) {
@@ -78,55 +175,30 @@ __global__ __launch_bounds__(kThreads) void fp8_quantize_bucket_kernel(uint8_t* 
                                       ? span_begin + (uint64_t)kBucketBlocks * kBlock : a.total;
         uint32_t t_first, t_last;
         wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, span_begin, span_end - 1, &t_first, &t_last);
-        uint4 lo[kBucketBlocks], hi[kBucketBlocks];
-        const bool one_tensor = t_first == t_last && span_end - span_begin == (uint64_t)kBucketBlocks * kBlock;
-        if (one_tensor) {  // wave-uniform
-            const char* src = a.tensors[t_first] + (span_begin - a.offsets[t_first]) * 2;
+        if (t_first != t_last || span_end - span_begin != (uint64_t)kBucketBlocks * kBlock) {  // wave-uniform, rare
+            quantize_bucket_span_slow(q, scales, a.tensors, a.offsets, a.total, a.nblocks, t_first, t_last, b0, lane);
+            continue;
+        }
+        // the whole span lies in one tensor: all loads of the lane back to back from one base pointer
+        const uint64_t t_begin = a.offsets[t_first], t_end = a.offsets[t_first + 1];
+        const char* src = a.tensors[t_first] + (span_begin - t_begin) * 2;
+        const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
+        uint4 row[2 * kBucketBlocks];  // row[2j] = first, row[2j + 1] = second 1 KiB of block j
+        if (shift != 0 && (span_begin - t_begin) * 2 >= shift && (t_end - span_end) * 2 >= 16 - shift) {
+            const char* base = src - shift;  // 16-byte aligned, and [base, base + 8 KiB + 16) lies inside the tensor
 #pragma unroll
-            for (int j = 0; j < kBucketBlocks; ++j) {
-                lo[j] = load16_unaligned(src + j * 2048 + lane * 16);
-                hi[j] = load16_unaligned(src + j * 2048 + 1024 + lane * 16);
-            }
+            for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_aligned(base + k * 1024 + lane * 16);
+            const uint4 tail = load16_aligned(base + 2 * kBucketBlocks * 1024);
+            shift_rows_into_place<2 * kBucketBlocks>(row, tail, shift);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_unaligned(src + k * 1024 + lane * 16);
         }
 #pragma unroll
         for (int j = 0; j < kBucketBlocks; ++j) {
             const uint64_t b = b0 + j;
-            if (b >= a.nblocks) break;
-            const uint64_t begin = b * kBlock;
-            const uint64_t end = begin + kBlock < a.total ? begin + kBlock : a.total;
-            if (end - begin < kBlock) {  // short final block
-                quantize_bucket_block_careful(q, scales, a, t_first, t_last, begin, (uint32_t)(end - begin), b, lane);
-                continue;
-            }
-            if (!one_tensor) {
-                lo[j] = bucket_load8_bf16(a, t_first, t_last, begin + lane * 8);
-                hi[j] = bucket_load8_bf16(a, t_first, t_last, begin + 512 + lane * 8);
-            }
-            const uint32_t w[8] = {lo[j].x, lo[j].y, lo[j].z, lo[j].w, hi[j].x, hi[j].y, hi[j].z, hi[j].w};
-            uint32_t m = 0;
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const uint32_t v = w[k] & 0x7fff7fffu;
-                const uint32_t v0 = v & 0xffffu, v1 = v >> 16;
-                m = v0 > m ? v0 : m;
-                m = v1 > m ? v1 : m;
-            }
-            m = wave_max_u32(m);
-            if (m >= 0x7f80u) {  // Inf or NaN in the block
-                quantize_bucket_block_careful(q, scales, a, t_first, t_last, begin, kBlock, b, lane);
-                continue;
-            }
-            float scale, inv;
-            block_factors(m, &scale, &inv);
-            if (lane == 0) scales[b] = scale;
-            int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
-            c0 = quant_pair<false>(w[0], inv, c0); c0 = quant_pair<true>(w[1], inv, c0);
-            c1 = quant_pair<false>(w[2], inv, c1); c1 = quant_pair<true>(w[3], inv, c1);
-            c2 = quant_pair<false>(w[4], inv, c2); c2 = quant_pair<true>(w[5], inv, c2);
-            c3 = quant_pair<false>(w[6], inv, c3); c3 = quant_pair<true>(w[7], inv, c3);
-            uint8_t* dst = q + begin;
-            store8_unaligned(dst + lane * 8, (uint32_t)c0, (uint32_t)c1);
-            store8_unaligned(dst + 512 + lane * 8, (uint32_t)c2, (uint32_t)c3);
+            if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane))
+                quantize_bucket_block_careful(q, scales, a.tensors, a.offsets, t_first, t_first, b * kBlock, kBlock, b, lane);
         }
     }
 }
@@ -168,12 +240,15 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_bucket_kernel
             }
             continue;
         }
-        // straddling or short block: element by element, 16 per lane at most
-        for (uint64_t e = begin + lane; e < end; e += 64) {
-            const uint32_t t = find_tensor(a.offsets, 1, t_lo, t_hi + 1, e);
-            float* p = reinterpret_cast<float*>(a.tensors[t]) + (e - a.offsets[t]);
-            const auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
-            *p = *p + v[0] * s;
+        // straddling or short block: tensor by tensor (wave-uniform loop), lanes on consecutive elements
+        for (uint32_t t = t_lo; t <= t_hi; ++t) {
+            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
+            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+            float* __restrict__ p = reinterpret_cast<float*>(a.tensors[t]) - off;  // p[e] is bucket element e
+            for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
+                const auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
+                p[e] = p[e] + v[0] * s;
+            }
         }
     }
 }
@@ -240,15 +315,18 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_bucket_many_k
                                                                       __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
             continue;
         }
-        for (uint64_t e = begin + lane; e < end; e += 64) {
-            const uint32_t t = find_tensor(a.offsets, 1, t_lo, t_hi + 1, e);
-            float* ptr = reinterpret_cast<float*>(a.tensors[t]) + (e - a.offsets[t]);
-            float x = *ptr;
-            for (uint32_t r = 0; r < p.n; ++r) {
-                const auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)p.q[r][e], false);
-                x = x + c[0] * p.scales[r][b];
+        for (uint32_t t = t_lo; t <= t_hi; ++t) {  // straddling or short block: tensor by tensor
+            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
+            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+            float* __restrict__ ptr = reinterpret_cast<float*>(a.tensors[t]) - off;
+            for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
+                float x = ptr[e];
+                for (uint32_t r = 0; r < p.n; ++r) {
+                    const auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)p.q[r][e], false);
+                    x = x + c[0] * p.scales[r][b];
+                }
+                ptr[e] = x;
             }
-            *ptr = x;
         }
     }
 }
