@@ -9,7 +9,8 @@
 //                             straddling a row boundary moves as two overlapping vectors
 //   slice_gather_kernel       runs shorter than (a few) chunks: the chunk's units are
 //                             gathered / scattered one by one
-//   contiguous_copy_kernel    one run: plain copy
+//   contiguous_copy_kernel    one run: plain copy (contiguous_copy_shift_kernel when an end or an
+//                             address is not 16-byte aligned)
 // (views whose memory-contiguous dimension is not the innermost one go to the LDS-tiled
 // transposing kernels instead).  The host picks the form per launch from the canonical slice.
 #include "mhip_device.h"
@@ -348,6 +349,79 @@ __global__ __launch_bounds__(kThreads) void contiguous_copy_kernel(char* __restr
     if (c < nchunks) store16_writethrough(dst + c * 16, load16_aligned(src + c * 16));
 }
 
+// Contiguous copy between byte ranges of any alignment.  The chunk grid is aligned on the destination
+// (aligned 128-bit write-through stores); the source is read as the enclosing aligned vectors, which
+// a wavefront shifts into place (shift_rows_into_place), so neither side sees an unaligned 128-bit
+// access.  A wavefront owns ROWS consecutive 1 KiB rows.  [head, head + 16 * nvec) of the range is the
+// part whose aligned source vectors all lie inside the source range; the bytes before and after it
+// (fewer than 32 each) are copied one by one by the first workgroup.
+struct ShiftCopyArgs {
+    char* dst;
+    const char* src;
+    uint64_t nbytes;
+    uint64_t head;   // bytes before the vector part
+    uint64_t nvec;   // 16-byte destination vectors in the vector part
+};
+
+template <int ROWS>
+__global__ __launch_bounds__(kThreads) void contiguous_copy_shift_kernel(ShiftCopyArgs a) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    char* __restrict__ dst = a.dst + a.head;            // 16-byte aligned
+    const char* src = a.src + a.head;
+    const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
+    const char* __restrict__ base = src - shift;        // 16-byte aligned
+    // source vectors 0 .. nvec are readable when the source is shifted (one more than is stored), 0 .. nvec - 1 otherwise
+    const uint64_t last = shift ? a.nvec : a.nvec - 1;
+    const uint64_t row0 = wave * (ROWS * 64);
+    if (row0 < a.nvec) {
+        uint4 v[ROWS];
+#pragma unroll
+        for (int k = 0; k < ROWS; ++k) {
+            const uint64_t c = row0 + k * 64 + lane;
+            v[k] = load16_aligned(base + (c < last ? c : last) * 16);  // clamped: never predicated
+        }
+        if (shift != 0) {  // wave-uniform
+            const uint64_t ct = row0 + ROWS * 64;
+            const uint4 tail = load16_aligned(base + (ct < last ? ct : last) * 16);
+            shift_rows_into_place<ROWS>(v, tail, shift);
+        }
+#pragma unroll
+        for (int k = 0; k < ROWS; ++k) {
+            const uint64_t c = row0 + k * 64 + lane;
+            if (c < a.nvec) store16_writethrough(dst + c * 16, v[k]);
+        }
+    }
+    if (blockIdx.x == 0) {
+        for (uint64_t i = threadIdx.x; i < a.head; i += kThreads) a.dst[i] = a.src[i];
+        for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kThreads) a.dst[i] = a.src[i];
+    }
+}
+
+constexpr int kShiftCopyRows = 2;
+
+// Plans and launches the copy above.  Returns false when the range is too short to have a vector part.
+static bool launch_shift_copy(char* dst, const char* src, uint64_t nbytes, hipStream_t stream, int* rc) {
+    if (nbytes < 96) return false;
+    uint64_t head = (16 - ((uintptr_t)dst & 15u)) & 15u;
+    const uint32_t shift = (uint32_t)(((uintptr_t)src + head) & 15u);
+    if (head < shift) head += 16;                       // the first aligned source vector must not start before src
+    uint64_t nvec = (nbytes - head) / 16;
+    uint64_t tail = nbytes - head - nvec * 16;
+    if (shift != 0 && tail < 16 - shift) {              // nor may the last one end after src + nbytes
+        --nvec;
+        tail += 16;
+    }
+    if (nvec == 0) return false;
+    ShiftCopyArgs a{dst, src, nbytes, head, nvec};
+    const uint64_t per_wg = (uint64_t)(kThreads / 64) * kShiftCopyRows * 64;
+    const uint64_t wgs = (nvec + per_wg - 1) / per_wg;
+    if (wgs > 0x7fffffffull) return false;
+    hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3((uint32_t)wgs), dim3(kThreads), 0, stream, a);
+    *rc = launch_status();
+    return true;
+}
+
 // ---------------- flat bucket <-> ragged tensors ----------------
 
 struct FlatArgs {
@@ -579,6 +653,15 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             if (int rc = launch_status()) return rc;
             ++k;
             continue;
+        }
+        if (first.ndim == 0 && unit < 16) {  // one run whose ends or addresses are not 16-byte aligned
+            char* strided = base + first.offset * unit;
+            int crc = MHIP_SUCCESS;
+            if (launch_shift_copy(PACK ? packed[k] : strided, PACK ? strided : packed[k], first.total * unit, stream, &crc)) {
+                if (crc) return crc;
+                ++k;
+                continue;
+            }
         }
         {
             int trc = MHIP_SUCCESS;

@@ -87,6 +87,32 @@ def test_fuzz_slices_with_longer_rows(elem_size):
         _roundtrip(s, elem_size, seed=i, misalign=(i % 5) * elem_size, dst_misalign=(i % 7) * elem_size)
 
 
+def test_contiguous_copy_at_every_alignment():
+    # one run of bytes, every combination of source and destination alignment, lengths around the
+    # point where the copy gets a vector part (aligned stores, shifted aligned loads) plus ragged ends
+    import ctypes as C
+    from monarch_amd._lib import check, lib
+    g = torch.Generator().manual_seed(9)
+    host = torch.randint(0, 256, (80_000,), dtype=torch.uint8, generator=g)
+    src_store = host.to(DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    for n in (1, 15, 95, 96, 97, 111, 128, 1000, 4097, 70_001):
+        s = Slice.new_row_major([n])
+        for so in (0, 1, 2, 5, 8, 15):
+            for do in (0, 1, 3, 8, 14):
+                dst_store = torch.full((n + 64,), 0xEE, dtype=torch.uint8, device=DEV)
+                check(lib().mhip_slice_pack(dst_store.data_ptr() + 16 + do, src_store.data_ptr() + so, C.byref(s.c), 1, stream))
+                back = torch.full((n + 64,), 0x11, dtype=torch.uint8, device=DEV)
+                check(lib().mhip_slice_unpack(back.data_ptr() + 16 + so, dst_store.data_ptr() + 16 + do, C.byref(s.c), 1, stream))
+                sync()
+                got = dst_store.cpu()
+                assert torch.equal(got[16 + do: 16 + do + n], host[so: so + n]), (n, so, do)
+                assert bool((got[:16 + do] == 0xEE).all()) and bool((got[16 + do + n:] == 0xEE).all()), (n, so, do)
+                gb = back.cpu()
+                assert torch.equal(gb[16 + so: 16 + so + n], host[so: so + n]), (n, so, do)
+                assert bool((gb[:16 + so] == 0x11).all()) and bool((gb[16 + so + n:] == 0x11).all()), (n, so, do)
+
+
 def test_odd_byte_alignment():
     for i, s in enumerate(fuzz_slices(40, seed=99)):
         _roundtrip(s, 1, seed=i, misalign=1 + (i % 15), dst_misalign=(i * 7) % 16)
