@@ -30,10 +30,10 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
     "c2": 452_980_098, "c2_inplace": 452_980_226, "c2_separate": 452_979_098, "c2p_pack": 100_663_296,
-    "c2p_unpack": 100_663_241, "c3_pack": 234_977_377, "c3_unpack": 234_958_725, "c4": 603_968_237,
-    "c4_slots": 603_969_709, "c5_flat_pack": 3_174_782_136, "c5_quantize": 2_366_058_518,
+    "c2p_unpack": 100_663_241, "c3_pack": 234_978_355, "c3_unpack": 234_963_309, "c4": 603_968_237,
+    "c4_slots": 603_969_709, "c5_flat_pack": 3_166_564_842, "c5_quantize": 2_366_058_518,
     "c5_dequant": 7_129_890_652, "c5_flat_unpack": 6_016_924_093, "c5_dequant_many8": 12_782_544_690,
-    "c5_quantize_bucket": 2_380_058_974, "c5_dequant_bucket": 7_179_240_731, "tr_f32_pack": 536_911_930,
+    "c5_quantize_bucket": 2_374_780_329, "c5_dequant_bucket": 7_177_730_135, "tr_f32_pack": 536_911_930,
     "tr_f32_unpack": 536_922_367, "tr_bf16_pack": 268_505_286,
 }
 
