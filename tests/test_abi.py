@@ -112,6 +112,26 @@ def test_rust_extern_block_names_match_header():
         assert re.search(rf"pub const {name}: i32 = {value};", text), name
 
 
+def _param_counts(text, pattern):
+    counts = {}
+    for name, params in re.findall(pattern, text, flags=re.S):
+        params = params.strip()
+        counts[name] = 0 if params in ("", "void") else params.count(",") + 1
+    return counts
+
+
+def test_every_binding_has_the_header_parameter_count():
+    # the header, the ctypes table and the Rust extern block declare the same number of parameters per symbol
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "monarch_hip.h")).read(), flags=re.S)
+    c_counts = _param_counts(header, r"\b(mhip_[a-z0-9_]+)\s*\(([^()]*)\)\s*;")
+    rust = open(os.path.join(ROOT, "hip-sys", "src", "lib.rs")).read()
+    rust_counts = _param_counts(rust, r"pub fn (mhip_[a-z0-9_]+)\(([^()]*)\)")
+    assert set(c_counts) == set(_lib.SIGNATURES) == set(rust_counts)
+    for name, n in c_counts.items():
+        assert len(_lib.SIGNATURES[name][1]) == n, (name, "ctypes", len(_lib.SIGNATURES[name][1]), n)
+        assert rust_counts[name] == n, (name, "rust", rust_counts[name], n)
+
+
 def test_product_never_touches_the_oracle_and_fails_loudly_without_the_library(monkeypatch, tmp_path):
     import monarch_amd
     pkg = os.path.dirname(monarch_amd.__file__)
