@@ -380,6 +380,21 @@ def test_transpose_large_square():
     assert torch.equal(back.view(torch.int16), x.view(torch.int16))
 
 
+def test_transpose_large_aligned_fp32_tiles():
+    # 2^25 four-byte elements with 512-byte aligned rows on both sides: the 128 x 128 tile form, with a batch dimension
+    g = torch.Generator(device=DEV).manual_seed(14)
+    x = torch.randn(2, 4096, 4096, generator=g, device=DEV)
+    view = x.transpose(1, 2)
+    s = Slice.of_tensor(view)
+    out = staging.pack(view, s)
+    sync()
+    assert torch.equal(out.view(2, 4096, 4096), view.contiguous())
+    back = torch.zeros_like(x)
+    staging.unpack(back, s, out)
+    sync()
+    assert torch.equal(back, x)
+
+
 def test_stream_send_tensor_semantics():
     from monarch_amd.reduce import Factory
     from monarch_amd.send_tensor import route, stream_send_tensor
