@@ -33,8 +33,8 @@ MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled 
     "c2p_unpack": 100_663_241, "c3_pack": 234_978_355, "c3_unpack": 234_963_309, "c4": 603_968_237,
     "c4_slots": 603_969_709, "c5_flat_pack": 3_166_564_842, "c5_quantize": 2_366_058_518,
     "c5_dequant": 7_129_890_652, "c5_flat_unpack": 6_016_924_093, "c5_dequant_many8": 12_782_544_690,
-    "c5_quantize_bucket": 2_374_780_329, "c5_dequant_bucket": 7_177_730_135, "tr_f32_pack": 536_910_860,
-    "tr_f32_unpack": 536_918_970, "tr_bf16_pack": 268_493_000,
+    "c5_quantize_bucket": 2_374_780_329, "c5_dequant_bucket": 7_177_730_135, "tr_f32_pack": 536_910_825,
+    "tr_f32_unpack": 536_919_994, "tr_bf16_pack": 268_493_000,
 }
 
 

@@ -225,6 +225,14 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
     const int v16 = threadIdx.x % G;  // which 16-byte vector of a row
     const int r16 = threadIdx.x / G;  // which row of a pass of ROWS rows
     constexpr int ROWS = THREADS / G;
+    // The side whose vectors run along q: lane -> (vector qv of the column, column cc of pass p).  With 16
+    // vectors per column a wavefront takes 16 vectors of 4 neighbouring columns, which is what makes its 64
+    // scalar LDS accesses fall into 64 banks.  With 32 vectors per column (512-byte rows) the same shape is
+    // kept - 16 vectors x 4 columns per wavefront, the two halves of a column going to neighbouring
+    // wavefronts - instead of 32 vectors x 2 columns, which would fold onto half of the banks.
+    const int qv = G == 16 ? v16 : (threadIdx.x % 16) + 16 * ((threadIdx.x / 64) % 2);
+    const int cc0 = G == 16 ? r16 : 4 * (threadIdx.x / 128) + (threadIdx.x % 64) / 16;
+    constexpr int CSTEP = G == 16 ? ROWS : 4 * (THREADS / 128);  // columns per pass
     if (full) {
         constexpr int PASSES = TQ / ROWS;
         Vec d[PASSES];
@@ -262,11 +270,11 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
             } else {
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
-                    const int cc = r16 + ROWS * p;
+                    const int cc = cc0 + CSTEP * p;
                     Vec o;
 #pragma unroll
-                    for (int j = 0; j < E; ++j) o.e[j] = tile[at(v16 * E + j, cc)];
-                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E) = o.v;
+                    for (int j = 0; j < E; ++j) o.e[j] = tile[at(qv * E + j, cc)];
+                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + qv * E) = o.v;
                 }
             }
         } else {
@@ -294,14 +302,14 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
             } else {
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
-                    const int cc = r16 + ROWS * p;
-                    d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + v16 * E);
+                    const int cc = cc0 + CSTEP * p;
+                    d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + qv * E);
                 }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
-                    const int cc = r16 + ROWS * p;
+                    const int cc = cc0 + CSTEP * p;
 #pragma unroll
-                    for (int j = 0; j < E; ++j) tile[at(v16 * E + j, cc)] = d[p].e[j];
+                    for (int j = 0; j < E; ++j) tile[at(qv * E + j, cc)] = d[p].e[j];
                 }
             }
             __syncthreads();
