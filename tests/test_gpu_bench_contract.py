@@ -1,0 +1,40 @@
+"""bench.py prints one JSON line with the fields the driver reads, and refuses more than one GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
+
+
+@pytest.mark.gpu
+def test_default_bench_line():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--steps", "10", "--warmup", "3"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [ln for ln in r.stdout.splitlines() if ln.startswith("{")]
+    assert len(lines) == 1
+    rec = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
+        assert key in rec, key
+    assert rec["n_gpus"] == 1 and rec["steps"] == 10 and rec["warmup"] == 3 and rec["vs_baseline"] is None
+    assert rec["unit"] == "GB/s" and rec["higher_is_better"] is True and rec["data"] == "synthetic"
+    assert rec["config"]["workload"] == "c2_bf16_bucket_reduce_avg8" and "model" not in rec["config"]
+    roof = rec["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-9 and 0.3 < roof["frac"] < 1.0
+    assert abs(rec["config"]["algorithmic_bytes_per_step"] - 9 * 25_165_824 * 2) == 0
+    assert 0.9 < roof["traffic"] / rec["config"]["algorithmic_bytes_per_step"] < 1.1
+    cpu = rec["cpu_baseline"]
+    assert cpu["kind"] in ("port", "reference") and cpu["cores"] == 1 and cpu["unit"] == "GB/s" and cpu["value"] > 0
+    assert cpu["sample"] and cpu["all_cores"]["cores"] >= 1
+    # wall-clock throughput cannot exceed the kernel-time throughput by more than timer noise
+    assert rec["value"] <= roof["achieved"] * 1.02
