@@ -148,6 +148,25 @@ def test_runs_shorter_than_a_chunk(elem_size):
             _roundtrip(s, elem_size, seed=40 + i, misalign=(i % 2) * elem_size, dst_misalign=dst_misalign)
 
 
+def test_maximum_number_of_dimensions():
+    # 32 dimensions (the library's limit): fourteen of size 2 that cannot merge, the rest of size 1
+    sizes, strides, acc = [], [], 1
+    for k in range(32):
+        if k % 2 == 0 and len([z for z in sizes if z == 2]) < 14:
+            sizes.append(2)
+            strides.append(acc)
+            acc *= 3
+        else:
+            sizes.append(1)
+            strides.append(acc)
+    s = Slice(offset=2, sizes=list(reversed(sizes)), strides=list(reversed(strides)))
+    assert s.ndim == 32 and len(s) == 2**14
+    _roundtrip(s, 2, seed=8)
+    _roundtrip(s, 16, seed=9)
+    with pytest.raises(ValueError, match="InvalidArgument"):
+        Slice(offset=0, sizes=[1] * 33, strides=[1] * 33)
+
+
 def test_many_dims_peels_on_host():
     # 10 dims that cannot merge (every stride leaves a gap): more than the kernel decodes at once
     sizes = [2] * 10
