@@ -20,6 +20,9 @@
 namespace mhip {
 
 constexpr int kMaxViews = 16;
+// Lanes per workgroup of the slice copy kernels: single wavefronts stream best (column-block pack 0.767 -> 0.775 of
+// peak, unpack 0.757 -> 0.792 against 256 lanes; ragged and short-run forms equal or better).
+constexpr int kPackThreads = 64;
 // Chunks per lane of slice_copy_kernel, all loads issued before the first store.  Large copies stream
 // fastest with one chunk per lane and many workgroups (8 column blocks of 14 MiB: 0.76 of peak against
 // 0.73 with eight chunks); copies of a few MiB finish sooner with fewer, fatter workgroups.
@@ -63,7 +66,7 @@ __device__ __forceinline__ void move_chunk_by_units(const PackArgs& a, char* str
 }
 
 template <int U, bool PACK, bool WIDE, int NDIM, int kUnroll>
-__global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
+__global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     constexpr int VU = 16 / U;  // units per chunk
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
@@ -72,26 +75,26 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     const uint32_t v = blockIdx.x % a.nviews;
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
-    const uint64_t c0 = tile * (kThreads * kUnroll) + threadIdx.x;
+    const uint64_t c0 = tile * (kPackThreads * kUnroll) + threadIdx.x;
 
     if constexpr (NDIM == 0) {
         // Contiguous view: when the whole 32 KiB tile of this workgroup lies inside the
         // buffer (decided on the scalar unit), no per-chunk tests are needed at all.
-        const uint64_t tile_first = tile * (kThreads * kUnroll) * VU;
-        const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
+        const uint64_t tile_first = tile * (kPackThreads * kUnroll) * VU;
+        const uint64_t tile_end = tile_first + (uint64_t)(kPackThreads * kUnroll) * VU;
         if (tile_first >= a.shift && tile_end - a.shift <= a.total) {
             char* __restrict__ p = packed + (c0 * VU - a.shift) * U;
             char* __restrict__ s = strided + (c0 * VU - a.shift) * U;
             uint4 d[kUnroll];
 #pragma unroll
             for (int i = 0; i < kUnroll; ++i) {
-                if constexpr (PACK) d[i] = load16_unaligned(s + (size_t)i * kThreads * 16);
-                else d[i] = load16_aligned(p + (size_t)i * kThreads * 16);
+                if constexpr (PACK) d[i] = load16_unaligned(s + (size_t)i * kPackThreads * 16);
+                else d[i] = load16_aligned(p + (size_t)i * kPackThreads * 16);
             }
 #pragma unroll
             for (int i = 0; i < kUnroll; ++i) {
-                if constexpr (PACK) store16_aligned(p + (size_t)i * kThreads * 16, d[i]);
-                else store16_unaligned(s + (size_t)i * kThreads * 16, d[i]);
+                if constexpr (PACK) store16_aligned(p + (size_t)i * kPackThreads * 16, d[i]);
+                else store16_unaligned(s + (size_t)i * kPackThreads * 16, d[i]);
             }
             return;
         }
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     bool live[kUnroll];
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
-        const uint64_t c = c0 + (uint64_t)i * kThreads;
+        const uint64_t c = c0 + (uint64_t)i * kPackThreads;
         live[i] = c < a.nchunks;
         const uint64_t tb = c * VU;  // position counted from the aligned-down start
         vec[i] = false;
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
     if constexpr (VU > 1) {
 #pragma unroll
         for (int i = 0; i < kUnroll; ++i) {
-            if (live[i] && !vec[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kThreads);
+            if (live[i] && !vec[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kPackThreads);
         }
     }
 }
@@ -175,19 +178,19 @@ __global__ __launch_bounds__(kThreads) void slice_copy_kernel(PackArgs a) {
 constexpr int kRaggedUnroll = 1;  // measured: 1 chunk per lane 0.75, 2 0.73, 4 0.72, 8 0.72 of peak (fp32 rows of 1791)
 
 template <int U, bool PACK, bool WIDE, int NDIM>
-__global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a) {
+__global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArgs a) {
     constexpr int VU = 16 / U;
     constexpr int UN = kRaggedUnroll;
     const uint64_t tile = blockIdx.x / a.nviews;
     const uint32_t v = blockIdx.x % a.nviews;
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
-    const uint64_t c0 = tile * (kThreads * UN) + threadIdx.x;
+    const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
     uint64_t pa[UN], sa[UN], pb[UN], sb[UN];  // packed / strided unit index of vector A and vector B
     bool do_a[UN], do_b[UN], edge[UN];
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        const uint64_t c = c0 + (uint64_t)i * kThreads;
+        const uint64_t c = c0 + (uint64_t)i * kPackThreads;
         const uint64_t tb = c * VU;
         const uint64_t first = tb - a.shift;
         pa[i] = sa[i] = pb[i] = sb[i] = 0;
@@ -234,7 +237,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a)
     }
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kThreads);
+        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, strided, packed, c0 + (uint64_t)i * kPackThreads);
     }
 }
 
@@ -249,7 +252,7 @@ __global__ __launch_bounds__(kThreads) void slice_copy_ragged_kernel(PackArgs a)
 constexpr int kGatherUnroll = 1;
 
 template <int U, bool PACK, bool WIDE, int NDIM>
-__global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
+__global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) {
     using T = typename UnitType<U>::type;
     constexpr int VU = 16 / U;
     constexpr int UN = kGatherUnroll;
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
     const uint32_t v = blockIdx.x % a.nviews;
     char* __restrict__ packed = a.packed[v];
     T* __restrict__ strided = reinterpret_cast<T*>(a.base) + a.offset[v];
-    const uint64_t c0 = tile * (kThreads * UN) + threadIdx.x;
+    const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
     const int nd = NDIM >= 0 ? NDIM : a.dims.ndim;
     const uint64_t run = a.dims.run;
     const uint64_t size_last = a.dims.size[nd - 1];
@@ -268,7 +271,7 @@ __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
     bool full[UN], edge[UN];
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        const uint64_t c = c0 + (uint64_t)i * kThreads;
+        const uint64_t c = c0 + (uint64_t)i * kPackThreads;
         const uint64_t tb = c * VU;
         const uint64_t first = tb - a.shift;
         full[i] = c < a.nchunks && tb >= a.shift && first + VU <= a.total;
@@ -318,11 +321,11 @@ __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
             for (int j = 0; j < VU; ++j) d[i].e[j] = strided[off[i][j]];
 #pragma unroll
         for (int i = 0; i < UN; ++i)
-            if (full[i]) store16_aligned(packed + ((c0 + (uint64_t)i * kThreads) * VU - a.shift) * U, d[i].v);
+            if (full[i]) store16_aligned(packed + ((c0 + (uint64_t)i * kPackThreads) * VU - a.shift) * U, d[i].v);
     } else {
 #pragma unroll
         for (int i = 0; i < UN; ++i) {
-            const uint64_t first = (c0 + (uint64_t)i * kThreads) * VU - a.shift;
+            const uint64_t first = (c0 + (uint64_t)i * kPackThreads) * VU - a.shift;
             d[i].v = load16_aligned(packed + (full[i] ? first : safe_first) * U);
         }
 #pragma unroll
@@ -335,17 +338,20 @@ __global__ __launch_bounds__(kThreads) void slice_gather_kernel(PackArgs a) {
     // ragged first and last chunk of the view: unit by unit
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
-        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, reinterpret_cast<char*>(strided), packed, c0 + (uint64_t)i * kThreads);
+        if (edge[i]) move_chunk_by_units<U, PACK, WIDE, NDIM>(a, reinterpret_cast<char*>(strided), packed, c0 + (uint64_t)i * kPackThreads);
     }
 }
 
 // Plain contiguous copy of 16-byte units, both sides 16-byte aligned (a contiguous view, the
 // "transfer" of a staging buffer): one chunk per lane, non-temporal load, write-through
 // store.  For a 50/50 read/write stream this shape beats the 8-deep tile above by ~5%
-// (16.6 vs 17.4 us for 48 MiB).
-__global__ __launch_bounds__(kThreads) void contiguous_copy_kernel(char* __restrict__ dst, const char* __restrict__ src,
-                                                                   uint64_t nchunks) {
-    const uint64_t c = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+// (16.6 vs 17.4 us for 48 MiB), and single-wavefront workgroups beat larger ones (48 MiB:
+// 64 lanes 15.9-16.4 us, 128 lanes 16.7-17.1, 256 lanes 16.6-16.9, 1024 lanes 16.5).
+constexpr int kCopyThreads = 64;
+
+__global__ __launch_bounds__(kCopyThreads) void contiguous_copy_kernel(char* __restrict__ dst, const char* __restrict__ src,
+                                                                       uint64_t nchunks) {
+    const uint64_t c = (uint64_t)blockIdx.x * kCopyThreads + threadIdx.x;
     if (c < nchunks) store16_writethrough(dst + c * 16, load16_aligned(src + c * 16));
 }
 
@@ -364,9 +370,9 @@ struct ShiftCopyArgs {
 };
 
 template <int ROWS>
-__global__ __launch_bounds__(kThreads) void contiguous_copy_shift_kernel(ShiftCopyArgs a) {
+__global__ __launch_bounds__(kPackThreads) void contiguous_copy_shift_kernel(ShiftCopyArgs a) {
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t wave = (uint64_t)blockIdx.x * (kPackThreads / 64) + (threadIdx.x >> 6);
     char* __restrict__ dst = a.dst + a.head;            // 16-byte aligned
     const char* src = a.src + a.head;
     const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
@@ -393,8 +399,8 @@ __global__ __launch_bounds__(kThreads) void contiguous_copy_shift_kernel(ShiftCo
         }
     }
     if (blockIdx.x == 0) {
-        for (uint64_t i = threadIdx.x; i < a.head; i += kThreads) a.dst[i] = a.src[i];
-        for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kThreads) a.dst[i] = a.src[i];
+        for (uint64_t i = threadIdx.x; i < a.head; i += kPackThreads) a.dst[i] = a.src[i];
+        for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kPackThreads) a.dst[i] = a.src[i];
     }
 }
 
@@ -414,10 +420,10 @@ static bool launch_shift_copy(char* dst, const char* src, uint64_t nbytes, hipSt
     }
     if (nvec == 0) return false;
     ShiftCopyArgs a{dst, src, nbytes, head, nvec};
-    const uint64_t per_wg = (uint64_t)(kThreads / 64) * kShiftCopyRows * 64;
+    const uint64_t per_wg = (uint64_t)(kPackThreads / 64) * kShiftCopyRows * 64;
     const uint64_t wgs = (nvec + per_wg - 1) / per_wg;
     if (wgs > 0x7fffffffull) return false;
-    hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3((uint32_t)wgs), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3((uint32_t)wgs), dim3(kPackThreads), 0, stream, a);
     *rc = launch_status();
     return true;
 }
@@ -437,17 +443,19 @@ struct FlatArgs {
 
 // Chunks per lane: 4 when gathering tensors into the flat buffer (0.74 of peak; 8 -> 0.71, 2 -> 0.69),
 // 2 when scattering the flat buffer back (0.72; 8 -> 0.66, 1 -> 0.58).
+// Lanes per workgroup: 256 (0.765 / 0.725 of peak gathering / scattering a bucket; 128 -> 0.744 / 0.708, 64 -> 0.755 / 0.715).
+constexpr int kFlatThreads = kThreads;
 template <bool PACK> struct FlatUnroll { static constexpr int value = PACK ? 4 : 2; };
 
 template <int U, bool PACK>
-__global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
+__global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
     constexpr int VU = 16 / U;
     constexpr int kUnroll = FlatUnroll<PACK>::value;
     __shared__ uint32_t s_range[2];
-    const uint64_t block_c0 = (uint64_t)blockIdx.x * (kThreads * kUnroll);
+    const uint64_t block_c0 = (uint64_t)blockIdx.x * (kFlatThreads * kUnroll);
     if (threadIdx.x < 64) {
         // wavefront 0 finds the tensors holding the first and the last unit this block touches
-        uint64_t c_last = block_c0 + kThreads * kUnroll - 1;
+        uint64_t c_last = block_c0 + kFlatThreads * kUnroll - 1;
         if (c_last >= a.nchunks) c_last = a.nchunks - 1;
         const uint64_t tb_first = block_c0 * VU, tb_last = c_last * VU + VU - 1;
         uint64_t u_first = tb_first >= a.shift ? tb_first - a.shift : 0;
@@ -469,7 +477,7 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
         // Workgroup-uniform fast path: the whole 32 KiB tile lies inside one tensor (most of a
         // bucket's bytes are in tensors much larger than a tile) and inside the flat buffer.
         const uint64_t tile_first = block_c0 * VU;
-        const uint64_t tile_end = tile_first + (uint64_t)(kThreads * kUnroll) * VU;
+        const uint64_t tile_end = tile_first + (uint64_t)(kFlatThreads * kUnroll) * VU;
         if (s_range[0] == s_range[1] && tile_first >= a.shift && tile_end - a.shift <= a.total) {
             if constexpr (PACK) {
                 // Gathering: the tensor side is the one that is read.  Each wavefront takes kUnroll consecutive
@@ -503,13 +511,13 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
             uint4 d[kUnroll];
 #pragma unroll
             for (int i = 0; i < kUnroll; ++i) {
-                if constexpr (PACK) d[i] = load16_unaligned(t + (size_t)i * kThreads * 16);
-                else d[i] = load16_aligned(f + (size_t)i * kThreads * 16);
+                if constexpr (PACK) d[i] = load16_unaligned(t + (size_t)i * kFlatThreads * 16);
+                else d[i] = load16_aligned(f + (size_t)i * kFlatThreads * 16);
             }
 #pragma unroll
             for (int i = 0; i < kUnroll; ++i) {
-                if constexpr (PACK) store16_aligned(f + (size_t)i * kThreads * 16, d[i]);
-                else store16_unaligned(t + (size_t)i * kThreads * 16, d[i]);
+                if constexpr (PACK) store16_aligned(f + (size_t)i * kFlatThreads * 16, d[i]);
+                else store16_unaligned(t + (size_t)i * kFlatThreads * 16, d[i]);
             }
             return;
         }
@@ -522,7 +530,7 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     bool all_vec = true;
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
-        const uint64_t c = block_c0 + (uint64_t)i * kThreads + threadIdx.x;
+        const uint64_t c = block_c0 + (uint64_t)i * kFlatThreads + threadIdx.x;
         const uint64_t tb = c * VU;
         const uint64_t first = tb - a.shift;
         vec[i] = false;
@@ -550,7 +558,7 @@ __global__ __launch_bounds__(kThreads) void flat_copy_kernel(FlatArgs a) {
     }
 #pragma unroll
     for (int i = 0; i < kUnroll; ++i) {
-        const uint64_t c = block_c0 + (uint64_t)i * kThreads + threadIdx.x;
+        const uint64_t c = block_c0 + (uint64_t)i * kFlatThreads + threadIdx.x;
         if (c >= a.nchunks) continue;
         if (vec[i]) {
             if constexpr (PACK) store16_aligned(fptr[i], load16_unaligned(tptr[i]));
@@ -577,7 +585,7 @@ enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns };
 
 template <int U, bool PACK, int UNROLL>
 static void launch_whole_chunks_u(bool wide, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
-    const dim3 block(kThreads);
+    const dim3 block(kPackThreads);
     if (wide) {
         hipLaunchKernelGGL((slice_copy_kernel<U, PACK, true, -1, UNROLL>), grid, block, 0, stream, a);
         return;
@@ -598,7 +606,7 @@ static void launch_whole_chunks(bool wide, bool large, int ndim, dim3 grid, hipS
 
 template <int U, bool PACK>
 static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
-    const dim3 block(kThreads);
+    const dim3 block(kPackThreads);
     if constexpr (U < 16) {
         if (form == kShortRuns) {
             if (wide) {
@@ -670,12 +678,12 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             ++k;
             continue;
         }
-        if (first.ndim == 0 && unit == 16 && (first.total + kThreads - 1) / kThreads <= 0x7fffffffull) {
+        if (first.ndim == 0 && unit == 16 && (first.total + kCopyThreads - 1) / kCopyThreads <= 0x7fffffffull) {
             char* strided = base + first.offset * 16;
             char* dst = PACK ? packed[k] : strided;
             const char* src = PACK ? strided : packed[k];
-            hipLaunchKernelGGL(contiguous_copy_kernel, dim3((uint32_t)((first.total + kThreads - 1) / kThreads)),
-                               dim3(kThreads), 0, stream, dst, src, first.total);
+            hipLaunchKernelGGL(contiguous_copy_kernel, dim3((uint32_t)((first.total + kCopyThreads - 1) / kCopyThreads)),
+                               dim3(kCopyThreads), 0, stream, dst, src, first.total);
             if (int rc = launch_status()) return rc;
             ++k;
             continue;
@@ -739,7 +747,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             else if (first.run >= vu) form = kRaggedRows;
         }
         const bool large = a.nchunks >= kLargeCopyChunks;
-        const uint64_t per_block = (uint64_t)kThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
+        const uint64_t per_block = (uint64_t)kPackThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
         if (blocks * nbatch > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
         a.nviews = nbatch;
@@ -787,18 +795,18 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
     a.shift = (uint32_t)(((uintptr_t)flat & 15u) / unit);
     const uint32_t vu = 16 / unit;
     a.nchunks = (a.total + a.shift + vu - 1) / vu;
-    const uint64_t per_block = (uint64_t)kThreads * FlatUnroll<PACK>::value;
+    const uint64_t per_block = (uint64_t)kFlatThreads * FlatUnroll<PACK>::value;
     const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
     if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     dim3 grid((uint32_t)blocks);
     switch (unit) {
-        case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, dim3(kThreads), 0, hs, a); break;
-        case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, dim3(kThreads), 0, hs, a); break;
-        case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, dim3(kThreads), 0, hs, a); break;
-        case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, dim3(kThreads), 0, hs, a); break;
-        default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, dim3(kThreads), 0, hs, a); break;
+        case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
+        case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
+        case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
+        case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
+        default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
     }
     return launch_status();
 }
