@@ -34,13 +34,14 @@ __device__ __noinline__ void quantize_block_careful(uint8_t* __restrict__ q, flo
 // the 756 M-element bucket: 1 block 0.81 of peak, 2 blocks 0.79, 4 blocks 0.78 - more, smaller wavefront
 // steps stream better than deeper ones here, as in the copy and reduce kernels.
 constexpr int kQuantBlocks = 1;
+constexpr int kQuantThreads = 64;  // single-wavefront workgroups: 0.825 of peak against 0.81 with 256 lanes
 
-__global__ __launch_bounds__(kThreads) void fp8_quantize_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
+__global__ __launch_bounds__(kQuantThreads) void fp8_quantize_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                 const uint16_t* __restrict__ x, uint64_t numel,
                                                                 uint64_t nblocks) {
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
-    const uint64_t nwaves = (uint64_t)gridDim.x * (kThreads / 64);
+    const uint64_t wave = (uint64_t)blockIdx.x * (kQuantThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t nwaves = (uint64_t)gridDim.x * (kQuantThreads / 64);
     for (uint64_t b0 = wave * kQuantBlocks; b0 < nblocks; b0 += nwaves * kQuantBlocks) {
         uint4 lo[kQuantBlocks], hi[kQuantBlocks];
         bool full[kQuantBlocks];
@@ -95,63 +96,38 @@ __global__ __launch_bounds__(kThreads) void fp8_quantize_kernel(uint8_t* __restr
     }
 }
 
-// acc[i] += float(q[i]) * scale[i / 1024].  A workgroup step covers 1024 consecutive
-// elements starting at a multiple of 1024, i.e. exactly one block.
-constexpr int kDeqSteps = 1;  // blocks per workgroup: 1 -> 0.81 of peak, 2 -> 0.77, 4 -> 0.78
+// acc[i] += float(q[i]) * scale[i / 1024].  A workgroup covers kDeqThreads * 4 consecutive
+// elements (a whole fraction of one block), four per lane: one 32-bit load of codes and one
+// 128-bit load / store of the accumulator.
+constexpr int kDeqThreads = 64;
+constexpr int kDeqTile = kDeqThreads * 4;  // elements per workgroup
+static_assert(kBlock % kDeqTile == 0, "a tile lies inside one block");
 
-__global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float* __restrict__ acc,
-                                                                          const uint8_t* __restrict__ q,
-                                                                          const float* __restrict__ scales,
-                                                                          uint64_t numel, uint64_t ntiles) {
+__global__ __launch_bounds__(kDeqThreads) void fp8_dequant_accumulate_kernel(float* __restrict__ acc,
+                                                                             const uint8_t* __restrict__ q,
+                                                                             const float* __restrict__ scales,
+                                                                             uint64_t numel, uint64_t ntiles) {
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const uint64_t b0 = tile * kDeqSteps;
-        const uint64_t i0 = b0 * kBlock + threadIdx.x * 4;
-        uint32_t codes[kDeqSteps];
-        uint4 a[kDeqSteps];
-        float s[kDeqSteps];
-        if ((b0 + kDeqSteps) * kBlock <= numel) {
-            // interior tile (workgroup-uniform): no per-step predicates, all loads first
-#pragma unroll
-            for (int j = 0; j < kDeqSteps; ++j) {
-                codes[j] = load4_unaligned(q + i0 + j * kBlock);
-                a[j] = load16_unaligned(acc + i0 + j * kBlock);
-                s[j] = scales[b0 + j];
-            }
-#pragma unroll
-            for (int j = 0; j < kDeqSteps; ++j) {
-                const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], false);
-                const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], true);
-                // product rounded to fp32, then added: two roundings (contraction is off)
-                uint4 r;
-                r.x = __float_as_uint(__uint_as_float(a[j].x) + p01[0] * s[j]);
-                r.y = __float_as_uint(__uint_as_float(a[j].y) + p01[1] * s[j]);
-                r.z = __float_as_uint(__uint_as_float(a[j].z) + p23[0] * s[j]);
-                r.w = __float_as_uint(__uint_as_float(a[j].w) + p23[1] * s[j]);
-                store16_unaligned(acc + i0 + j * kBlock, r);
-            }
+        const uint64_t i0 = tile * kDeqTile + threadIdx.x * 4;
+        if ((tile + 1) * kDeqTile <= numel) {  // interior tile (workgroup-uniform)
+            const uint32_t c = load4_unaligned(q + i0);
+            const uint4 v = load16_unaligned(acc + i0);
+            const float sc = scales[tile * kDeqTile / kBlock];
+            const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, false);
+            const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, true);
+            // product rounded to fp32, then added: two roundings (contraction is off)
+            uint4 r;
+            r.x = __float_as_uint(__uint_as_float(v.x) + p01[0] * sc);
+            r.y = __float_as_uint(__uint_as_float(v.y) + p01[1] * sc);
+            r.z = __float_as_uint(__uint_as_float(v.z) + p23[0] * sc);
+            r.w = __float_as_uint(__uint_as_float(v.w) + p23[1] * sc);
+            store16_unaligned(acc + i0, r);
             continue;
         }
-        // last tile: per-step bounds, single elements at the ragged end
-        for (int j = 0; j < kDeqSteps; ++j) {
-            const uint64_t i = i0 + (uint64_t)j * kBlock;
-            if (i + 4 <= numel) {
-                const uint32_t c = load4_unaligned(q + i);
-                const uint4 v = load16_unaligned(acc + i);
-                const float sc = scales[b0 + j];
-                const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, false);
-                const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, true);
-                uint4 r;
-                r.x = __float_as_uint(__uint_as_float(v.x) + p01[0] * sc);
-                r.y = __float_as_uint(__uint_as_float(v.y) + p01[1] * sc);
-                r.z = __float_as_uint(__uint_as_float(v.z) + p23[0] * sc);
-                r.w = __float_as_uint(__uint_as_float(v.w) + p23[1] * sc);
-                store16_unaligned(acc + i, r);
-            } else {
-                for (uint64_t e = i; e < numel && e < i + 4; ++e) {
-                    const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
-                    acc[e] = acc[e] + p[0] * scales[e / kBlock];
-                }
-            }
+        // last tile: single elements at the ragged end
+        for (uint64_t e = i0; e < numel && e < i0 + 4; ++e) {
+            const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
+            acc[e] = acc[e] + p[0] * scales[e / kBlock];
         }
     }
 }
@@ -161,8 +137,6 @@ __global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_kernel(float*
 // accumulator crosses HBM once instead of n times (n + 8 bytes per element instead of 9n;
 // n + 4 when `overwrite` starts from zero instead of reading acc).
 constexpr int kMaxPeers = 64;
-constexpr int kManySteps = 1;  // blocks per workgroup: 1 -> 0.80 of peak with 8 peers, 2 -> 0.77
-
 struct DequantManyArgs {
     float* acc;
     const uint8_t* q[kMaxPeers];
@@ -173,70 +147,73 @@ struct DequantManyArgs {
     uint32_t overwrite;
 };
 
-template <int N>  // N > 0: peers known at compile time; N == 0: a.n peers, eight at a time
-__global__ __launch_bounds__(kThreads) void fp8_dequant_accumulate_many_kernel(DequantManyArgs a) {
+// N > 0: peers known at compile time; N == 0: a.n peers, eight at a time.  THREADS lanes cover THREADS * 4
+// elements: single wavefronts are best when the accumulator is read (8 peers: 0.805 of peak against 0.80),
+// 256 lanes when it is only written (0.82 against 0.78).
+template <int N, int THREADS>
+__global__ __launch_bounds__(THREADS) void fp8_dequant_accumulate_many_kernel(DequantManyArgs a) {
+    constexpr int TILE = THREADS * 4;
+    static_assert(kBlock % TILE == 0, "a tile lies inside one block");
     float* __restrict__ acc = a.acc;
     const uint32_t n = N > 0 ? N : a.n;
     for (uint64_t tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
-        const uint64_t b0 = tile * kManySteps;
-        const uint64_t i0 = b0 * kBlock + threadIdx.x * 4;
-        if ((b0 + kManySteps) * kBlock <= a.numel) {  // interior tile, workgroup-uniform
-            float v[kManySteps][4];
-#pragma unroll
-            for (int j = 0; j < kManySteps; ++j) {
-                if (a.overwrite) {
-                    v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.0f;
-                } else {
-                    const uint4 r = load16_unaligned(acc + i0 + j * kBlock);
-                    v[j][0] = __uint_as_float(r.x); v[j][1] = __uint_as_float(r.y);
-                    v[j][2] = __uint_as_float(r.z); v[j][3] = __uint_as_float(r.w);
-                }
+        const uint64_t i0 = tile * TILE + threadIdx.x * 4;
+        if ((tile + 1) * TILE <= a.numel) {  // interior tile, workgroup-uniform
+            const uint64_t b = tile * TILE / kBlock;
+            float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (!a.overwrite) {
+                const uint4 r = load16_unaligned(acc + i0);
+                v[0] = __uint_as_float(r.x); v[1] = __uint_as_float(r.y);
+                v[2] = __uint_as_float(r.z); v[3] = __uint_as_float(r.w);
             }
             for (uint32_t r0 = 0; r0 < n; r0 += 8) {
                 constexpr int G = N > 0 && N < 8 ? N : 8;
-                uint32_t codes[kManySteps][G];
-                float s[kManySteps][G];
+                uint32_t codes[G];
+                float s[G];
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     const uint32_t r = r0 + g < n ? r0 + g : n - 1;  // clamped: the extra loads of a short last group are unused
-#pragma unroll
-                    for (int j = 0; j < kManySteps; ++j) {
-                        codes[j][g] = load4_unaligned(a.q[r] + i0 + j * kBlock);
-                        s[j][g] = a.scales[r][b0 + j];
-                    }
+                    codes[g] = load4_unaligned(a.q[r] + i0);
+                    s[g] = a.scales[r][b];
                 }
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     if (r0 + g < n) {
-#pragma unroll
-                        for (int j = 0; j < kManySteps; ++j) {
-                            const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j][g], false);
-                            const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j][g], true);
-                            v[j][0] = v[j][0] + p01[0] * s[j][g];
-                            v[j][1] = v[j][1] + p01[1] * s[j][g];
-                            v[j][2] = v[j][2] + p23[0] * s[j][g];
-                            v[j][3] = v[j][3] + p23[1] * s[j][g];
-                        }
+                        const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g], false);
+                        const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g], true);
+                        v[0] = v[0] + p01[0] * s[g];
+                        v[1] = v[1] + p01[1] * s[g];
+                        v[2] = v[2] + p23[0] * s[g];
+                        v[3] = v[3] + p23[1] * s[g];
                     }
                 }
             }
-#pragma unroll
-            for (int j = 0; j < kManySteps; ++j)
-                store16_unaligned(acc + i0 + j * kBlock, make_uint4(__float_as_uint(v[j][0]), __float_as_uint(v[j][1]),
-                                                                     __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
+            store16_unaligned(acc + i0, make_uint4(__float_as_uint(v[0]), __float_as_uint(v[1]),
+                                                   __float_as_uint(v[2]), __float_as_uint(v[3])));
             continue;
         }
         // last tile: element by element
-        for (int j = 0; j < kManySteps; ++j) {
-            for (uint64_t e = i0 + (uint64_t)j * kBlock; e < a.numel && e < i0 + (uint64_t)j * kBlock + 4; ++e) {
-                float x = a.overwrite ? 0.0f : acc[e];
-                for (uint32_t r = 0; r < n; ++r) {
-                    const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)a.q[r][e], false);
-                    x = x + p[0] * a.scales[r][e / kBlock];
-                }
-                acc[e] = x;
+        for (uint64_t e = i0; e < a.numel && e < i0 + 4; ++e) {
+            float x = a.overwrite ? 0.0f : acc[e];
+            for (uint32_t r = 0; r < n; ++r) {
+                const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)a.q[r][e], false);
+                x = x + p[0] * a.scales[r][e / kBlock];
             }
+            acc[e] = x;
         }
+    }
+}
+
+template <int THREADS>
+static void launch_dequant_many(DequantManyArgs& a, hipStream_t hs) {
+    a.ntiles = (a.numel + THREADS * 4 - 1) / (THREADS * 4);
+    const uint64_t cap = 0x7fffffffull;
+    const dim3 grid((uint32_t)(a.ntiles > cap ? cap : a.ntiles)), blockdim(THREADS);
+    switch (a.n) {
+        case 2: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<2, THREADS>), grid, blockdim, 0, hs, a); break;
+        case 4: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<4, THREADS>), grid, blockdim, 0, hs, a); break;
+        case 8: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<8, THREADS>), grid, blockdim, 0, hs, a); break;
+        default: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<0, THREADS>), grid, blockdim, 0, hs, a); break;
     }
 }
 
@@ -253,12 +230,12 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
     if (!q || !scales || !x_bf16) return MHIP_ERR_UNDEFINED_TENSOR;
     if (((uintptr_t)x_bf16 & 1u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
     const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
-    const uint64_t per_wg = (kThreads / 64) * kQuantBlocks;
+    const uint64_t per_wg = (kQuantThreads / 64) * kQuantBlocks;
     const uint64_t wgs = (nblocks + per_wg - 1) / per_wg;
     const uint64_t cap = 0x7fffffffull;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads), 0, hs, q, scales,
+    hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kQuantThreads), 0, hs, q, scales,
                        static_cast<const uint16_t*>(x_bf16), numel, nblocks);
     return launch_status();
 }
@@ -269,12 +246,11 @@ int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scale
     if (numel == 0) return MHIP_SUCCESS;
     if (!acc || !q || !scales) return MHIP_ERR_UNDEFINED_TENSOR;
     if (((uintptr_t)acc & 3u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
-    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
-    const uint64_t ntiles = (nblocks + kDeqSteps - 1) / kDeqSteps;
+    const uint64_t ntiles = (numel + kDeqTile - 1) / kDeqTile;
     const uint64_t cap = 0x7fffffffull;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kThreads), 0,
+    hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kDeqThreads), 0,
                        hs, acc, q, scales, numel, ntiles);
     return launch_status();
 }
@@ -298,18 +274,10 @@ int mhip_fp8_dequant_accumulate_many(float* acc, const uint8_t* const* q, const 
     a.numel = numel;
     a.n = n;
     a.overwrite = overwrite ? 1u : 0u;
-    const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
-    a.ntiles = (nblocks + kManySteps - 1) / kManySteps;
-    const uint64_t cap = 0x7fffffffull;
-    const dim3 grid((uint32_t)(a.ntiles > cap ? cap : a.ntiles)), blockdim(kThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    switch (n) {
-        case 2: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<2>, grid, blockdim, 0, hs, a); break;
-        case 4: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<4>, grid, blockdim, 0, hs, a); break;
-        case 8: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<8>, grid, blockdim, 0, hs, a); break;
-        default: hipLaunchKernelGGL(fp8_dequant_accumulate_many_kernel<0>, grid, blockdim, 0, hs, a); break;
-    }
+    if (a.overwrite) launch_dequant_many<256>(a, hs);
+    else launch_dequant_many<kDeqThreads>(a, hs);
     return launch_status();
 }
 
