@@ -306,7 +306,7 @@ int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_ten
     a.ntensors = ntensors;
     const uint64_t per_wg = (kBucketThreads / 64) * kBucketBlocks;
     const uint64_t wgs = (a.nblocks + per_wg - 1) / per_wg;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_quantize_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0, hs, q,
@@ -328,7 +328,7 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
     a.nblocks = (total + kBlock - 1) / kBlock;
     a.ntensors = ntensors;
     const uint64_t wgs = (a.nblocks + 3) / 4;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0,
@@ -358,7 +358,7 @@ int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const ui
     p.b.nblocks = (total + kBlock - 1) / kBlock;
     p.b.ntensors = ntensors;
     const uint64_t wgs = (p.b.nblocks + 3) / 4;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_many_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads),

@@ -207,7 +207,7 @@ __global__ __launch_bounds__(THREADS) void fp8_dequant_accumulate_many_kernel(De
 template <int THREADS>
 static void launch_dequant_many(DequantManyArgs& a, hipStream_t hs) {
     a.ntiles = (a.numel + THREADS * 4 - 1) / (THREADS * 4);
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(THREADS);
     const dim3 grid((uint32_t)(a.ntiles > cap ? cap : a.ntiles)), blockdim(THREADS);
     switch (a.n) {
         case 2: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<2, THREADS>), grid, blockdim, 0, hs, a); break;
@@ -232,7 +232,7 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
     const uint64_t nblocks = (numel + kBlock - 1) / kBlock;
     const uint64_t per_wg = (kQuantThreads / 64) * kQuantBlocks;
     const uint64_t wgs = (nblocks + per_wg - 1) / per_wg;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kQuantThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kQuantThreads), 0, hs, q, scales,
@@ -247,7 +247,7 @@ int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scale
     if (!acc || !q || !scales) return MHIP_ERR_UNDEFINED_TENSOR;
     if (((uintptr_t)acc & 3u) || ((uintptr_t)scales & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
     const uint64_t ntiles = (numel + kDeqTile - 1) / kDeqTile;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kDeqThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kDeqThreads), 0,

@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "mhip_internal.h"
 
 namespace mhip {
@@ -225,9 +227,42 @@ private:
     bool restore_ = false;
 };
 
+// The runtime forms the global size of a launch (workgroups x lanes) in 32 bits.  A launch of exactly
+// 2^32 lanes is refused, and a larger one wraps silently: (2^26 + 1) workgroups of 64 lanes ran as ONE
+// workgroup and reported success.  Every host launch therefore keeps its grid at or below this bound;
+// grid-stride kernels clamp to it, one-shot kernels are launched in several pieces.
+// MONARCH_HIP_MAX_LAUNCH_LANES lowers the bound (a test aid: it drives small inputs through the
+// clamped and multi-piece paths).
+inline uint64_t max_launch_lanes() {
+    static const uint64_t limit = [] {
+        uint64_t v = 0xffffffffull;
+        if (const char* e = std::getenv("MONARCH_HIP_MAX_LAUNCH_LANES")) {
+            const unsigned long long x = std::strtoull(e, nullptr, 10);
+            if (x >= 8192 && x < v) v = x;
+        }
+        return v;
+    }();
+    return limit;
+}
+inline uint64_t max_workgroups(uint32_t lanes) { return max_launch_lanes() / lanes; }
+
 inline int launch_status() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? MHIP_SUCCESS : (int)e;
+}
+
+// Launches `wgs` workgroups of `lanes` lanes as one or more grids within the bound above:
+// launch(first_workgroup, count) enqueues one piece, whose kernel adds first_workgroup to blockIdx.x.
+// Pieces after the first start at a multiple of `multiple` workgroups.
+template <typename F>
+inline int launch_in_pieces(uint64_t wgs, uint32_t lanes, uint32_t multiple, F&& launch) {
+    const uint64_t most = max_workgroups(lanes) / multiple * multiple;
+    if (most == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    for (uint64_t first = 0; first < wgs; first += most) {
+        launch(first, (uint32_t)(wgs - first < most ? wgs - first : most));
+        if (int rc = launch_status()) return rc;
+    }
+    return MHIP_SUCCESS;
 }
 
 }  // namespace mhip

@@ -37,6 +37,7 @@ struct PackArgs {
     uint64_t nchunks;            // 16-byte chunks per view, including a ragged first one
     uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
     uint32_t nviews;             // views handled by this launch
+    uint64_t wg0;                // workgroups of this copy launched before this grid
     DimsArg dims;
 };
 
@@ -71,8 +72,9 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
-    const uint64_t tile = blockIdx.x / a.nviews;
-    const uint32_t v = blockIdx.x % a.nviews;
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile = wg / a.nviews;
+    const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = tile * (kPackThreads * kUnroll) + threadIdx.x;
@@ -181,8 +183,9 @@ template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArgs a) {
     constexpr int VU = 16 / U;
     constexpr int UN = kRaggedUnroll;
-    const uint64_t tile = blockIdx.x / a.nviews;
-    const uint32_t v = blockIdx.x % a.nviews;
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile = wg / a.nviews;
+    const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
@@ -256,8 +259,9 @@ __global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) 
     using T = typename UnitType<U>::type;
     constexpr int VU = 16 / U;
     constexpr int UN = kGatherUnroll;
-    const uint64_t tile = blockIdx.x / a.nviews;
-    const uint32_t v = blockIdx.x % a.nviews;
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile = wg / a.nviews;
+    const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
     T* __restrict__ strided = reinterpret_cast<T*>(a.base) + a.offset[v];
     const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
@@ -367,12 +371,13 @@ struct ShiftCopyArgs {
     uint64_t nbytes;
     uint64_t head;   // bytes before the vector part
     uint64_t nvec;   // 16-byte destination vectors in the vector part
+    uint64_t wg0;    // workgroups of this copy launched before this grid
 };
 
 template <int ROWS>
 __global__ __launch_bounds__(kPackThreads) void contiguous_copy_shift_kernel(ShiftCopyArgs a) {
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kPackThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t wave = (a.wg0 + blockIdx.x) * (kPackThreads / 64) + (threadIdx.x >> 6);
     char* __restrict__ dst = a.dst + a.head;            // 16-byte aligned
     const char* src = a.src + a.head;
     const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
@@ -398,7 +403,7 @@ __global__ __launch_bounds__(kPackThreads) void contiguous_copy_shift_kernel(Shi
             if (c < a.nvec) store16_writethrough(dst + c * 16, v[k]);
         }
     }
-    if (blockIdx.x == 0) {
+    if (a.wg0 + blockIdx.x == 0) {
         for (uint64_t i = threadIdx.x; i < a.head; i += kPackThreads) a.dst[i] = a.src[i];
         for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kPackThreads) a.dst[i] = a.src[i];
     }
@@ -419,12 +424,12 @@ static bool launch_shift_copy(char* dst, const char* src, uint64_t nbytes, hipSt
         tail += 16;
     }
     if (nvec == 0) return false;
-    ShiftCopyArgs a{dst, src, nbytes, head, nvec};
+    ShiftCopyArgs a{dst, src, nbytes, head, nvec, 0};
     const uint64_t per_wg = (uint64_t)(kPackThreads / 64) * kShiftCopyRows * 64;
-    const uint64_t wgs = (nvec + per_wg - 1) / per_wg;
-    if (wgs > 0x7fffffffull) return false;
-    hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3((uint32_t)wgs), dim3(kPackThreads), 0, stream, a);
-    *rc = launch_status();
+    *rc = launch_in_pieces((nvec + per_wg - 1) / per_wg, kPackThreads, 1, [&](uint64_t first, uint32_t count) {
+        a.wg0 = first;
+        hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3(count), dim3(kPackThreads), 0, stream, a);
+    });
     return true;
 }
 
@@ -439,6 +444,7 @@ struct FlatArgs {
     uint32_t ntensors;
     uint32_t shift;           // units
     uint32_t units_per_elem;
+    uint64_t wg0;             // workgroups of this copy launched before this grid
 };
 
 // Chunks per lane: 4 when gathering tensors into the flat buffer (0.74 of peak; 8 -> 0.71, 2 -> 0.69),
@@ -452,7 +458,7 @@ __global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
     constexpr int VU = 16 / U;
     constexpr int kUnroll = FlatUnroll<PACK>::value;
     __shared__ uint32_t s_range[2];
-    const uint64_t block_c0 = (uint64_t)blockIdx.x * (kFlatThreads * kUnroll);
+    const uint64_t block_c0 = (a.wg0 + blockIdx.x) * (kFlatThreads * kUnroll);
     if (threadIdx.x < 64) {
         // wavefront 0 finds the tensors holding the first and the last unit this block touches
         uint64_t c_last = block_c0 + kFlatThreads * kUnroll - 1;
@@ -678,13 +684,17 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             ++k;
             continue;
         }
-        if (first.ndim == 0 && unit == 16 && (first.total + kCopyThreads - 1) / kCopyThreads <= 0x7fffffffull) {
+        if (first.ndim == 0 && unit == 16) {
             char* strided = base + first.offset * 16;
             char* dst = PACK ? packed[k] : strided;
             const char* src = PACK ? strided : packed[k];
-            hipLaunchKernelGGL(contiguous_copy_kernel, dim3((uint32_t)((first.total + kCopyThreads - 1) / kCopyThreads)),
-                               dim3(kCopyThreads), 0, stream, dst, src, first.total);
-            if (int rc = launch_status()) return rc;
+            const uint64_t wgs = (first.total + kCopyThreads - 1) / kCopyThreads;
+            if (int rc = launch_in_pieces(wgs, kCopyThreads, 1, [&](uint64_t wg0, uint32_t count) {
+                    const uint64_t c0 = wg0 * kCopyThreads;  // chunks already launched
+                    hipLaunchKernelGGL(contiguous_copy_kernel, dim3(count), dim3(kCopyThreads), 0, stream, dst + c0 * 16,
+                                       src + c0 * 16, first.total - c0);
+                }))
+                return rc;
             ++k;
             continue;
         }
@@ -749,11 +759,12 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         const bool large = a.nchunks >= kLargeCopyChunks;
         const uint64_t per_block = (uint64_t)kPackThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
-        if (blocks * nbatch > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
         a.nviews = nbatch;
-        dim3 grid((uint32_t)(blocks * nbatch));
-        launch_slice_copy<PACK>(unit, !fits32, large, form, grid, stream, a);
-        if (int rc = launch_status()) return rc;
+        if (int rc = launch_in_pieces(blocks * nbatch, kPackThreads, 1, [&](uint64_t wg0, uint32_t count) {
+                a.wg0 = wg0;
+                launch_slice_copy<PACK>(unit, !fits32, large, form, dim3(count), stream, a);
+            }))
+            return rc;
         k += nbatch;
     }
     return MHIP_SUCCESS;
@@ -797,18 +808,19 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
     a.nchunks = (a.total + a.shift + vu - 1) / vu;
     const uint64_t per_block = (uint64_t)kFlatThreads * FlatUnroll<PACK>::value;
     const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
-    if (blocks > 0x7fffffffull) return MHIP_ERR_INVALID_ARGUMENT;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    dim3 grid((uint32_t)blocks);
-    switch (unit) {
-        case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
-        case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
-        case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
-        case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
-        default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, dim3(kFlatThreads), 0, hs, a); break;
-    }
-    return launch_status();
+    return launch_in_pieces(blocks, kFlatThreads, 1, [&](uint64_t wg0, uint32_t count) {
+        a.wg0 = wg0;
+        const dim3 grid(count), block(kFlatThreads);
+        switch (unit) {
+            case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, block, 0, hs, a); break;
+            case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, block, 0, hs, a); break;
+            case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, block, 0, hs, a); break;
+            case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, block, 0, hs, a); break;
+            default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, block, 0, hs, a); break;
+        }
+    });
 }
 
 }  // namespace mhip

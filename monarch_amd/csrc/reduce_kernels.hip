@@ -391,9 +391,9 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
 // ---------------- host side ----------------
 
 static uint32_t grid_for(uint64_t items) {
-    // one pass over the data; the grid-stride loop only engages beyond 2^31 workgroups
+    // one pass over the data; the grid-stride loop only engages beyond the largest grid a launch can hold
     const uint64_t blocks = (items + kReduceThreads - 1) / kReduceThreads;
-    const uint64_t cap = 0x7fffffffull;
+    const uint64_t cap = max_workgroups(kReduceThreads);
     return (uint32_t)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
 }
 
@@ -625,7 +625,7 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         // element-granular views with rows of at least one vector on both sides: V-element chunks
         const bool ragged = !vec && V > 1 && oc.run >= V && ic.run >= V;
         uint64_t tiles = grid_for(ragged ? (a.total + V - 1) / V : a.total);
-        while (tiles * nbatch > 0x7fffffffull) tiles = (tiles + 1) / 2;  // grid-stride takes over
+        while (tiles > 1 && tiles * nbatch > max_workgroups(kReduceThreads)) tiles = (tiles + 1) / 2;  // grid-stride takes over
         dim3 grid((uint32_t)(tiles * nbatch));
         const bool avg = op == MHIP_OP_AVG;
         switch (dtype) {

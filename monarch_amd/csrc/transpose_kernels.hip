@@ -21,6 +21,7 @@ struct TransArgs {
     uint64_t ntiles;   // nbatch * qtiles * ctiles
     uint32_t Sc, Q;    // extent along c and along q
     uint32_t ctiles, qtiles;
+    uint64_t wg0;      // workgroups of this copy launched before this grid (a multiple of 8)
     uint32_t group;    // tiles are walked in group x group blocks so that concurrently running workgroups
     uint32_t cgroups;  // touch neighbouring segments on BOTH sides (DRAM row locality); cgroups = ceil(ctiles/group)
     int n_inner;       // dimensions after c (decode q -> memory offset), outermost first
@@ -180,7 +181,8 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 
     // XCD-contiguous tile ranges: workgroup w runs on XCD w % 8
     const uint64_t per_xcd = (a.ntiles + 7) / 8;
-    const uint64_t tile_id = (uint64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile_id = (wg % 8) * per_xcd + wg / 8;
     if (tile_id >= a.ntiles) return;
 
     const uint64_t b = tile_id / per_batch;
@@ -423,24 +425,28 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
     const uint64_t qgroups = (a.qtiles + a.group - 1) / a.group;
     a.ntiles = nbatch * a.cgroups * qgroups * a.group * a.group;
-    const uint64_t cap = 0x7fffffffull;
-    const dim3 block(kThreads);
     if (vec) {
         const uint64_t nblocks = 8 * ((a.ntiles + 7) / 8);  // one tile per workgroup, eight XCD ranges
-        if (nblocks > cap) return false;
-        const dim3 grid((uint32_t)nblocks);
-        switch (unit) {
-            case 1: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-            case 2: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-            case 4: if (big) hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a); else hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-            case 8: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
-            default: return false;
-        }
-    } else {
-        const dim3 grid((uint32_t)(a.ntiles < cap ? a.ntiles : cap));
-        if (unit != 16) return false;
-        hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), grid, block, 0, stream, a);
+        const uint32_t lanes = unit == 8 ? 256 : big ? 1024 : 512;
+        *rc = launch_in_pieces(nblocks, lanes, 8, [&](uint64_t wg0, uint32_t count) {
+            a.wg0 = wg0;
+            const dim3 grid(count);
+            switch (unit) {
+                case 1: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                case 2: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                case 4:
+                    if (big) hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a);
+                    else hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a);
+                    break;
+                default: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+            }
+        });
+        return true;
     }
+    if (unit != 16) return false;
+    const uint64_t cap = max_workgroups(kThreads);  // grid-stride kernel
+    hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), dim3((uint32_t)(a.ntiles < cap ? a.ntiles : cap)), dim3(kThreads), 0,
+                       stream, a);
     *rc = launch_status();
     return true;
 }
