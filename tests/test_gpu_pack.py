@@ -287,6 +287,49 @@ def test_wide_index_path_over_2g_units():
     assert torch.equal(dst[1: n + 1], src[1: n + 1])
 
 
+def _check_large_view(dtype, sizes, strides, offset=0):
+    """pack against torch's own strided gather on the GPU (the CPU walk would take minutes at this size),
+    then unpack into zeros: the view comes back and nothing else is written."""
+    s = Slice(offset=offset, sizes=sizes, strides=strides)
+    _, hi = s.bounds()
+    es = torch.empty(0, dtype=dtype).element_size()
+    src = torch.empty(hi + 1, dtype=dtype, device=DEV)
+    raw = src.view(torch.uint8)
+    step = 1 << 28
+    for i in range(0, raw.numel(), step):  # a pattern with no short period
+        k = torch.arange(i, min(i + step, raw.numel()), device=DEV, dtype=torch.int64)
+        raw[i:i + step] = ((k * 2654435761) >> 13).to(torch.uint8)
+        del k
+    want = torch.as_strided(src, sizes, strides, offset).contiguous().reshape(-1)
+    got = staging.pack(src, s)
+    sync()
+    assert got.numel() * es >= 2**31
+    assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
+    del want
+    back = torch.zeros_like(src)
+    staging.unpack(back, s, got)
+    sync()
+    view = torch.as_strided(back, sizes, strides, offset)
+    assert torch.equal(view.contiguous().reshape(-1).view(torch.uint8), got.view(torch.uint8))
+    # every byte outside the view is still zero: the non-zero count of the whole equals that of the view
+    assert int(torch.count_nonzero(back.view(torch.uint8))) == int(torch.count_nonzero(got.view(torch.uint8)))
+
+
+def test_wide_index_rows_that_are_not_whole_chunks():
+    # 2^31 + 2^19 one-byte units in rows of 65535 at a pitch of 65537: 64-bit decode in the two-vector form
+    _check_large_view(torch.uint8, [32776, 65535], [65537, 1], offset=3)
+
+
+def test_wide_index_short_runs():
+    # more than 2^31 one-byte units in runs of 3 of 5: 64-bit decode in the gathering form
+    _check_large_view(torch.uint8, [716_000_000, 3], [5, 1], offset=1)
+
+
+def test_wide_index_whole_chunks():
+    # more than 2^31 two-byte units in rows of 4096 bf16 at an odd pitch: 64-bit decode in the whole-chunk form
+    _check_large_view(torch.bfloat16, [524_296, 4096], [4097, 1])
+
+
 def test_tensor_buffer_round_trip():
     # the RDMABuffer contract: 1-D contiguous uint8 only; TensorBuffer stages a strided view through it
     g = torch.Generator().manual_seed(9)

@@ -383,6 +383,31 @@ def test_reduce_scatter_fuzz(dtype):
             assert np.array_equal(bits(outs[k]), want[k]), (i, in_view, out_views[k], G, op)
 
 
+@pytest.mark.parametrize("sizes,strides", [([32776, 65535], [65537, 1]),    # rows of at least one vector: chunk form
+                                           ([716_000_000, 3], [5, 1])])   # runs of 3: element form
+def test_reduce_scatter_wide_index(sizes, strides):
+    # an output of more than 2^31 elements: 64-bit decode of both the output view and the input layout.
+    # int8 sums wrap, so torch's own add on the GPU is the expected value.
+    view = Slice(offset=1, sizes=sizes, strides=strides)
+    _, hi = view.bounds()
+    group = []
+    for g in range(2):
+        t = torch.empty(hi + 1, dtype=torch.int8, device=DEV)
+        step = 1 << 28
+        for i in range(0, t.numel(), step):
+            k = torch.arange(i, min(i + step, t.numel()), device=DEV, dtype=torch.int64)
+            t[i:i + step] = ((k * (2654435761 + 2 * g)) >> (11 + g)).to(torch.int8)
+            del k
+        group.append(t)
+    out = torch.empty(len(view), dtype=torch.int8, device=DEV)
+    assert out.numel() >= 2**31
+    R.reduce_scatter_views([out], [view], group, None, R.ReduceOp.Sum)
+    sync()
+    total = group[0] + group[1]
+    want = torch.as_strided(total, sizes, strides, 1).contiguous().reshape(-1)
+    assert torch.equal(out, want)
+
+
 def test_config4_mesh_dim_reduce_scatter_full_size():
     H, G, Rr, Cc, K = 2, 8, 2048, 4096, 8
     x, group, in_view, out_views, w = _c4(H, G, Rr, Cc, K, seed=4000)
