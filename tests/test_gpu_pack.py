@@ -457,6 +457,23 @@ def test_transpose_large_aligned_fp32_tiles():
     assert torch.equal(back, x)
 
 
+def test_transpose_large_aligned_bf16_tiles():
+    # 2^25 and more two-byte elements with 512-byte aligned rows: the 256 x 128 tile form, with a batch
+    # dimension and with tile counts that are not multiples of the walk's block size
+    g = torch.Generator(device=DEV).manual_seed(15)
+    for shape in [(2, 4096, 4096), (1, 4224, 8192 + 256), (3, 2944, 3840)]:
+        x = torch.randn(*shape, generator=g, device=DEV).bfloat16()
+        view = x.transpose(1, 2)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.view(view.shape).view(torch.int16), view.contiguous().view(torch.int16)), shape
+        back = torch.zeros_like(x)
+        staging.unpack(back, s, out)
+        sync()
+        assert torch.equal(back.view(torch.int16), x.view(torch.int16)), shape
+
+
 def test_stream_send_tensor_semantics():
     from monarch_amd.reduce import Factory
     from monarch_amd.send_tensor import route, stream_send_tensor
