@@ -29,12 +29,12 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_868_408, "c2_inplace": 452_868_594, "c2_separate": 452_867_524, "c2p_pack": 100_663_296,
-    "c2p_unpack": 100_663_296, "c3_pack": 234_866_695, "c3_unpack": 234_866_357, "c4": 603_819_427,
-    "c4_slots": 603_821_027, "c5_flat_pack": 3_166_108_494, "c5_quantize": 2_384_058_544,
-    "c5_dequant": 7_127_815_160, "c5_flat_unpack": 6_014_977_151, "c5_dequant_many8": 12_779_865_267,
-    "c5_quantize_bucket": 2_374_360_623, "c5_dequant_bucket": 7_176_516_908, "tr_f32_pack": 536_836_326,
-    "tr_f32_unpack": 536_845_701, "tr_bf16_pack": 268_455_780,
+    "c2": 452_870_600, "c2_inplace": 452_870_787, "c2_separate": 452_869_716, "c2p_pack": 100_663_296,
+    "c2p_unpack": 100_663_570, "c3_pack": 234_865_833, "c3_unpack": 234_865_798, "c4": 603_822_351,
+    "c4_slots": 603_823_951, "c5_flat_pack": 3_166_117_170, "c5_quantize": 2_384_067_112,
+    "c5_dequant": 7_127_836_847, "c5_flat_unpack": 6_014_993_348, "c5_dequant_many8": 12_779_917_743,
+    "c5_quantize_bucket": 2_374_369_255, "c5_dequant_bucket": 7_176_538_659, "tr_f32_pack": 536_837_788,
+    "tr_f32_unpack": 536_847_163, "tr_bf16_pack": 268_456_511,
 }
 
 
