@@ -255,7 +255,7 @@ def wl_c2(torch, in_place=False, sets=3, separate=False):
                  for _ in range(n)]
         out = np.empty_like(hosts[0])
         reps, t0 = 0, time.perf_counter()
-        while reps < 3 or time.perf_counter() - t0 < 5.0:
+        while reps < 3 or time.perf_counter() - t0 < 10.0:
             oracle.reduce(hosts, oracle.AVG, out=out)
             reps += 1
         dt = (time.perf_counter() - t0) / reps
