@@ -9,7 +9,7 @@
 //!
 //! This crate is written against the header by hand (no bindgen) and has not been
 //! compiled in the build environment of this repository, which ships no Rust toolchain;
-//! `tests/test_abi.py` checks that the function names here and in the header agree.
+//! `tests/test_abi.py` checks every declaration here against the header, name by name and type by type.
 #![allow(non_camel_case_types)]
 
 use std::os::raw::{c_char, c_int, c_void};
@@ -85,53 +85,53 @@ extern "C" {
     pub fn mhip_error_string(status: c_int) -> *const c_char;
     pub fn mhip_version() -> c_int;
     pub fn mhip_dtype_size(dtype: c_int) -> u32;
-    pub fn mhip_slice_validate(offset: usize, sizes: *mut u64, nsizes: u32, strides: *mut u64, nstrides: u32) -> c_int;
+    pub fn mhip_slice_validate(offset: u64, sizes: *const u64, nsizes: u32, strides: *const u64, nstrides: u32) -> c_int;
     pub fn mhip_slice_len(s: *const mhip_slice_t, len: *mut u64) -> c_int;
     pub fn mhip_slice_is_contiguous(s: *const mhip_slice_t, result: *mut c_int) -> c_int;
-    pub fn mhip_slice_get(s: *const mhip_slice_t, index: usize, loc: *mut u64) -> c_int;
-    pub fn mhip_slice_location(s: *const mhip_slice_t, coord: *mut u64, ncoord: u32, loc: *mut u64) -> c_int;
-    pub fn mhip_slice_coordinates(s: *const mhip_slice_t, value: usize, coords: *mut u64) -> c_int;
-    pub fn mhip_slice_index(s: *const mhip_slice_t, value: usize, index: *mut u64) -> c_int;
-    pub fn mhip_slice_iter(s: *const mhip_slice_t, start: usize, count: usize, locs: *mut c_void, written: *mut u64) -> c_int;
-    pub fn mhip_slice_select(s: *const mhip_slice_t, dim: u32, begin: usize, end: usize, step: usize, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
-    pub fn mhip_slice_at(s: *const mhip_slice_t, dim: u32, index: usize, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
-    pub fn mhip_slice_subview(s: *const mhip_slice_t, starts: *mut u64, nstarts: u32, lens: *mut u64, nlens: u32, out_offset: *mut u64) -> c_int;
-    pub fn mhip_slice_view(s: *const mhip_slice_t, new_sizes: *mut u64, nnew: u32, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_get(s: *const mhip_slice_t, index: u64, loc: *mut u64) -> c_int;
+    pub fn mhip_slice_location(s: *const mhip_slice_t, coord: *const u64, ncoord: u32, loc: *mut u64) -> c_int;
+    pub fn mhip_slice_coordinates(s: *const mhip_slice_t, value: u64, coords: *mut u64) -> c_int;
+    pub fn mhip_slice_index(s: *const mhip_slice_t, value: u64, index: *mut u64) -> c_int;
+    pub fn mhip_slice_iter(s: *const mhip_slice_t, start: u64, count: u64, locs: *mut u64, written: *mut u64) -> c_int;
+    pub fn mhip_slice_select(s: *const mhip_slice_t, dim: u32, begin: u64, end: u64, step: u64, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_at(s: *const mhip_slice_t, dim: u32, index: u64, out_offset: *mut u64, out_sizes: *mut u64, out_strides: *mut u64) -> c_int;
+    pub fn mhip_slice_subview(s: *const mhip_slice_t, starts: *const u64, nstarts: u32, lens: *const u64, nlens: u32, out_offset: *mut u64) -> c_int;
+    pub fn mhip_slice_view(s: *const mhip_slice_t, new_sizes: *const u64, nnew: u32, out_strides: *mut u64) -> c_int;
     pub fn mhip_slice_enforce_embedding(s: *const mhip_slice_t, other: *const mhip_slice_t) -> c_int;
     pub fn mhip_slice_bounds(s: *const mhip_slice_t, min_loc: *mut u64, max_loc: *mut u64) -> c_int;
-    pub fn mhip_mesh_dim_members(ranks: *const mhip_slice_t, rank: usize, dim: u32, members: *mut u64, dim_rank: *mut u64) -> c_int;
-    pub fn mhip_mesh_ranks_for_dims(ranks: *const mhip_slice_t, rank: usize, dims: *const u32, ndims: u32, out: *mut u64, cap: usize, count: *mut u64) -> c_int;
-    pub fn mhip_slice_pack(dst: *mut c_void, src_base: *mut c_void, s: *const mhip_slice_t, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_slice_unpack(dst_base: *mut c_void, src: *mut c_void, s: *const mhip_slice_t, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_slice_pack_many(dsts: *const *mut c_void, src_base: *mut c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_slice_unpack_many(dst_base: *mut c_void, srcs: *const *mut c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_flat_pack(flat: *mut c_void, d_tensors: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: usize, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_flat_unpack(d_tensors: *mut c_void, flat: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: usize, elem_size: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_reduce(out: *mut c_void, input: *const *mut c_void, n: u32, numel: usize, dtype: c_int, op: c_int, stream: *mut c_void) -> c_int;
-    pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *mut c_void, in_view: *const mhip_slice_t, in_numel: usize, n_in: u32, dtype: c_int, op: c_int, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_quantize(q: *mut c_void, scales: *mut c_void, x_bf16: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate(acc: *mut c_void, q: *mut c_void, scales: *mut c_void, numel: usize, block: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate_many(acc: *mut c_void, q: *const *mut c_void, scales: *const *mut c_void, n: u32, numel: usize, block: u32, overwrite: c_int, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_quantize_bucket(q: *mut c_void, scales: *mut c_void, d_tensors: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *mut c_void, q: *mut c_void, scales: *mut c_void, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *mut c_void, q: *const *mut c_void, scales: *const *mut c_void, n: u32, d_offsets: *mut c_void, ntensors: u32, total: u64, block: u32, stream: *mut c_void) -> c_int;
+    pub fn mhip_mesh_dim_members(ranks: *const mhip_slice_t, rank: u64, dim: u32, members: *mut u64, dim_rank: *mut u64) -> c_int;
+    pub fn mhip_mesh_ranks_for_dims(ranks: *const mhip_slice_t, rank: u64, dims: *const u32, ndims: u32, out: *mut u64, cap: u64, count: *mut u64) -> c_int;
+    pub fn mhip_slice_pack(dst: *mut c_void, src_base: *const c_void, s: *const mhip_slice_t, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_slice_unpack(dst_base: *mut c_void, src: *const c_void, s: *const mhip_slice_t, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_slice_pack_many(dsts: *const *mut c_void, src_base: *const c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_slice_unpack_many(dst_base: *mut c_void, srcs: *const *const c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_flat_pack(flat: *mut c_void, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_flat_unpack(d_tensors: *const *mut c_void, flat: *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_reduce(out: *mut c_void, input: *const *const c_void, n: u32, numel: u64, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *const c_void, in_view: *const mhip_slice_t, in_numel: u64, n_in: u32, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_quantize(q: *mut u8, scales: *mut f32, x_bf16: *const c_void, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate(acc: *mut f32, q: *const u8, scales: *const f32, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_many(acc: *mut f32, q: *const *const u8, scales: *const *const f32, n: u32, numel: u64, block: u32, overwrite: c_int, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_quantize_bucket(q: *mut u8, scales: *mut f32, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *const *mut c_void, q: *const u8, scales: *const f32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *const *mut c_void, q: *const *const u8, scales: *const *const f32, n: u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_device_count(count: *mut c_int) -> c_int;
     pub fn mhip_set_device(device: c_int) -> c_int;
     pub fn mhip_device_synchronize() -> c_int;
-    pub fn mhip_stream_create(stream: *const *mut c_void) -> c_int;
-    pub fn mhip_stream_destroy(stream: *mut c_void) -> c_int;
-    pub fn mhip_stream_synchronize(stream: *mut c_void) -> c_int;
-    pub fn mhip_event_create(event: *const *mut c_void) -> c_int;
-    pub fn mhip_event_destroy(event: *mut c_void) -> c_int;
-    pub fn mhip_event_record(event: *mut c_void, stream: *mut c_void) -> c_int;
-    pub fn mhip_event_synchronize(event: *mut c_void) -> c_int;
-    pub fn mhip_event_elapsed_ms(ms: *mut f32, start: *mut c_void, stop: *mut c_void) -> c_int;
-    pub fn mhip_stream_wait_event(stream: *mut c_void, event: *mut c_void) -> c_int;
-    pub fn mhip_malloc(ptr: *const *mut c_void, bytes: usize) -> c_int;
+    pub fn mhip_stream_create(stream: *mut mhip_stream_t) -> c_int;
+    pub fn mhip_stream_destroy(stream: mhip_stream_t) -> c_int;
+    pub fn mhip_stream_synchronize(stream: mhip_stream_t) -> c_int;
+    pub fn mhip_event_create(event: *mut mhip_event_t) -> c_int;
+    pub fn mhip_event_destroy(event: mhip_event_t) -> c_int;
+    pub fn mhip_event_record(event: mhip_event_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_event_synchronize(event: mhip_event_t) -> c_int;
+    pub fn mhip_event_elapsed_ms(ms: *mut f32, start: mhip_event_t, stop: mhip_event_t) -> c_int;
+    pub fn mhip_stream_wait_event(stream: mhip_stream_t, event: mhip_event_t) -> c_int;
+    pub fn mhip_malloc(ptr: *mut *mut c_void, bytes: usize) -> c_int;
     pub fn mhip_free(ptr: *mut c_void) -> c_int;
-    pub fn mhip_memcpy_htod(dst: *mut c_void, src: *mut c_void, bytes: usize, stream: *mut c_void) -> c_int;
-    pub fn mhip_memcpy_dtoh(dst: *mut c_void, src: *mut c_void, bytes: usize, stream: *mut c_void) -> c_int;
-    pub fn mhip_memset(dst: *mut c_void, value: c_int, bytes: usize, stream: *mut c_void) -> c_int;
+    pub fn mhip_memcpy_htod(dst: *mut c_void, src: *const c_void, bytes: usize, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_memcpy_dtoh(dst: *mut c_void, src: *const c_void, bytes: usize, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_memset(dst: *mut c_void, value: c_int, bytes: usize, stream: mhip_stream_t) -> c_int;
     pub fn mhip_staging_alloc(ptr: *mut *mut c_void, padded_bytes: *mut usize, bytes: usize, device: c_int) -> c_int;
     pub fn mhip_staging_free(ptr: *mut c_void, padded_bytes: usize) -> c_int;
     pub fn mhip_staging_slot_pitch(slot_bytes: usize, pitch_bytes: *mut usize) -> c_int;
@@ -150,7 +150,7 @@ mod tests {
             assert!(mhip_version() >= 100);
             let sizes = [2u64, 3];
             let strides = [3u64, 1];
-            assert_eq!(mhip_slice_validate(0, sizes.as_ptr() as *mut u64, 2, strides.as_ptr() as *mut u64, 2), status::SUCCESS);
+            assert_eq!(mhip_slice_validate(0, sizes.as_ptr(), 2, strides.as_ptr(), 2), status::SUCCESS);
             let s = mhip_slice_t { offset: 0, ndim: 2, sizes: sizes.as_ptr(), strides: strides.as_ptr() };
             let mut loc = 0u64;
             assert_eq!(mhip_slice_get(&s, 4, &mut loc), status::SUCCESS);

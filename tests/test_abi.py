@@ -112,6 +112,66 @@ def test_rust_extern_block_names_match_header():
         assert re.search(rf"pub const {name}: i32 = {value};", text), name
 
 
+# C parameter / return types of the header -> the Rust spelling the extern block must use
+_RUST_TYPE = {
+    "const float*": "*const f32", "const float* const*": "*const *const f32", "const mhip_slice_t*": "*const mhip_slice_t",
+    "const uint32_t*": "*const u32", "const uint64_t*": "*const u64", "const uint8_t*": "*const u8",
+    "const uint8_t* const*": "*const *const u8", "const void*": "*const c_void", "const void* const*": "*const *const c_void",
+    "float*": "*mut f32", "int": "c_int", "int*": "*mut c_int", "mhip_event_t": "mhip_event_t",
+    "mhip_event_t*": "*mut mhip_event_t", "mhip_stream_t": "mhip_stream_t", "mhip_stream_t*": "*mut mhip_stream_t",
+    "size_t": "usize", "size_t*": "*mut usize", "uint32_t": "u32", "uint64_t": "u64", "uint64_t*": "*mut u64",
+    "uint8_t*": "*mut u8", "void*": "*mut c_void", "void* const*": "*const *mut c_void", "void**": "*mut *mut c_void",
+    "const char*": "*const c_char",
+}
+
+
+def test_rust_extern_block_types_match_header():
+    # every parameter and return type of the Rust declarations is the header's, spelled in Rust: no `*mut` for a
+    # `const` pointer, no `usize` for a `uint64_t`, out-parameters as `*mut`
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "monarch_hip.h")).read(), flags=re.S)
+    rust = open(os.path.join(ROOT, "hip-sys", "src", "lib.rs")).read()
+    rust_decl = {name: (params, ret) for name, params, ret in
+                 re.findall(r"pub fn (mhip_[a-z0-9_]+)\(([^()]*)\) -> ([^;]+);", rust)}
+    protos = re.findall(r"^\s*([A-Za-z_][A-Za-z0-9_ \*]*?)\s*\b(mhip_[a-z0-9_]+)\s*\(([^()]*)\)\s*;", header, flags=re.M)
+    assert len(protos) == len(declared_symbols())
+    for ret, name, params in protos:
+        want = []
+        for p in params.split(","):
+            p = " ".join(p.split())
+            if p in ("", "void"):
+                continue
+            ctype = re.match(r"(.*?)([A-Za-z_][A-Za-z0-9_]*)$", p).group(1).strip().replace(" *", "*")
+            want.append(_RUST_TYPE[ctype])
+        got_params, got_ret = rust_decl[name]
+        got = [a.split(":", 1)[1].strip() for a in got_params.split(",") if a.strip()]
+        assert got == want, (name, got, want)
+        assert got_ret.strip() == _RUST_TYPE[" ".join(ret.split()).replace(" *", "*")], (name, got_ret)
+
+
+def test_ctypes_table_scalar_widths_match_header():
+    # scalars are passed by value: a wrong width in the ctypes table shifts every later argument.  Pointers may be
+    # declared as c_void_p or as a typed POINTER in the table; both are pointer-sized.
+    import ctypes as C
+    scalar = {"int": C.c_int, "uint32_t": C.c_uint32, "uint64_t": C.c_uint64, "size_t": C.c_size_t}
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "monarch_hip.h")).read(), flags=re.S)
+    protos = re.findall(r"^\s*([A-Za-z_][A-Za-z0-9_ \*]*?)\s*\b(mhip_[a-z0-9_]+)\s*\(([^()]*)\)\s*;", header, flags=re.M)
+    for ret, name, params in protos:
+        restype, argtypes = _lib.SIGNATURES[name]
+        ctypes_of = []
+        for p in params.split(","):
+            p = " ".join(p.split())
+            if p in ("", "void"):
+                continue
+            ctypes_of.append(re.match(r"(.*?)([A-Za-z_][A-Za-z0-9_]*)$", p).group(1).strip().replace(" *", "*"))
+        for i, (ct, at) in enumerate(zip(ctypes_of, argtypes)):
+            if ct in scalar:
+                assert C.sizeof(at) == C.sizeof(scalar[ct]) and not hasattr(at, "contents") and at is not C.c_void_p, (name, i, ct, at)
+            else:  # every other parameter type of the header is a pointer or an opaque handle
+                assert C.sizeof(at) == C.sizeof(C.c_void_p), (name, i, ct, at)
+        ret = " ".join(ret.split()).replace(" *", "*")
+        assert C.sizeof(restype) == (C.sizeof(scalar[ret]) if ret in scalar else C.sizeof(C.c_void_p)), (name, ret)
+
+
 def _param_counts(text, pattern):
     counts = {}
     for name, params in re.findall(pattern, text, flags=re.S):
