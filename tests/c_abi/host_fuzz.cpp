@@ -1,0 +1,196 @@
+// Host-only fuzz of the library's Slice code (slice_host.cpp) and copy planner (plan.cpp), meant to be
+// built with -fsanitize=address,undefined: random valid and invalid Slices go through every host entry
+// point, and what comes back is checked against the definitions (iter == get, index(get(i)) == i,
+// the canonical form decodes to the same byte offsets as get).  No GPU, no HIP headers.
+#include <cinttypes>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "../../monarch_amd/csrc/mhip_internal.h"
+
+using namespace mhip;
+
+static uint64_t rng_state = 0x9e3779b97f4a7c15ull;
+static uint64_t rnd() {
+    rng_state ^= rng_state << 13;
+    rng_state ^= rng_state >> 7;
+    rng_state ^= rng_state << 17;
+    return rng_state;
+}
+static uint64_t below(uint64_t n) { return rnd() % n; }
+
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        if (!(cond)) {                                                               \
+            std::printf("FAILED %s at line %d (case %" PRIu64 ")\n", #cond, __LINE__, case_no); \
+            std::exit(1);                                                            \
+        }                                                                            \
+    } while (0)
+
+static uint64_t case_no = 0;
+
+// byte offset of packed byte `byte` by the definition: element get(i), byte within the element
+static uint64_t byte_by_definition(const mhip_slice_t& s, uint32_t elem_size, uint64_t byte) {
+    uint64_t loc = 0;
+    const int rc = mhip_slice_get(&s, byte / elem_size, &loc);
+    if (rc != MHIP_SUCCESS) {
+        std::printf("get failed with %d\n", rc);
+        std::exit(1);
+    }
+    return loc * elem_size + byte % elem_size;
+}
+
+// the same through the canonical form: row-major decode of the dimensions outside the run
+static uint64_t byte_by_canonical_form(const CanonSlice& c, uint32_t unit, uint64_t byte) {
+    const uint64_t t = byte / unit;
+    uint64_t row = t / c.run, off = c.offset + t % c.run;
+    for (int k = c.ndim - 1; k >= 0; --k) {
+        off += (row % c.dims[k].size) * c.dims[k].stride;
+        row /= c.dims[k].size;
+    }
+    return off * unit + byte % unit;
+}
+
+int main() {
+    const uint32_t elem_sizes[] = {1, 2, 3, 4, 6, 8, 12, 16};
+    uint64_t n_valid = 0, n_invalid = 0;
+    for (case_no = 0; case_no < 8000; ++case_no) {
+        // a valid slice: row-major over a random permutation of the dimensions, with random gaps
+        const uint32_t nd = (uint32_t)below(6);
+        std::vector<uint64_t> sizes(nd), strides(nd);
+        std::vector<uint32_t> order(nd);
+        for (uint32_t k = 0; k < nd; ++k) {
+            sizes[k] = 1 + below(7);
+            order[k] = k;
+        }
+        for (uint32_t k = nd; k > 1; --k) std::swap(order[k - 1], order[below(k)]);
+        uint64_t step = 1 + (below(4) == 0 ? below(3) : 0);
+        for (uint32_t j = 0; j < nd; ++j) {
+            const uint32_t k = order[j];
+            strides[k] = step;
+            step *= sizes[k] * (1 + (below(3) == 0 ? below(3) : 0));
+        }
+        bool mutated = false;  // set when a change may have made the slice invalid
+        if (nd && below(10) == 0) {  // empty; invalid when the dimension shared its stride as one of size 1
+            sizes[below(nd)] = 0;
+            mutated = true;
+        }
+        if (nd && below(4) == 0) {
+            strides[below(nd)] = below(2) ? below(40) : strides[below(nd)];
+            mutated = true;
+        }
+        const uint64_t offset = below(50);
+        mhip_slice_t s{offset, nd, sizes.data(), strides.data()};
+
+        const int rc = mhip_slice_validate(offset, sizes.data(), nd, strides.data(), nd);
+        CHECK(mutated || rc == MHIP_SUCCESS);
+        if (rc != MHIP_SUCCESS) {
+            ++n_invalid;
+            CHECK(rc >= 10000);
+            continue;
+        }
+        ++n_valid;
+        uint64_t len = 0;
+        CHECK(mhip_slice_len(&s, &len) == MHIP_SUCCESS);
+        uint64_t expect_len = 1;
+        for (uint64_t v : sizes) expect_len *= v;
+        CHECK(len == expect_len);
+        int contiguous = -1;
+        CHECK(mhip_slice_is_contiguous(&s, &contiguous) == MHIP_SUCCESS);
+
+        // iter == get, in pieces that start anywhere; index(get(i)) == i; bounds hold
+        std::vector<uint64_t> locs(len + 3, ~0ull);
+        uint64_t done = 0;
+        while (done < len) {
+            const uint64_t want = 1 + below(len);
+            uint64_t written = 0;
+            CHECK(mhip_slice_iter(&s, done, want, locs.data() + done, &written) == MHIP_SUCCESS);
+            CHECK(written == (want < len - done ? want : len - done));
+            done += written;
+        }
+        uint64_t written = 7;
+        CHECK(mhip_slice_iter(&s, len, 5, locs.data() + len, &written) == MHIP_SUCCESS && written == 0);
+        uint64_t lo = 0, hi = 0;
+        const int brc = mhip_slice_bounds(&s, &lo, &hi);
+        CHECK(len == 0 || brc == MHIP_SUCCESS);
+        std::vector<uint64_t> coords(nd + 1);
+        for (uint64_t i = 0; i < len; ++i) {
+            uint64_t loc = 0, index = ~0ull;
+            CHECK(mhip_slice_get(&s, i, &loc) == MHIP_SUCCESS && loc == locs[i]);
+            CHECK(loc >= lo && loc <= hi);
+            CHECK(mhip_slice_index(&s, loc, &index) == MHIP_SUCCESS && index == i);
+            CHECK(mhip_slice_coordinates(&s, loc, coords.data()) == MHIP_SUCCESS);
+            uint64_t back = 0;
+            CHECK(mhip_slice_location(&s, coords.data(), nd, &back) == MHIP_SUCCESS && back == loc);
+        }
+        uint64_t loc = 0;
+        CHECK(mhip_slice_get(&s, len, &loc) == MHIP_ERR_INDEX_OUT_OF_RANGE);
+        if (contiguous == 1)
+            for (uint64_t i = 0; i < len; ++i) CHECK(locs[i] == offset + i);
+
+        // select / at produce slices whose elements are elements of s
+        if (nd && len) {
+            const uint32_t dim = (uint32_t)below(nd);
+            std::vector<uint64_t> osz(nd), ost(nd);
+            uint64_t ooff = 0;
+            const uint64_t b = below(sizes[dim]), e = b + 1 + below(sizes[dim] - b), st = 1 + below(3);
+            // a step can leave a stride that an outer stride is no multiple of, or that is too small for
+            // the dimension sorted after it: the result is then refused, as Slice::select refuses it when
+            // it re-validates (slice.rs:325)
+            const int src = mhip_slice_select(&s, dim, b, e, st, &ooff, osz.data(), ost.data());
+            CHECK(src == MHIP_SUCCESS || (st > 1 && (src == MHIP_ERR_NONRECTANGULAR_SHAPE || src == MHIP_ERR_STRIDE_TOO_SMALL)));
+            if (src == MHIP_SUCCESS) {
+                mhip_slice_t sub{ooff, nd, osz.data(), ost.data()};
+                uint64_t sublen = 0;
+                CHECK(mhip_slice_len(&sub, &sublen) == MHIP_SUCCESS && sublen >= 1 && sublen <= len);
+                for (uint64_t i = 0; i < sublen; ++i) {
+                    uint64_t l = 0, idx = 0;
+                    CHECK(mhip_slice_get(&sub, i, &l) == MHIP_SUCCESS);
+                    CHECK(mhip_slice_index(&s, l, &idx) == MHIP_SUCCESS);
+                }
+                CHECK(mhip_slice_enforce_embedding(&sub, &s) == MHIP_SUCCESS);
+            }
+            std::vector<uint64_t> asz(nd), ast(nd);
+            uint64_t aoff = 0;
+            CHECK(mhip_slice_at(&s, dim, b, &aoff, asz.data(), ast.data()) == MHIP_SUCCESS);
+            CHECK(mhip_slice_at(&s, dim, sizes[dim], &aoff, asz.data(), ast.data()) != MHIP_SUCCESS);
+        }
+
+        // the planner: every packed byte lands where the definition says, for several element sizes,
+        // address alignments and unit limits
+        for (int rep = 0; rep < 3; ++rep) {
+            const uint32_t es = elem_sizes[below(8)];
+            const uint64_t mask = below(3) == 0 ? below(64) : 0;
+            const uint32_t max_unit = 1u << below(5);
+            CanonSlice c;
+            uint32_t unit = 0;
+            const bool nonempty = canonicalize(s, es, mask, max_unit, &c, &unit);
+            CHECK(nonempty == (len != 0));
+            if (!nonempty) continue;
+            CHECK(unit >= 1 && unit <= max_unit && (unit & (unit - 1)) == 0 && (mask & (unit - 1)) == 0);
+            CHECK(c.total * unit == len * es && c.run >= 1 && c.ndim >= 0 && c.ndim <= (int)nd + 1);
+            CHECK(same_shape(c, c));
+            uint64_t rows = 1;
+            for (int k = 0; k < c.ndim; ++k) rows *= c.dims[k].size;
+            CHECK(rows * c.run == c.total);
+            const uint64_t nbytes = len * es;
+            const uint64_t stride = nbytes > 4096 ? 1 + below(7) : 1;  // sample long ones
+            for (uint64_t byte = below(stride); byte < nbytes; byte += stride)
+                CHECK(byte_by_canonical_form(c, unit, byte) == byte_by_definition(s, es, byte));
+        }
+
+        // a mesh over the same slice: the members of each dimension contain the rank itself
+        if (nd && len && len <= 512) {
+            const uint64_t rank = locs[below(len)];
+            for (uint32_t dim = 0; dim < nd; ++dim) {
+                std::vector<uint64_t> members(sizes[dim] + 1, ~0ull);
+                uint64_t dim_rank = ~0ull;
+                CHECK(mhip_mesh_dim_members(&s, rank, dim, members.data(), &dim_rank) == MHIP_SUCCESS);
+                CHECK(dim_rank < sizes[dim] && members[dim_rank] == rank && members[sizes[dim]] == ~0ull);
+            }
+        }
+    }
+    std::printf("ok: %" PRIu64 " valid and %" PRIu64 " invalid slices\n", n_valid, n_invalid);
+    return 0;
+}
