@@ -280,6 +280,8 @@ int mhip_malloc(void** ptr, size_t bytes);
 int mhip_free(void* ptr);
 int mhip_memcpy_htod(void* dst, const void* src, size_t bytes, mhip_stream_t stream);
 int mhip_memcpy_dtoh(void* dst, const void* src, size_t bytes, mhip_stream_t stream);
+/* Fills `bytes` bytes with the low byte of `value` (cuMemsetD8Async semantics).  Runs as a kernel, not as a memset
+ * node, so it can be recorded into a HIP graph like the data-path entry points. */
 int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream);
 
 

@@ -3,9 +3,32 @@
 #include <cstdint>
 #include <hip/hip_runtime.h>
 
-#include "mhip_internal.h"
+#include "mhip_device.h"
 
 #define MHIP_VERSION 100
+
+namespace mhip {
+
+// Byte fill as a kernel rather than hipMemsetAsync: memset nodes recorded into a HIP graph have produced wrong
+// results on replays after the first on this platform, kernel nodes have not, and callers may capture this call
+// (clearing a staging chunk after it has been summed, parameter_server.rs:200-205).  16-byte vectors over the
+// aligned middle of the range, single bytes at its ends.
+constexpr int kFillThreads = 256;
+
+__global__ __launch_bounds__(kFillThreads) void fill_kernel(unsigned char* dst, uint32_t word, uint64_t bytes, uint64_t head,
+                                                            uint64_t nvec, uint64_t wg0) {
+    const uint64_t wg = wg0 + blockIdx.x;
+    const uint64_t v = wg * kFillThreads + threadIdx.x;
+    if (v < nvec) store16_aligned(dst + head + v * 16, make_uint4(word, word, word, word));
+    if (wg == 0) {
+        for (uint64_t i = threadIdx.x; i < head; i += kFillThreads) dst[i] = (unsigned char)word;
+        for (uint64_t i = head + nvec * 16 + threadIdx.x; i < bytes; i += kFillThreads) dst[i] = (unsigned char)word;
+    }
+}
+
+}  // namespace mhip
+
+using namespace mhip;
 
 extern "C" {
 
@@ -85,7 +108,19 @@ int mhip_memcpy_dtoh(void* dst, const void* src, size_t bytes, mhip_stream_t str
     return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
 }
 int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream) {
-    return (int)hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream));
+    if (bytes == 0) return MHIP_SUCCESS;
+    if (!dst) return MHIP_ERR_UNDEFINED_TENSOR;
+    const uint32_t b = (uint32_t)value & 0xffu, word = b * 0x01010101u;
+    uint64_t head = (16 - ((uintptr_t)dst & 15u)) & 15u;
+    if (head > bytes) head = bytes;
+    const uint64_t nvec = (bytes - head) / 16;
+    const uint64_t wgs = nvec ? (nvec + kFillThreads - 1) / kFillThreads : 1;  // workgroup 0 also writes the ends
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    return launch_in_pieces(wgs, kFillThreads, 1, [&](uint64_t wg0, uint32_t count) {
+        hipLaunchKernelGGL(fill_kernel, dim3(count), dim3(kFillThreads), 0, hs, static_cast<unsigned char*>(dst), word,
+                           (uint64_t)bytes, head, nvec, wg0);
+    });
 }
 
 // ---- staging-buffer lifecycle -------------------------------------------------------

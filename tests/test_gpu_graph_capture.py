@@ -1,5 +1,5 @@
 """The device entry points only enqueue kernels on the caller's stream (no allocation, no
-synchronisation, no memset), so a caller can record them into a HIP graph.  A captured
+synchronisation, no memset node: mhip_memset itself is a fill kernel), so a caller can record them into a HIP graph.  A captured
 pack -> reduce -> unpack pipeline and a captured fp8 round trip are replayed several times with
 new input data and eager work in between, and every replay is compared with the eager result."""
 import numpy as np
@@ -98,3 +98,50 @@ def test_fp8_bucket_round_trip_replays():
         oracle.fp8_dequant_accumulate(want, hq, hs, 1024)
         assert np.array_equal(q.cpu().numpy(), hq) and np.array_equal(scales.cpu().numpy(), hs)
         assert np.array_equal(torch.cat(accs).cpu().numpy(), want), rep
+
+
+def test_memset_every_alignment_and_in_a_graph():
+    # the byte fill is a kernel: exact at every start alignment and length, nothing written outside the
+    # range, and it can be recorded into a graph (clear a staging chunk, then accumulate into it)
+    import ctypes as C
+    from monarch_amd._lib import check, lib
+    stream = torch.cuda.current_stream().cuda_stream
+    buf = torch.empty(4096, dtype=torch.uint8, device=DEV)
+    for start in list(range(0, 19)) + [31, 33]:
+        for nbytes in [0, 1, 2, 15, 16, 17, 31, 32, 33, 100, 1000, 4000]:
+            buf.fill_(0xEE)
+            check(lib().mhip_memset(buf.data_ptr() + start, 0x1A5, nbytes, stream))  # only the low byte counts
+            sync()
+            got = buf.cpu().numpy()
+            assert (got[start:start + nbytes] == 0xA5).all() and (got[:start] == 0xEE).all() \
+                and (got[start + nbytes:] == 0xEE).all(), (start, nbytes)
+    big = torch.empty((3 << 20) + 5, dtype=torch.uint8, device=DEV)
+    check(lib().mhip_memset(big.data_ptr() + 3, 7, big.numel() - 5, stream))
+    sync()
+    assert bool((big[3:-2] == 7).all())
+
+    n = 5000
+    acc = torch.empty(n, dtype=torch.float32, device=DEV)
+    x = [torch.zeros(n, dtype=torch.float32, device=DEV) for _ in range(3)]
+
+    def pipeline():
+        check(lib().mhip_memset(acc.data_ptr(), 0, n * 4, torch.cuda.current_stream().cuda_stream))
+        R.all_reduce(acc, [acc, *x], R.ReduceOp.Sum)  # in place: acc = 0 + sum of x
+
+    pipeline()
+    sync()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        pipeline()
+    g = torch.Generator().manual_seed(9)
+    for rep in range(4):
+        hosts = [torch.randn(n, generator=g) for _ in x]
+        for t, h in zip(x, hosts):
+            t.copy_(h)
+        acc.fill_(float("nan"))  # must be cleared by the replayed fill, every time
+        junk = torch.randn(1 << 18, device=DEV).sum()
+        graph.replay()
+        sync()
+        want = ((torch.zeros(n) + hosts[0]) + hosts[1]) + hosts[2]
+        assert torch.equal(acc.cpu(), want), rep
+        assert torch.isfinite(junk)
