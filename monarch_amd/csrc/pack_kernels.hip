@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     const uint64_t c0 = tile * (kPackThreads * kUnroll) + threadIdx.x;
 
     if constexpr (NDIM == 0) {
-        // Contiguous view: when the whole 32 KiB tile of this workgroup lies inside the
+        // Contiguous view: when the whole tile of this workgroup lies inside the
         // buffer (decided on the scalar unit), no per-chunk tests are needed at all.
         const uint64_t tile_first = tile * (kPackThreads * kUnroll) * VU;
         const uint64_t tile_end = tile_first + (uint64_t)(kPackThreads * kUnroll) * VU;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
 
 // The same copy for views whose rows are not whole chunks (row length not a multiple of 16
 // bytes, or a staging address that is not 16-byte aligned): then about one chunk per row
-// straddles a row boundary, and with 512 chunks per wavefront step every wavefront would
+// straddles a row boundary, and with several rows per wavefront step nearly every wavefront would
 // fall off the predicate-free path above.  A straddling chunk is moved as two whole
 // 16-byte vectors instead, each inside one row on both sides: "A" ends where the row ends,
 // "B" starts where the next row starts.  They overlap the neighbouring chunks, which write
@@ -486,7 +486,7 @@ __global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
     const uint32_t upe = a.units_per_elem;
 
     {
-        // Workgroup-uniform fast path: the whole 32 KiB tile lies inside one tensor (most of a
+        // Workgroup-uniform fast path: the whole tile (8 or 16 KiB) lies inside one tensor (most of a
         // bucket's bytes are in tensors much larger than a tile) and inside the flat buffer.
         const uint64_t tile_first = block_c0 * VU;
         const uint64_t tile_end = tile_first + (uint64_t)(kFlatThreads * kUnroll) * VU;
