@@ -474,6 +474,32 @@ def test_transpose_large_aligned_bf16_tiles():
         assert torch.equal(back.view(torch.int16), x.view(torch.int16)), shape
 
 
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.float32, torch.float64])
+def test_transposes_whose_rows_are_a_multiple_of_8k_apart(dtype):
+    # at these pitches the tile walk is rotated per eighth of the tiles; shapes with ragged edges, batches,
+    # fewer and more c-groups than eight, and eighths that end in the middle of a row of groups
+    es = torch.empty(0, dtype=dtype).element_size()
+    g = torch.Generator(device=DEV).manual_seed(16)
+    for batch, rows, pitch_bytes in [(1, 1000, 8192), (3, 700, 8192), (1, 2100, 16384), (5, 300, 24576), (2, 515, 32768),
+                                     (1, 4100, 8192), (7, 129, 16384)]:
+        cols = pitch_bytes // es
+        x = torch.randint(0, 255, (batch, rows, cols), dtype=torch.uint8, generator=g, device=DEV).to(dtype) \
+            if dtype != torch.uint8 else torch.randint(0, 255, (batch, rows, cols), dtype=torch.uint8, generator=g, device=DEV)
+        if dtype.is_floating_point:
+            x = x * 1.5 - 100
+        for view in (x.transpose(1, 2), x.transpose(1, 2)[:, 3:, 1:]):
+            s = Slice.of_tensor(view)
+            out = staging.pack(view, s)
+            sync()
+            assert torch.equal(out.view(view.shape), view.contiguous()), (dtype, batch, rows, pitch_bytes)
+            back = torch.zeros_like(x)
+            staging.unpack(back, s, out)
+            sync()
+            want = torch.zeros_like(x)
+            want.transpose(1, 2)[:, view.shape[1] * -1:, view.shape[2] * -1:] = view
+            assert torch.equal(back, want), (dtype, batch, rows, pitch_bytes)
+
+
 def test_stream_send_tensor_semantics():
     from monarch_amd.reduce import Factory
     from monarch_amd.send_tensor import route, stream_send_tensor
