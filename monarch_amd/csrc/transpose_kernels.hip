@@ -25,6 +25,7 @@ struct TransArgs {
     uint32_t rotate;    // rotate the c-groups of each eighth of the walk against the previous one (see the host side)
     uint32_t qgroups;   // ceil(qtiles / group)
     uint64_t rows_per_eighth;  // ceil(nbatch * qgroups / 8)
+    uint32_t aligned_stores;  // every 16-byte store of this launch is 16-byte aligned
     uint32_t group;    // tiles are walked in group x group blocks so that concurrently running workgroups
     uint32_t cgroups;  // touch neighbouring segments on BOTH sides (DRAM row locality); cgroups = ceil(ctiles/group)
     int n_inner;       // dimensions after c (decode q -> memory offset), outermost first
@@ -42,6 +43,14 @@ struct TransArgs {
 // between neighbouring workgroups matter (measured: bf16 4.4 TB/s cached vs 2.4 TB/s with nt).
 template <typename T> __device__ __forceinline__ T ldg(const T* p) { return *p; }
 template <typename T> __device__ __forceinline__ void stg(T* p, T v) { *p = v; }
+// A tile row stored to HBM.  Rows that start on 16-byte boundaries go out write-through: switched on and off in
+// turn on one GPU over eleven shapes and both directions, +0.014 of peak on average for fp32 (-0.003 to +0.029) and
+// +0.006 for bf16.  Rows that do not are written through the cache, which combines the partial lines that
+// neighbouring tiles share.
+__device__ __forceinline__ void tstore(void* p, const u32x4& v, bool write_through) {
+    if (write_through) asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+    else *static_cast<u32x4_unaligned*>(p) = v;
+}
 
 template <typename T, int TILE, bool PACK>
 __global__ __launch_bounds__(kThreads) void slice_transpose_kernel(TransArgs a) {
@@ -275,8 +284,8 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
                         lo[k] = (w[2 * k] & 0xffffu) | (w[2 * k + 1] << 16);
                         hi[k] = (w[2 * k] >> 16) | (w[2 * k + 1] & 0xffff0000u);
                     }
-                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)c * a.Q + v16 * E) = lo;
-                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E) = hi;
+                    tstore(packed_tile + (uint64_t)c * a.Q + v16 * E, lo, a.aligned_stores);
+                    tstore(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E, hi, a.aligned_stores);
                 }
             } else {
 #pragma unroll
@@ -285,7 +294,7 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
                     Vec o;
 #pragma unroll
                     for (int j = 0; j < E; ++j) o.e[j] = tile[at(qv * E + j, cc)];
-                    *reinterpret_cast<u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + qv * E) = o.v;
+                    tstore(packed_tile + (uint64_t)cc * a.Q + qv * E, o.v, a.aligned_stores);
                 }
             }
         } else {
@@ -328,7 +337,7 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
             for (int p = 0; p < PASSES; ++p) {
                 const int q = r16 + ROWS * p;
                 const u32x4 o = *reinterpret_cast<const u32x4*>(&tile[at(q, v16 * E)]);
-                *reinterpret_cast<u32x4_unaligned*>(mem_tile + s_off[q] + v16 * E) = o;
+                tstore(mem_tile + s_off[q] + v16 * E, o, a.aligned_stores);
             }
         }
         return;
@@ -432,6 +441,18 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     // 16 0.65 of peak; 2-byte elements do best at 8.
     a.group = big ? 8 : (unit == 4 || unit == 8) ? 16 : vec ? 8 : 4;
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
+    if (vec) {
+        // 16-byte stores land on 16-byte boundaries when the rows of the side that is written do
+        const uint64_t e16 = 16 / unit;  // elements per vector
+        if (PACK) {
+            a.aligned_stores = ((uintptr_t)packed & 15u) == 0 && Q % e16 == 0;
+        } else {
+            bool ok = ((uintptr_t)base & 15u) == 0 && c.offset % e16 == 0 && Sc % e16 == 0;
+            for (int k = 0; ok && k < c.ndim; ++k)
+                if (k != cd && c.dims[k].stride % e16 != 0) ok = false;
+            a.aligned_stores = ok;
+        }
+    }
     {
         // Rows that are a multiple of 8 KiB apart share at most two of the 64 positions at which HBM interleaves
         // 256-byte pieces (a bare walk down such rows reads 4.0 TB/s at a 16 KiB pitch against 6.4 TB/s at
