@@ -33,8 +33,8 @@ MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled 
     "c2p_unpack": 100_663_570, "c3_pack": 234_865_833, "c3_unpack": 234_865_798, "c4": 603_822_351,
     "c4_slots": 603_823_951, "c5_flat_pack": 3_166_117_170, "c5_quantize": 2_384_067_112,
     "c5_dequant": 7_127_836_847, "c5_flat_unpack": 6_014_993_348, "c5_dequant_many8": 12_779_917_743,
-    "c5_quantize_bucket": 2_374_369_255, "c5_dequant_bucket": 7_176_538_659, "tr_f32_pack": 536_837_788,
-    "tr_f32_unpack": 536_847_163, "tr_bf16_pack": 268_456_511,
+    "c5_quantize_bucket": 2_374_369_255, "c5_dequant_bucket": 7_176_538_659, "tr_f32_pack": 536_871_660,
+    "tr_f32_unpack": 536_871_869, "tr_bf16_pack": 268_488_359,
 }
 
 
