@@ -29,12 +29,12 @@ METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
 # None until a counter run exists for the workload.
 MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_870_600, "c2_inplace": 452_870_787, "c2_separate": 452_869_716, "c2p_pack": 100_663_296,
-    "c2p_unpack": 100_663_570, "c3_pack": 234_865_833, "c3_unpack": 234_865_798, "c4": 603_822_351,
-    "c4_slots": 603_823_951, "c5_flat_pack": 3_166_117_170, "c5_quantize": 2_384_067_112,
-    "c5_dequant": 7_127_836_847, "c5_flat_unpack": 6_014_993_348, "c5_dequant_many8": 12_779_917_743,
-    "c5_quantize_bucket": 2_374_369_255, "c5_dequant_bucket": 7_176_538_659, "tr_f32_pack": 536_871_660,
-    "tr_f32_unpack": 536_871_869, "tr_bf16_pack": 268_488_359,
+    "c2": 452_868_627, "c2_inplace": 452_868_813, "c2_separate": 452_867_743, "c2p_pack": 100_663_296,
+    "c2p_unpack": 100_663_323, "c3_pack": 234_865_257, "c3_unpack": 234_865_222, "c4": 603_819_720,
+    "c4_slots": 603_821_319, "c5_flat_pack": 3_166_109_361, "c5_quantize": 2_384_059_401,
+    "c5_dequant": 7_127_817_329, "c5_flat_unpack": 6_014_978_770, "c5_dequant_many8": 12_779_870_515,
+    "c5_quantize_bucket": 2_374_361_487, "c5_dequant_bucket": 7_176_519_083, "tr_f32_pack": 536_870_344,
+    "tr_f32_unpack": 536_870_553, "tr_bf16_pack": 268_487_701, "tr_bf16_unpack": 268_483_118,
 }
 
 
@@ -589,6 +589,7 @@ WORKLOADS = {
     "tr_f32_pack": lambda t: wl_transpose(t, "f32", False),
     "tr_f32_unpack": lambda t: wl_transpose(t, "f32", True),
     "tr_bf16_pack": lambda t: wl_transpose(t, "bf16", False),
+    "tr_bf16_unpack": lambda t: wl_transpose(t, "bf16", True),
     "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
     "c5_quantize": lambda t: wl_c5(t, "quantize"),
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
