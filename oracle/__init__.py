@@ -54,18 +54,24 @@ class _CSlice(C.Structure):
 _lib = None
 
 
+def load(path: str):
+    """A handle on an oracle build at ``path`` with the non-int return types declared."""
+    h = C.CDLL(path)
+    h.o_slice_len.restype = C.c_uint64
+    h.o_slice_iter.restype = C.c_uint64
+    h.o_mesh_ranks_for_dims.restype = C.c_int64
+    h.o_e4m3fn_encode.restype = C.c_uint8
+    h.o_e4m3fn_encode.argtypes = [C.c_float, C.c_int]
+    h.o_e4m3fn_decode.restype = C.c_float
+    h.o_e4m3fn_decode.argtypes = [C.c_uint8]
+    return h
+
+
 def lib():
     global _lib
     if _lib is None:
         build()
-        _lib = C.CDLL(_SO)
-        _lib.o_slice_len.restype = C.c_uint64
-        _lib.o_slice_iter.restype = C.c_uint64
-        _lib.o_mesh_ranks_for_dims.restype = C.c_int64
-        _lib.o_e4m3fn_encode.restype = C.c_uint8
-        _lib.o_e4m3fn_encode.argtypes = [C.c_float, C.c_int]
-        _lib.o_e4m3fn_decode.restype = C.c_float
-        _lib.o_e4m3fn_decode.argtypes = [C.c_uint8]
+        _lib = load(_SO)
     return _lib
 
 

@@ -321,3 +321,96 @@ def test_fp8_dequant_accumulate_and_flat():
     outs = oracle.flat_unpack(acc, offsets)
     assert [o.size for o in outs] == sizes
     assert np.array_equal(np.concatenate(outs), acc)
+
+
+# ---------------- pins for f64 reduce and for bf16 / Avg reduce-scatter ----------------
+# Reference semantics: ncclReduceScatter's flat-chunk rule, torch-sys-cuda/src/nccl.rs:683,693-701
+# (output r = chunk r of the elementwise reduction over the group), Avg = sum / group size
+# (nccl.rs:285-292).  The expected values below are built from explicit member-order adds in
+# torch / numpy, never from the oracle's own formula, with n_in != n_out so that dividing by the
+# number of outputs instead of the number of group members fails, and with values whose partial
+# sums are not representable in bf16 so that rounding after every add fails.
+
+@pytest.mark.parametrize("n", [1, 2, 3, 7])
+def test_reduce_f64_left_to_right(n):
+    rng = np.random.default_rng(640 + n)
+    # magnitudes spread over 30 binades: the order of the adds changes the low bits
+    ins = [(rng.uniform(-1, 1, size=2053) * 10.0 ** rng.integers(-15, 15, size=2053)).astype(np.float64)
+           for _ in range(n)]
+    acc = ins[0].copy()
+    for x in ins[1:]:
+        acc = acc + x                      # IEEE double adds in member order
+    got = oracle.reduce(ins, SUM)
+    assert got.dtype == np.float64 and np.array_equal(got.view(np.uint64), acc.view(np.uint64))
+    got = oracle.reduce(ins, AVG)
+    assert np.array_equal(got.view(np.uint64), (acc / np.float64(n)).view(np.uint64))
+    # the sum is a double sum, not a float one: it keeps bits an fp32 accumulator would drop
+    if n > 1:
+        a = np.array([1.0, 2.0**-40], dtype=np.float64)
+        assert oracle.reduce([a, a[::-1].copy()], SUM).tolist() == [1.0 + 2.0**-40] * 2
+    # in place on member 0
+    first = ins[0].copy()
+    oracle.reduce([first] + ins[1:], AVG, out=first)
+    assert np.array_equal(first, acc / np.float64(n))
+
+
+def _strided_inputs(n_in, rows, cols, pitch, slab, seed, bf16):
+    """n_in flat storages holding a [rows, cols] tensor at row pitch `pitch` starting at `slab`."""
+    g = torch.Generator().manual_seed(seed)
+    ts = []
+    for _ in range(n_in):
+        t = torch.randn(slab + rows * pitch + 5, generator=g)
+        ts.append(t.bfloat16() if bf16 else t)
+    return ts
+
+
+@pytest.mark.parametrize("op", [SUM, AVG])
+@pytest.mark.parametrize("n_in,n_out", [(3, 2), (5, 4), (2, 6)])
+def test_reduce_scatter_bf16_member_order(op, n_in, n_out):
+    rows, cols, pitch, slab = 12, 24, 40, 7
+    ts = _strided_inputs(n_in, rows, cols, pitch, slab, 900 + 10 * n_in + n_out, bf16=True)
+    in_view = OSlice(slab, [rows, cols], [pitch, 1])
+    w = cols // n_out
+    out_views = [OSlice(k * w, [rows, w], [cols, 1]) for k in range(n_out)]
+    outs = oracle.reduce_scatter([bits(t) for t in ts], in_view, out_views, op)
+    # explicit adds in member order on the strided views, fp32 accumulate, one rounding at the end
+    views = [torch.as_strided(t, (rows, cols), (pitch, 1), slab).float() for t in ts]
+    acc = views[0].clone()
+    for v in views[1:]:
+        acc = acc + v
+    if op == AVG:
+        acc = acc / n_in
+    want = acc.bfloat16()
+    for k in range(n_out):
+        assert np.array_equal(outs[k], bits(want[:, k * w:(k + 1) * w].contiguous().flatten())), (k, op)
+    if n_in > 2:
+        # rounding to bf16 after every add gives another answer on these inputs: the pin can tell
+        per_add = views[0].bfloat16()
+        for v in views[1:]:
+            per_add = (per_add.float() + v).bfloat16()
+        assert not torch.equal(per_add, acc.bfloat16() if op == SUM else (acc * n_in).bfloat16())
+
+
+@pytest.mark.parametrize("n_in,n_out", [(3, 2), (5, 4), (2, 6)])
+def test_reduce_scatter_f32_avg_member_order(n_in, n_out):
+    rows, cols, pitch, slab = 12, 24, 40, 7
+    ts = _strided_inputs(n_in, rows, cols, pitch, slab, 700 + 10 * n_in + n_out, bf16=False)
+    in_view = OSlice(slab, [rows, cols], [pitch, 1])
+    # the flat-chunk rule of nccl.rs:683,693-701 on the reduced tensor: output r = elements [r*c, (r+1)*c)
+    c = rows * cols // n_out
+    out_views = [OSlice(r * c, [c], [1]) for r in range(n_out)]
+    outs = oracle.reduce_scatter([t.numpy() for t in ts], in_view, out_views, AVG)
+    views = [torch.as_strided(t, (rows, cols), (pitch, 1), slab) for t in ts]
+    acc = views[0].clone()
+    for v in views[1:]:
+        acc = acc + v
+    want = (acc / n_in).flatten()
+    for r in range(n_out):
+        assert np.array_equal(outs[r], want[r * c:(r + 1) * c].numpy()), r
+    assert not torch.equal(acc / n_out, acc / n_in)
+    # and a column-block scatter of the same average
+    w = cols // n_out
+    outs = oracle.reduce_scatter([t.numpy() for t in ts], in_view,
+                                 [OSlice(k * w, [rows, w], [cols, 1]) for k in range(n_out)], AVG)
+    for k in range(n_out):
+        assert np.array_equal(outs[k], (acc / n_in)[:, k * w:(k + 1) * w].contiguous().flatten().numpy())
