@@ -30,6 +30,17 @@ pub struct mhip_slice_t {
     pub strides: *const u64,
 }
 
+/// `monarch_rdma::RdmaBuffer` without its NIC fields: `{addr, size}` of a registered byte range.
+#[repr(C)]
+#[derive(Debug, Clone, Copy)]
+pub struct mhip_rdma_buffer_t {
+    pub addr: *mut c_void,
+    pub size: usize,
+}
+
+/// `Option::None` of `WorkerActor::send_tensor`'s `from_rank` / `to_rank`.
+pub const MHIP_NO_RANK: u64 = u64::MAX;
+
 pub mod status {
     pub const SUCCESS: i32 = 0;
     pub const INVALID_DIMS: i32 = 10001;
@@ -54,6 +65,9 @@ pub mod status {
     pub const UNSUPPORTED_OP: i32 = 10202;
     pub const TOO_MANY_INPUTS: i32 = 10203;
     pub const UNSUPPORTED_BLOCK: i32 = 10204;
+    pub const BUFFER_TOO_SMALL: i32 = 10205;
+    pub const MESH_DIM_LENGTH_MISMATCH: i32 = 10301;
+    pub const MESH_DIM_MISSING: i32 = 10302;
 }
 
 /// `c10::ScalarType` numbering, as carried by `monarch_messages::worker::Factory::dtype`.
@@ -109,6 +123,14 @@ extern "C" {
     pub fn mhip_flat_unpack(d_tensors: *const *mut c_void, flat: *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_reduce(out: *mut c_void, input: *const *const c_void, n: u32, numel: u64, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
     pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *const c_void, in_view: *const mhip_slice_t, in_numel: u64, n_in: u32, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_stack(out: *mut c_void, input: *const *const c_void, n: u32, numel: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_stack_scatter(out: *mut c_void, input: *const *const c_void, n: u32, rank: u32, numel: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_buffer_read_into(local: *const mhip_rdma_buffer_t, remote: *const mhip_rdma_buffer_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_buffer_write_from(local: *const mhip_rdma_buffer_t, remote: *const mhip_rdma_buffer_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_buffer_transfer(dst: *mut c_void, src: *const c_void, bytes: usize, max_segment_bytes: usize, stream: mhip_stream_t, segments: *mut u32) -> c_int;
+    pub fn mhip_send_tensor_route(from_ranks: *const mhip_slice_t, to_ranks: *const mhip_slice_t, rank: u64, from_rank: *mut u64, to_rank: *mut u64) -> c_int;
+    pub fn mhip_to_mesh_from_ranks(slicing_names: *const *const c_char, slicing: *const mhip_slice_t, mesh_names: *const *const c_char, mesh_sizes: *const u64, mesh_ndim: u32, out_sizes: *mut u64, out_strides: *mut u64, out_ndim: *mut u32, broadcast_dims: *mut u32, n_broadcast: *mut u32, culprit: *mut u32) -> c_int;
+    pub fn mhip_send_tensor(result: *mut c_void, result_bytes: usize, src_base: *const c_void, src_view: *const mhip_slice_t, elem_size: u32, staging: *mut c_void, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_quantize(q: *mut u8, scales: *mut f32, x_bf16: *const c_void, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate(acc: *mut f32, q: *const u8, scales: *const f32, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_many(acc: *mut f32, q: *const *const u8, scales: *const *const f32, n: u32, numel: u64, block: u32, overwrite: c_int, stream: mhip_stream_t) -> c_int;

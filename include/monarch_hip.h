@@ -59,7 +59,11 @@ enum {
     MHIP_ERR_INVALID_ARGUMENT = 10201,
     MHIP_ERR_UNSUPPORTED_OP = 10202,
     MHIP_ERR_TOO_MANY_INPUTS = 10203,
-    MHIP_ERR_UNSUPPORTED_BLOCK = 10204
+    MHIP_ERR_UNSUPPORTED_BLOCK = 10204,
+    MHIP_ERR_BUFFER_TOO_SMALL = 10205,
+    /* Tensor.to_mesh checks, python/monarch/common/tensor.py:426-437 */
+    MHIP_ERR_MESH_DIM_LENGTH_MISMATCH = 10301,
+    MHIP_ERR_MESH_DIM_MISSING = 10302
 };
 
 /* Text for any status this library returns (hipGetErrorString for HIP codes);
@@ -193,10 +197,13 @@ int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d
  * (torch-sys-cuda/src/nccl.rs:464-489) as StreamActor::reduce uses it
  * (monarch_tensor_worker/src/stream.rs:1437-1462).  out may coincide with exactly one of
  * the inputs (the in-place form); any other overlap is undefined.  Floating types accumulate in fp32 (f64 in f64)
- * in rank order and round once; Avg divides the sum by n.  Integer Sum wraps.
+ * in rank order and round once; Avg divides the sum by n.  Integer Sum and Prod wrap.
+ * Max / Min keep the accumulator on ties and skip NaN operands unless all are NaN (fmaxf / fminf,
+ * which is how NCCL's own kernels define ncclMax / ncclMin; NCCL is outside the reference tree);
+ * I8 / I32 / I64 compare as signed, U8 as unsigned.
  * Argument checks follow nccl.rs:300-316,474-476: null pointer -> UNDEFINED_TENSOR,
- * unknown dtype -> INVALID_DATA_TYPE, fp8 dtype -> FLOAT8_REDUCTION; ops other than
- * Sum/Avg -> UNSUPPORTED_OP; n > 64 -> TOO_MANY_INPUTS. */
+ * unknown dtype -> INVALID_DATA_TYPE, fp8 dtype -> FLOAT8_REDUCTION; an op outside
+ * nccl.rs:285-292, or Avg on an integer dtype -> UNSUPPORTED_OP; n > 64 -> TOO_MANY_INPUTS. */
 int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, int dtype, int op,
                 mhip_stream_t stream);
 
@@ -210,6 +217,78 @@ int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, in
 int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32_t n_out,
                         const void* const* in, const mhip_slice_t* in_view, uint64_t in_numel,
                         uint32_t n_in, int dtype, int op, mhip_stream_t stream);
+
+/* Reduction::Stack without scatter: the data movement of Communicator::all_gather_into_tensor as
+ * StreamActor::reduce uses it (monarch_tensor_worker/src/stream.rs:1408-1417; result shape
+ * [n, *factory.size], the reference's test is torch-sys-cuda/src/nccl.rs:927-959):
+ * out[g * numel + i] = in[g][i] for the n <= 64 members' tensors, in one launch.  out must not
+ * overlap an input. */
+int mhip_stack(void* out, const void* const* in, uint32_t n, uint64_t numel, uint32_t elem_size,
+               mhip_stream_t stream);
+/* Reduction::Stack with scatter: Communicator::all_to_all_single (nccl.rs:760-812; stream.rs:1381-1399)
+ * as member `rank` sees it, every member's tensor holding numel elements cut into n equal chunks of
+ * c = numel / n:  out[g * c + i] = in[g][rank * c + i].  numel % n != 0 -> INPUT_SIZE_MISMATCH.
+ * out may be in[rank] (the in-place form); chunks g != rank of that tensor are then overwritten. */
+int mhip_stack_scatter(void* out, const void* const* in, uint32_t n, uint32_t rank, uint64_t numel,
+                       uint32_t elem_size, mhip_stream_t stream);
+
+/* ====================================================================== */
+/* RdmaBuffer transfers and SendTensor                                     */
+/* ====================================================================== */
+
+/* RdmaBuffer (monarch_rdma/src/rdma_components.rs:94-102) without its NIC fields (owner, mr_id,
+ * lkey, rkey): a contiguous registered byte range.  Owns nothing. */
+typedef struct {
+    void* addr;
+    size_t size;
+} mhip_rdma_buffer_t;
+
+/* local.read_into(remote), rdma_components.rs:117-137 -> RdmaQueuePair::put (:842-858): local.size bytes
+ * go from local.addr to remote.addr.  On one GPU the transport is a device copy on `stream`, posted as
+ * one copy per work request: a request's length is a 32-bit field (rdma_components.rs:1041,1063), so
+ * transfers are cut into requests of at most 2^32 - 16 bytes instead of being truncated.
+ * local.size > remote.size -> BUFFER_TOO_SMALL (a NIC refuses a write past the remote region). */
+int mhip_buffer_read_into(const mhip_rdma_buffer_t* local, const mhip_rdma_buffer_t* remote,
+                          mhip_stream_t stream);
+/* local.write_from(remote), rdma_components.rs:152-171 -> RdmaQueuePair::get (:986-1002): local.size
+ * bytes go from remote.addr to local.addr. */
+int mhip_buffer_write_from(const mhip_rdma_buffer_t* local, const mhip_rdma_buffer_t* remote,
+                           mhip_stream_t stream);
+/* The request walk both calls share: `bytes` bytes from src to dst in requests of at most
+ * max_segment_bytes (0, or anything above it, means the wire limit of 2^32 - 16); *segments, when not
+ * NULL, receives the number of requests posted. */
+int mhip_buffer_transfer(void* dst, const void* src, size_t bytes, size_t max_segment_bytes,
+                         mhip_stream_t stream, uint32_t* segments);
+
+#define MHIP_NO_RANK UINT64_MAX
+/* WorkerActor::send_tensor's routing (monarch_tensor_worker/src/lib.rs:722-731): the i-th rank of
+ * from_ranks sends to the i-th rank of to_ranks.  *to_rank = to_ranks.get(from_ranks.index(rank)),
+ * *from_rank = from_ranks.get(to_ranks.index(rank)), each MHIP_NO_RANK when `rank` is not in the
+ * respective slice (Option::None in the reference). */
+int mhip_send_tensor_route(const mhip_slice_t* from_ranks, const mhip_slice_t* to_ranks, uint64_t rank,
+                           uint64_t* from_rank, uint64_t* to_rank);
+/* Tensor.to_mesh's client-side check (python/monarch/common/tensor.py:417-438): for every dimension
+ * of the destination mesh (names and sizes, in mesh order) that the source slicing names, its size
+ * must match; the from_ranks slice is {slicing.offset, out_sizes, out_strides} with *out_ndim entries;
+ * destination dimensions the slicing does not name are broadcast dimensions (indices into the mesh).
+ * Errors: MESH_DIM_LENGTH_MISMATCH (*culprit = the mesh dimension), MESH_DIM_MISSING (*culprit = the
+ * first slicing dimension the destination lacks).  out_sizes / out_strides hold slicing->ndim
+ * entries, broadcast_dims mesh_ndim entries; culprit may be NULL. */
+int mhip_to_mesh_from_ranks(const char* const* slicing_names, const mhip_slice_t* slicing,
+                            const char* const* mesh_names, const uint64_t* mesh_sizes,
+                            uint32_t mesh_ndim, uint64_t* out_sizes, uint64_t* out_strides,
+                            uint32_t* out_ndim, uint32_t* broadcast_dims, uint32_t* n_broadcast,
+                            uint32_t* culprit);
+/* StreamActor::send_tensor (monarch_tensor_worker/src/stream.rs:1470-1560) for data on one GPU.  The
+ * sender's tensor may be any view (NCCL point-to-point tolerates non-contiguous tensors,
+ * torch-sys-cuda/src/nccl.rs:300-316): it is gathered in Slice::iter order into `staging`
+ * (len * elem_size bytes, what an RdmaBuffer moves), and those bytes are transferred into `result`,
+ * the receiver's fresh contiguous tensor of factory.size (stream.rs:1533-1538).  staging == NULL is
+ * the local case from_rank == to_rank (stream.rs:1497-1516): a defensive copy straight into result.
+ * result_bytes != len * elem_size -> OUTPUT_SIZE_MISMATCH. */
+int mhip_send_tensor(void* result, size_t result_bytes, const void* src_base,
+                     const mhip_slice_t* src_view, uint32_t elem_size, void* staging,
+                     mhip_stream_t stream);
 
 /* ====================================================================== */
 /* Block-scaled fp8 (e4m3fn) transfer codec                                 */

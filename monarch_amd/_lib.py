@@ -39,6 +39,10 @@ ERR_INVALID_ARGUMENT = 10201
 ERR_UNSUPPORTED_OP = 10202
 ERR_TOO_MANY_INPUTS = 10203
 ERR_UNSUPPORTED_BLOCK = 10204
+ERR_BUFFER_TOO_SMALL = 10205
+ERR_MESH_DIM_LENGTH_MISMATCH = 10301
+ERR_MESH_DIM_MISSING = 10302
+NO_RANK = (1 << 64) - 1
 
 STATUS_NAMES = {
     ERR_INVALID_DIMS: "InvalidDims", ERR_NONRECTANGULAR_SHAPE: "NonrectangularShape",
@@ -52,6 +56,8 @@ STATUS_NAMES = {
     ERR_INPUT_SIZE_MISMATCH: "InputSizeMismatch", ERR_UNDEFINED_TENSOR: "UndefinedTensor",
     ERR_INVALID_ARGUMENT: "InvalidArgument", ERR_UNSUPPORTED_OP: "UnsupportedOp",
     ERR_TOO_MANY_INPUTS: "TooManyInputs", ERR_UNSUPPORTED_BLOCK: "UnsupportedBlock",
+    ERR_BUFFER_TOO_SMALL: "BufferTooSmall", ERR_MESH_DIM_LENGTH_MISMATCH: "MeshDimLengthMismatch",
+    ERR_MESH_DIM_MISSING: "MeshDimMissing",
 }
 
 # dtype codes (c10::ScalarType numbering)
@@ -75,6 +81,10 @@ class MhipError(RuntimeError):
         super().__init__(f"{self.name} ({status}): {text}")
 
 
+class RdmaBufferC(C.Structure):
+    _fields_ = [("addr", C.c_void_p), ("size", C.c_size_t)]
+
+
 class SliceC(C.Structure):
     _fields_ = [("offset", C.c_uint64), ("ndim", C.c_uint32),
                 ("sizes", C.POINTER(C.c_uint64)), ("strides", C.POINTER(C.c_uint64))]
@@ -85,6 +95,8 @@ _u32p = C.POINTER(C.c_uint32)
 _slicep = C.POINTER(SliceC)
 _vp = C.c_void_p
 _vpp = C.POINTER(C.c_void_p)
+_bufp = C.POINTER(RdmaBufferC)
+_cpp = C.POINTER(C.c_char_p)
 
 # name -> (restype, argtypes); mirrors include/monarch_hip.h declaration by declaration
 SIGNATURES = {
@@ -116,6 +128,14 @@ SIGNATURES = {
     "mhip_reduce": (C.c_int, [_vp, _vpp, C.c_uint32, C.c_uint64, C.c_int, C.c_int, _vp]),
     "mhip_reduce_scatter": (C.c_int, [_vpp, _slicep, C.c_uint32, _vpp, _slicep, C.c_uint64, C.c_uint32,
                                       C.c_int, C.c_int, _vp]),
+    "mhip_stack": (C.c_int, [_vp, _vpp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
+    "mhip_stack_scatter": (C.c_int, [_vp, _vpp, C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
+    "mhip_buffer_read_into": (C.c_int, [_bufp, _bufp, _vp]),
+    "mhip_buffer_write_from": (C.c_int, [_bufp, _bufp, _vp]),
+    "mhip_buffer_transfer": (C.c_int, [_vp, _vp, C.c_size_t, C.c_size_t, _vp, _u32p]),
+    "mhip_send_tensor_route": (C.c_int, [_slicep, _slicep, C.c_uint64, _u64p, _u64p]),
+    "mhip_to_mesh_from_ranks": (C.c_int, [_cpp, _slicep, _cpp, _u64p, C.c_uint32, _u64p, _u64p, _u32p, _u32p, _u32p, _u32p]),
+    "mhip_send_tensor": (C.c_int, [_vp, C.c_size_t, _vp, _slicep, C.c_uint32, _vp, _vp]),
     "mhip_fp8_quantize": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int, _vp]),

@@ -309,7 +309,7 @@ int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_ten
     const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_quantize_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0, hs, q,
+    MHIP_LAUNCH(fp8_quantize_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0, hs, q,
                        scales, a);
     return launch_status();
 }
@@ -331,7 +331,7 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
     const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0,
+    MHIP_LAUNCH(fp8_dequant_accumulate_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0,
                        hs, q, scales, a);
     return launch_status();
 }
@@ -361,7 +361,7 @@ int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const ui
     const uint64_t cap = max_workgroups(kBucketThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_dequant_accumulate_bucket_many_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads),
+    MHIP_LAUNCH(fp8_dequant_accumulate_bucket_many_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads),
                        0, hs, p);
     return launch_status();
 }

@@ -210,10 +210,10 @@ static void launch_dequant_many(DequantManyArgs& a, hipStream_t hs) {
     const uint64_t cap = max_workgroups(THREADS);
     const dim3 grid((uint32_t)(a.ntiles > cap ? cap : a.ntiles)), blockdim(THREADS);
     switch (a.n) {
-        case 2: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<2, THREADS>), grid, blockdim, 0, hs, a); break;
-        case 4: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<4, THREADS>), grid, blockdim, 0, hs, a); break;
-        case 8: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<8, THREADS>), grid, blockdim, 0, hs, a); break;
-        default: hipLaunchKernelGGL((fp8_dequant_accumulate_many_kernel<0, THREADS>), grid, blockdim, 0, hs, a); break;
+        case 2: MHIP_LAUNCH((fp8_dequant_accumulate_many_kernel<2, THREADS>), grid, blockdim, 0, hs, a); break;
+        case 4: MHIP_LAUNCH((fp8_dequant_accumulate_many_kernel<4, THREADS>), grid, blockdim, 0, hs, a); break;
+        case 8: MHIP_LAUNCH((fp8_dequant_accumulate_many_kernel<8, THREADS>), grid, blockdim, 0, hs, a); break;
+        default: MHIP_LAUNCH((fp8_dequant_accumulate_many_kernel<0, THREADS>), grid, blockdim, 0, hs, a); break;
     }
 }
 
@@ -235,7 +235,7 @@ int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t nu
     const uint64_t cap = max_workgroups(kQuantThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kQuantThreads), 0, hs, q, scales,
+    MHIP_LAUNCH(fp8_quantize_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kQuantThreads), 0, hs, q, scales,
                        static_cast<const uint16_t*>(x_bf16), numel, nblocks);
     return launch_status();
 }
@@ -250,7 +250,7 @@ int mhip_fp8_dequant_accumulate(float* acc, const uint8_t* q, const float* scale
     const uint64_t cap = max_workgroups(kDeqThreads);
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
-    hipLaunchKernelGGL(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kDeqThreads), 0,
+    MHIP_LAUNCH(fp8_dequant_accumulate_kernel, dim3((uint32_t)(ntiles > cap ? cap : ntiles)), dim3(kDeqThreads), 0,
                        hs, acc, q, scales, numel, ntiles);
     return launch_status();
 }

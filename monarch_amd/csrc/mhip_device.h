@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <tuple>
+#include <utility>
 
 #include "mhip_internal.h"
 
@@ -246,8 +248,37 @@ inline uint64_t max_launch_lanes() {
 }
 inline uint64_t max_workgroups(uint32_t lanes) { return max_launch_lanes() / lanes; }
 
+// Every kernel of the library is launched through MHIP_LAUNCH, which keeps the launch's own return value in a
+// thread-local slot; launch_status() reports and clears that slot.  The thread's HIP "last error" is neither
+// read nor reset, so an error an unrelated earlier call of the host application left there is not mistaken for a
+// failed launch, and the application still finds it afterwards.
+inline hipError_t& last_launch_error() {
+    static thread_local hipError_t e = hipSuccess;
+    return e;
+}
+
+template <typename... Params, typename... Args, size_t... I>
+inline hipError_t launch_kernel_impl(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                                     std::index_sequence<I...>, Args&&... args) {
+    std::tuple<Params...> values{static_cast<Params>(std::forward<Args>(args))...};  // converted to the kernel's own types
+    void* ptrs[] = {static_cast<void*>(&std::get<I>(values))...};
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds_bytes, stream);
+}
+
+template <typename... Params, typename... Args>
+inline void launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream, Args&&... args) {
+    static_assert(sizeof...(Params) == sizeof...(Args) && sizeof...(Params) > 0, "argument count");
+    const hipError_t e = launch_kernel_impl(kernel, grid, block, lds_bytes, stream, std::index_sequence_for<Params...>{},
+                                            std::forward<Args>(args)...);
+    if (e != hipSuccess) last_launch_error() = e;  // the first failure of a multi-piece launch stays visible
+}
+#define MHIP_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
+    ::mhip::launch_kernel(kernel, grid, block, lds_bytes, stream, __VA_ARGS__)
+
 inline int launch_status() {
-    hipError_t e = hipGetLastError();
+    hipError_t& slot = last_launch_error();
+    const hipError_t e = slot;
+    slot = hipSuccess;
     return e == hipSuccess ? MHIP_SUCCESS : (int)e;
 }
 

@@ -434,7 +434,7 @@ static bool launch_shift_copy(char* dst, const char* src, uint64_t nbytes, hipSt
     const uint64_t per_wg = (uint64_t)(kPackThreads / 64) * kShiftCopyRows * 64;
     *rc = launch_in_pieces((nvec + per_wg - 1) / per_wg, kPackThreads, 1, [&](uint64_t first, uint32_t count) {
         a.wg0 = first;
-        hipLaunchKernelGGL(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3(count), dim3(kPackThreads), 0, stream, a);
+        MHIP_LAUNCH(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3(count), dim3(kPackThreads), 0, stream, a);
     });
     return true;
 }
@@ -599,14 +599,14 @@ template <int U, bool PACK, int UNROLL>
 static void launch_whole_chunks_u(bool wide, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
     const dim3 block(kPackThreads);
     if (wide) {
-        hipLaunchKernelGGL((slice_copy_kernel<U, PACK, true, -1, UNROLL>), grid, block, 0, stream, a);
+        MHIP_LAUNCH((slice_copy_kernel<U, PACK, true, -1, UNROLL>), grid, block, 0, stream, a);
         return;
     }
     switch (ndim) {  // the common shapes get a decode without loops
-        case 0: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 0, UNROLL>), grid, block, 0, stream, a); break;
-        case 1: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 1, UNROLL>), grid, block, 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, 2, UNROLL>), grid, block, 0, stream, a); break;
-        default: hipLaunchKernelGGL((slice_copy_kernel<U, PACK, false, -1, UNROLL>), grid, block, 0, stream, a); break;
+        case 0: MHIP_LAUNCH((slice_copy_kernel<U, PACK, false, 0, UNROLL>), grid, block, 0, stream, a); break;
+        case 1: MHIP_LAUNCH((slice_copy_kernel<U, PACK, false, 1, UNROLL>), grid, block, 0, stream, a); break;
+        case 2: MHIP_LAUNCH((slice_copy_kernel<U, PACK, false, 2, UNROLL>), grid, block, 0, stream, a); break;
+        default: MHIP_LAUNCH((slice_copy_kernel<U, PACK, false, -1, UNROLL>), grid, block, 0, stream, a); break;
     }
 }
 
@@ -622,25 +622,25 @@ static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, 
     if constexpr (U < 16) {
         if (form == kShortRuns) {
             if (wide) {
-                hipLaunchKernelGGL((slice_gather_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
+                MHIP_LAUNCH((slice_gather_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
                 return;
             }
             switch (ndim) {
-                case 1: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
-                case 2: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
-                default: hipLaunchKernelGGL((slice_gather_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
+                case 1: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
+                case 2: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
+                default: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
             }
             return;
         }
         if (form == kRaggedRows) {
             if (wide) {
-                hipLaunchKernelGGL((slice_copy_ragged_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
+                MHIP_LAUNCH((slice_copy_ragged_kernel<U, PACK, true, -1>), grid, block, 0, stream, a);
                 return;
             }
             switch (ndim) {
-                case 1: hipLaunchKernelGGL((slice_copy_ragged_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
-                case 2: hipLaunchKernelGGL((slice_copy_ragged_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
-                default: hipLaunchKernelGGL((slice_copy_ragged_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
+                case 1: MHIP_LAUNCH((slice_copy_ragged_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
+                case 2: MHIP_LAUNCH((slice_copy_ragged_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
+                default: MHIP_LAUNCH((slice_copy_ragged_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
             }
             return;
         }
@@ -697,7 +697,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             const uint64_t wgs = (first.total + kCopyThreads - 1) / kCopyThreads;
             if (int rc = launch_in_pieces(wgs, kCopyThreads, 1, [&](uint64_t wg0, uint32_t count) {
                     const uint64_t c0 = wg0 * kCopyThreads;  // chunks already launched
-                    hipLaunchKernelGGL(contiguous_copy_kernel, dim3(count), dim3(kCopyThreads), 0, stream, dst + c0 * 16,
+                    MHIP_LAUNCH(contiguous_copy_kernel, dim3(count), dim3(kCopyThreads), 0, stream, dst + c0 * 16,
                                        src + c0 * 16, first.total - c0);
                 }))
                 return rc;
@@ -820,11 +820,11 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
         a.wg0 = wg0;
         const dim3 grid(count), block(kFlatThreads);
         switch (unit) {
-            case 1: hipLaunchKernelGGL((flat_copy_kernel<1, PACK>), grid, block, 0, hs, a); break;
-            case 2: hipLaunchKernelGGL((flat_copy_kernel<2, PACK>), grid, block, 0, hs, a); break;
-            case 4: hipLaunchKernelGGL((flat_copy_kernel<4, PACK>), grid, block, 0, hs, a); break;
-            case 8: hipLaunchKernelGGL((flat_copy_kernel<8, PACK>), grid, block, 0, hs, a); break;
-            default: hipLaunchKernelGGL((flat_copy_kernel<16, PACK>), grid, block, 0, hs, a); break;
+            case 1: MHIP_LAUNCH((flat_copy_kernel<1, PACK>), grid, block, 0, hs, a); break;
+            case 2: MHIP_LAUNCH((flat_copy_kernel<2, PACK>), grid, block, 0, hs, a); break;
+            case 4: MHIP_LAUNCH((flat_copy_kernel<4, PACK>), grid, block, 0, hs, a); break;
+            case 8: MHIP_LAUNCH((flat_copy_kernel<8, PACK>), grid, block, 0, hs, a); break;
+            default: MHIP_LAUNCH((flat_copy_kernel<16, PACK>), grid, block, 0, hs, a); break;
         }
     });
 }

@@ -1,4 +1,4 @@
-// Reduce (sum / avg) over the chunks one GPU holds, with and without scatter.
+// Reduce (sum / avg / prod / max / min) over the chunks one GPU holds, with and without scatter.
 //
 // HBM-bound: (n + 1) * numel * sizeof(T) bytes per call.  Each lane moves 16 bytes per
 // input per step; all n loads of a step are issued before the first add so that a
@@ -22,7 +22,12 @@ struct ReduceArgs {
     float scale;   // 1/n when n is a power of two and op is Avg (exact), else 0
     float divisor; // n as a float
     uint32_t xcd_contiguous;  // see inputs_alias()
+    uint32_t op;              // MHIP_OP_*, read by the kGeneric kernels only
 };
+
+// How a kernel combines: Sum and Avg (the hot ops) are compiled as plain adds; Prod / Max / Min share one
+// instantiation per type that switches on the (wave-uniform) op in the arguments.
+enum : int { kSum = 0, kAvg = 1, kGeneric = 2 };
 
 // ---- per-type vector traits: 16 bytes <-> accumulator lanes ----
 template <typename T> struct Vec;
@@ -112,6 +117,36 @@ template <typename UT> struct IntVec {
 template <> struct Vec<uint8_t> : IntVec<uint8_t> {};
 template <> struct Vec<uint32_t> : IntVec<uint32_t> {};
 template <> struct Vec<uint64_t> : IntVec<uint64_t> {};
+// signed flavours: Max / Min compare them as signed, Prod wraps like Sum does
+template <> struct Vec<int8_t> : IntVec<int8_t> {};
+template <> struct Vec<int32_t> : IntVec<int32_t> {};
+template <> struct Vec<int64_t> : IntVec<int64_t> {};
+
+// acc (op) x.  Max / Min keep the accumulator on ties (so the first of +0 / -0 in member order wins) and skip
+// NaN operands unless every operand is NaN, which is what ncclMax / ncclMin compute with fmaxf / fminf
+// (the op numbering is torch-sys-cuda/src/nccl.rs:285-292; NCCL itself is not part of the reference tree).
+// Integer Prod wraps (computed in the unsigned type of the same width).
+template <int MODE, typename A>
+__device__ __forceinline__ A combine(A acc, A x, uint32_t op) {
+    if constexpr (MODE != kGeneric) {
+        return acc + x;
+    } else if constexpr (std::is_floating_point<A>::value) {
+        switch (op) {
+            case MHIP_OP_PROD: return acc * x;
+            case MHIP_OP_MAX: return (x > acc || acc != acc) ? x : acc;
+            case MHIP_OP_MIN: return (x < acc || acc != acc) ? x : acc;
+            default: return acc + x;
+        }
+    } else {
+        using UA = typename std::make_unsigned<A>::type;
+        switch (op) {
+            case MHIP_OP_PROD: return (A)(UA)((UA)acc * (UA)x);
+            case MHIP_OP_MAX: return x > acc ? x : acc;
+            case MHIP_OP_MIN: return x < acc ? x : acc;
+            default: return (A)(UA)((UA)acc + (UA)x);
+        }
+    }
+}
 
 template <typename A> __device__ __forceinline__ A finish(A acc, bool avg, float scale, float divisor) {
     if constexpr (std::is_same<A, float>::value) {
@@ -151,7 +186,7 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block() {
     return blockIdx.x < per * 8 ? (blockIdx.x & 7u) * per + (blockIdx.x >> 3) : blockIdx.x;
 }
 
-template <typename T, int N, bool AVG>
+template <typename T, int N, int MODE>
 __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
     using VT = Vec<T>;
     using acc_t = typename VT::acc_t;
@@ -171,7 +206,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
                 acc_t x[V];
                 VT::widen(raw[r], x);
 #pragma unroll
-                for (int k = 0; k < V; ++k) acc[k] += x[k];
+                for (int k = 0; k < V; ++k) acc[k] = combine<MODE>(acc[k], x[k], a.op);
             }
         } else {
             VT::widen(load16_unaligned(static_cast<const char*>(a.in[0]) + v * 16), acc);
@@ -185,18 +220,18 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
                     acc_t x[V];
                     VT::widen(raw[j], x);
 #pragma unroll
-                    for (int k = 0; k < V; ++k) acc[k] += x[k];
+                    for (int k = 0; k < V; ++k) acc[k] = combine<MODE>(acc[k], x[k], a.op);
                 }
             }
             for (; r < a.n; ++r) {
                 acc_t x[V];
                 VT::widen(load16_unaligned(static_cast<const char*>(a.in[r]) + v * 16), x);
 #pragma unroll
-                for (int k = 0; k < V; ++k) acc[k] += x[k];
+                for (int k = 0; k < V; ++k) acc[k] = combine<MODE>(acc[k], x[k], a.op);
             }
         }
 #pragma unroll
-        for (int k = 0; k < V; ++k) acc[k] = finish(acc[k], AVG, a.scale, a.divisor);
+        for (int k = 0; k < V; ++k) acc[k] = finish(acc[k], MODE == kAvg, a.scale, a.divisor);
         store16_writethrough(static_cast<char*>(a.out) + v * 16, VT::narrow(acc));
     }
     // ragged tail: fewer than V elements, one lane each
@@ -204,8 +239,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
         const uint64_t i = nvec * V + threadIdx.x;
         if (threadIdx.x < V && i < a.numel) {
             acc_t acc = VT::widen1(a.in[0], i);
-            for (uint32_t r = 1; r < a.n; ++r) acc += VT::widen1(a.in[r], i);
-            VT::narrow1(a.out, i, finish(acc, AVG, a.scale, a.divisor));
+            for (uint32_t r = 1; r < a.n; ++r) acc = combine<MODE>(acc, VT::widen1(a.in[r], i), a.op);
+            VT::narrow1(a.out, i, finish(acc, MODE == kAvg, a.scale, a.divisor));
         }
     }
 }
@@ -223,6 +258,7 @@ struct ScatterArgs {
     float scale;
     float divisor;
     uint32_t xcd_contiguous;           // see inputs_alias()
+    uint32_t op;                       // MHIP_OP_*, read by the kGeneric kernels only
     DimsArg out_dims;                  // packed output index -> reduced-tensor index
     DimsArg in_dims;                   // reduced-tensor index -> input memory
 };
@@ -230,7 +266,7 @@ struct ScatterArgs {
 // VEC: a unit is 16 bytes (V elements) and never straddles a row of either view.
 // D: number of dimensions (outside the run) both decodes are compiled for; shorter views
 // are padded on the host.  D < 0 reads the counts from the arguments.
-template <typename T, bool VEC, bool AVG, bool WIDE, int D>
+template <typename T, bool VEC, int MODE, bool WIDE, int D>
 __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterArgs a) {
     using VT = Vec<T>;
     using acc_t = typename VT::acc_t;
@@ -262,22 +298,22 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
                     acc_t x[V];
                     VT::widen(raw[j], x);
 #pragma unroll
-                    for (int e = 0; e < V; ++e) acc[e] += x[e];
+                    for (int e = 0; e < V; ++e) acc[e] = combine<MODE>(acc[e], x[e], a.op);
                 }
             }
             for (; g < a.n_in; ++g) {
                 acc_t x[V];
                 VT::widen(load16_unaligned(static_cast<const char*>(a.in[g]) + loc * 16), x);
 #pragma unroll
-                for (int e = 0; e < V; ++e) acc[e] += x[e];
+                for (int e = 0; e < V; ++e) acc[e] = combine<MODE>(acc[e], x[e], a.op);
             }
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc[e] = finish(acc[e], AVG, a.scale, a.divisor);
+            for (int e = 0; e < V; ++e) acc[e] = finish(acc[e], MODE == kAvg, a.scale, a.divisor);
             store16_writethrough(static_cast<char*>(a.outs[k]) + t * 16, VT::narrow(acc));
         } else {
             acc_t acc = VT::widen1(a.in[0], loc);
-            for (uint32_t g = 1; g < a.n_in; ++g) acc += VT::widen1(a.in[g], loc);
-            VT::narrow1(a.outs[k], t, finish(acc, AVG, a.scale, a.divisor));
+            for (uint32_t g = 1; g < a.n_in; ++g) acc = combine<MODE>(acc, VT::widen1(a.in[g], loc), a.op);
+            VT::narrow1(a.outs[k], t, finish(acc, MODE == kAvg, a.scale, a.divisor));
         }
     }
 }
@@ -290,7 +326,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
 // issued without predicates (lanes without a B read reduced index 0, one address per wavefront).
 // A vector that would cross a row of the INPUT view, and the last partial chunk, go element by
 // element.  Against the purely scalar form: fp32 rows of 511 0.44 -> 0.68 of peak, bf16 rows of 1022 0.24 -> 0.66.
-template <typename T, bool AVG, bool WIDE, int D>
+template <typename T, int MODE, bool WIDE, int D>
 __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(ScatterArgs a) {
     using VT = Vec<T>;
     using acc_t = typename VT::acc_t;
@@ -309,8 +345,8 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
         const uint64_t r = a.out_offset[k] + decode<WIDE, D>(a.out_dims, t, &col);
         const uint64_t loc = a.in_offset + decode<WIDE, D>(a.in_dims, r, &col);
         acc_t acc = VT::widen1(a.in[0], loc);
-        for (uint32_t g = 1; g < a.n_in; ++g) acc += VT::widen1(a.in[g], loc);
-        VT::narrow1(out, t, finish(acc, AVG, a.scale, a.divisor));
+        for (uint32_t g = 1; g < a.n_in; ++g) acc = combine<MODE>(acc, VT::widen1(a.in[g], loc), a.op);
+        VT::narrow1(out, t, finish(acc, MODE == kAvg, a.scale, a.divisor));
     };
 
     for (uint64_t c = tile0 * kReduceThreads + threadIdx.x; c < nchunks; c += stride) {
@@ -354,24 +390,24 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
                 acc_t x[V];
                 VT::widen(raw_a[j], x);
 #pragma unroll
-                for (int e = 0; e < V; ++e) acc_a[e] += x[e];
+                for (int e = 0; e < V; ++e) acc_a[e] = combine<MODE>(acc_a[e], x[e], a.op);
                 VT::widen(raw_b[j], x);
 #pragma unroll
-                for (int e = 0; e < V; ++e) acc_b[e] += x[e];
+                for (int e = 0; e < V; ++e) acc_b[e] = combine<MODE>(acc_b[e], x[e], a.op);
             }
         }
         for (; g < a.n_in; ++g) {
             acc_t x[V];
             VT::widen(load16_unaligned(static_cast<const char*>(a.in[g]) + va * ES), x);
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc_a[e] += x[e];
+            for (int e = 0; e < V; ++e) acc_a[e] = combine<MODE>(acc_a[e], x[e], a.op);
             VT::widen(load16_unaligned(static_cast<const char*>(a.in[g]) + vb * ES), x);
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc_b[e] += x[e];
+            for (int e = 0; e < V; ++e) acc_b[e] = combine<MODE>(acc_b[e], x[e], a.op);
         }
         if (a_vec) {
 #pragma unroll
-            for (int e = 0; e < V; ++e) acc_a[e] = finish(acc_a[e], AVG, a.scale, a.divisor);
+            for (int e = 0; e < V; ++e) acc_a[e] = finish(acc_a[e], MODE == kAvg, a.scale, a.divisor);
             store16_writethrough(out + ta * ES, VT::narrow(acc_a));
         } else {
             for (int e = 0; e < V; ++e) one_element(ta + e);
@@ -379,7 +415,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
         if (do_b) {
             if (b_vec) {
 #pragma unroll
-                for (int e = 0; e < V; ++e) acc_b[e] = finish(acc_b[e], AVG, a.scale, a.divisor);
+                for (int e = 0; e < V; ++e) acc_b[e] = finish(acc_b[e], MODE == kAvg, a.scale, a.divisor);
                 store16_writethrough(out + tb * ES, VT::narrow(acc_b));
             } else {
                 for (int e = 0; e < V; ++e) one_element(tb + e);
@@ -409,72 +445,89 @@ static int check_dtype_op(int dtype, int op) {
         default:
             return MHIP_ERR_INVALID_DATA_TYPE;
     }
-    if (op != MHIP_OP_SUM && op != MHIP_OP_AVG) return MHIP_ERR_UNSUPPORTED_OP;
+    if (op < MHIP_OP_SUM || op > MHIP_OP_AVG) return MHIP_ERR_UNSUPPORTED_OP;  // nccl.rs:285-292
     return MHIP_SUCCESS;
 }
+
+static int mode_of(int op) { return op == MHIP_OP_SUM ? kSum : op == MHIP_OP_AVG ? kAvg : kGeneric; }
 
 static void avg_factors(uint32_t n, int op, float* scale, float* divisor) {
     *divisor = (float)n;
     *scale = (op == MHIP_OP_AVG && (n & (n - 1)) == 0) ? 1.0f / (float)n : 0.0f;
 }
 
-template <typename T, bool AVG>
+template <typename T, int MODE>
 static void launch_reduce_n(const ReduceArgs& a, hipStream_t s) {
     const dim3 grid(grid_for(a.numel / Vec<T>::V)), block(kReduceThreads);
-    switch (a.n) {
-        case 1: hipLaunchKernelGGL((reduce_kernel<T, 1, AVG>), grid, block, 0, s, a); break;
-        case 2: hipLaunchKernelGGL((reduce_kernel<T, 2, AVG>), grid, block, 0, s, a); break;
-        case 3: hipLaunchKernelGGL((reduce_kernel<T, 3, AVG>), grid, block, 0, s, a); break;
-        case 4: hipLaunchKernelGGL((reduce_kernel<T, 4, AVG>), grid, block, 0, s, a); break;
-        case 8: hipLaunchKernelGGL((reduce_kernel<T, 8, AVG>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((reduce_kernel<T, 0, AVG>), grid, block, 0, s, a); break;
+    if constexpr (MODE == kGeneric) {
+        MHIP_LAUNCH((reduce_kernel<T, 0, MODE>), grid, block, 0, s, a);
+    } else {
+        switch (a.n) {
+            case 1: MHIP_LAUNCH((reduce_kernel<T, 1, MODE>), grid, block, 0, s, a); break;
+            case 2: MHIP_LAUNCH((reduce_kernel<T, 2, MODE>), grid, block, 0, s, a); break;
+            case 3: MHIP_LAUNCH((reduce_kernel<T, 3, MODE>), grid, block, 0, s, a); break;
+            case 4: MHIP_LAUNCH((reduce_kernel<T, 4, MODE>), grid, block, 0, s, a); break;
+            case 8: MHIP_LAUNCH((reduce_kernel<T, 8, MODE>), grid, block, 0, s, a); break;
+            default: MHIP_LAUNCH((reduce_kernel<T, 0, MODE>), grid, block, 0, s, a); break;
+        }
     }
 }
 
-template <typename T>
+// T: the type Sum / Avg run in (integers as the unsigned type of their width); G: the type Prod / Max / Min run in
+// (signed where the dtype is).
+template <typename T, typename G = T>
 static void launch_reduce(const ReduceArgs& a, int op, hipStream_t s) {
-    if (op == MHIP_OP_AVG) launch_reduce_n<T, true>(a, s); else launch_reduce_n<T, false>(a, s);
+    switch (mode_of(op)) {
+        case kSum: launch_reduce_n<T, kSum>(a, s); break;
+        case kAvg: launch_reduce_n<T, kAvg>(a, s); break;
+        default: launch_reduce_n<G, kGeneric>(a, s); break;
+    }
 }
 
-template <typename T, bool VEC, bool AVG>
+template <typename T, bool VEC, int MODE>
 static void launch_scatter_d(const ScatterArgs& a, dim3 grid, bool wide, int d, hipStream_t s) {
     const dim3 block(kReduceThreads);
-    if (wide) { hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, true, -1>), grid, block, 0, s, a); return; }
-    switch (d) {
-        case 2: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, 2>), grid, block, 0, s, a); break;
-        case 4: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, 4>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((reduce_scatter_kernel<T, VEC, AVG, false, -1>), grid, block, 0, s, a); break;
+    if (wide) { MHIP_LAUNCH((reduce_scatter_kernel<T, VEC, MODE, true, -1>), grid, block, 0, s, a); return; }
+    if constexpr (MODE != kGeneric) {
+        switch (d) {
+            case 2: MHIP_LAUNCH((reduce_scatter_kernel<T, VEC, MODE, false, 2>), grid, block, 0, s, a); return;
+            case 4: MHIP_LAUNCH((reduce_scatter_kernel<T, VEC, MODE, false, 4>), grid, block, 0, s, a); return;
+            default: break;
+        }
     }
+    MHIP_LAUNCH((reduce_scatter_kernel<T, VEC, MODE, false, -1>), grid, block, 0, s, a);
 }
 
-template <typename T, bool AVG>
+template <typename T, int MODE>
 static void launch_scatter_ragged(const ScatterArgs& a, dim3 grid, bool wide, int d, hipStream_t s) {
     const dim3 block(kReduceThreads);
-    if (wide) { hipLaunchKernelGGL((reduce_scatter_ragged_kernel<T, AVG, true, -1>), grid, block, 0, s, a); return; }
-    switch (d) {
-        case 2: hipLaunchKernelGGL((reduce_scatter_ragged_kernel<T, AVG, false, 2>), grid, block, 0, s, a); break;
-        case 4: hipLaunchKernelGGL((reduce_scatter_ragged_kernel<T, AVG, false, 4>), grid, block, 0, s, a); break;
-        default: hipLaunchKernelGGL((reduce_scatter_ragged_kernel<T, AVG, false, -1>), grid, block, 0, s, a); break;
+    if (wide) { MHIP_LAUNCH((reduce_scatter_ragged_kernel<T, MODE, true, -1>), grid, block, 0, s, a); return; }
+    if constexpr (MODE != kGeneric) {
+        switch (d) {
+            case 2: MHIP_LAUNCH((reduce_scatter_ragged_kernel<T, MODE, false, 2>), grid, block, 0, s, a); return;
+            case 4: MHIP_LAUNCH((reduce_scatter_ragged_kernel<T, MODE, false, 4>), grid, block, 0, s, a); return;
+            default: break;
+        }
     }
+    MHIP_LAUNCH((reduce_scatter_ragged_kernel<T, MODE, false, -1>), grid, block, 0, s, a);
 }
 
-template <typename T>
-static void launch_scatter(const ScatterArgs& a, dim3 grid, bool vec, bool ragged, bool avg, bool wide, int d, hipStream_t s) {
+template <typename T, int MODE>
+static void launch_scatter_mode(const ScatterArgs& a, dim3 grid, bool vec, bool ragged, bool wide, int d, hipStream_t s) {
+    if (ragged) launch_scatter_ragged<T, MODE>(a, grid, wide, d, s);
+    else if (vec) launch_scatter_d<T, true, MODE>(a, grid, wide, d, s);
+    else launch_scatter_d<T, false, MODE>(a, grid, wide, d, s);
+}
+
+template <typename T, typename G = T>
+static void launch_scatter(const ScatterArgs& a, dim3 grid, bool vec, bool ragged, int op, bool wide, int d, hipStream_t s) {
     constexpr bool kFloat = std::is_floating_point<typename Vec<T>::acc_t>::value;
-    if (ragged) {
-        if constexpr (kFloat) {
-            if (avg) { launch_scatter_ragged<T, true>(a, grid, wide, d, s); return; }
-        }
-        launch_scatter_ragged<T, false>(a, grid, wide, d, s);
-        return;
-    }
+    const int mode = mode_of(op);
+    if (mode == kGeneric) { launch_scatter_mode<G, kGeneric>(a, grid, vec, ragged, wide, d, s); return; }
     if constexpr (kFloat) {
-        if (avg) {
-            if (vec) launch_scatter_d<T, true, true>(a, grid, wide, d, s); else launch_scatter_d<T, false, true>(a, grid, wide, d, s);
-            return;
-        }
+        if (mode == kAvg) { launch_scatter_mode<T, kAvg>(a, grid, vec, ragged, wide, d, s); return; }
     }
-    if (vec) launch_scatter_d<T, true, false>(a, grid, wide, d, s); else launch_scatter_d<T, false, false>(a, grid, wide, d, s);
+    launch_scatter_mode<T, kSum>(a, grid, vec, ragged, wide, d, s);
 }
 
 }  // namespace mhip
@@ -515,6 +568,7 @@ int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, in
     a.n = n;
     avg_factors(n, op, &a.scale, &a.divisor);
     a.xcd_contiguous = inputs_alias(in, n);
+    a.op = (uint32_t)op;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     switch (dtype) {
@@ -522,9 +576,10 @@ int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, in
         case MHIP_DTYPE_BF16: launch_reduce<bf16_tag>(a, op, hs); break;
         case MHIP_DTYPE_F16: launch_reduce<_Float16>(a, op, hs); break;
         case MHIP_DTYPE_F64: launch_reduce<double>(a, op, hs); break;
-        case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_reduce<uint8_t>(a, op, hs); break;
-        case MHIP_DTYPE_I32: launch_reduce<uint32_t>(a, op, hs); break;
-        case MHIP_DTYPE_I64: launch_reduce<uint64_t>(a, op, hs); break;
+        case MHIP_DTYPE_U8: launch_reduce<uint8_t>(a, op, hs); break;
+        case MHIP_DTYPE_I8: launch_reduce<uint8_t, int8_t>(a, op, hs); break;
+        case MHIP_DTYPE_I32: launch_reduce<uint32_t, int32_t>(a, op, hs); break;
+        case MHIP_DTYPE_I64: launch_reduce<uint64_t, int64_t>(a, op, hs); break;
         default: return MHIP_ERR_INVALID_DATA_TYPE;
     }
     return launch_status();
@@ -627,15 +682,16 @@ int mhip_reduce_scatter(void* const* outs, const mhip_slice_t* out_views, uint32
         uint64_t tiles = grid_for(ragged ? (a.total + V - 1) / V : a.total);
         while (tiles > 1 && tiles * nbatch > max_workgroups(kReduceThreads)) tiles = (tiles + 1) / 2;  // grid-stride takes over
         dim3 grid((uint32_t)(tiles * nbatch));
-        const bool avg = op == MHIP_OP_AVG;
+        a.op = (uint32_t)op;
         switch (dtype) {
-            case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_BF16: launch_scatter<bf16_tag>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_F16: launch_scatter<_Float16>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_F64: launch_scatter<double>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_U8: case MHIP_DTYPE_I8: launch_scatter<uint8_t>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_I32: launch_scatter<uint32_t>(a, grid, vec, ragged, avg, wide, d, hs); break;
-            case MHIP_DTYPE_I64: launch_scatter<uint64_t>(a, grid, vec, ragged, avg, wide, d, hs); break;
+            case MHIP_DTYPE_F32: launch_scatter<float>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_BF16: launch_scatter<bf16_tag>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_F16: launch_scatter<_Float16>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_F64: launch_scatter<double>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_U8: launch_scatter<uint8_t>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_I8: launch_scatter<uint8_t, int8_t>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_I32: launch_scatter<uint32_t, int32_t>(a, grid, vec, ragged, op, wide, d, hs); break;
+            case MHIP_DTYPE_I64: launch_scatter<uint64_t, int64_t>(a, grid, vec, ragged, op, wide, d, hs); break;
             default: return MHIP_ERR_INVALID_DATA_TYPE;
         }
         if (int rc = launch_status()) return rc;

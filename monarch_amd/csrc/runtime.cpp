@@ -54,9 +54,12 @@ const char* mhip_error_string(int status) {
         case MHIP_ERR_INPUT_SIZE_MISMATCH: return "input tensor must be the same size as output size times world size";
         case MHIP_ERR_UNDEFINED_TENSOR: return "undefined tensor (null pointer) used for operation";
         case MHIP_ERR_INVALID_ARGUMENT: return "an argument has an invalid value";
-        case MHIP_ERR_UNSUPPORTED_OP: return "reduction op not supported for this dtype (Sum and Avg only; Avg on floating types)";
+        case MHIP_ERR_UNSUPPORTED_OP: return "reduction op not supported for this dtype (Sum, Prod, Max, Min; Avg on floating types)";
         case MHIP_ERR_TOO_MANY_INPUTS: return "too many inputs for one reduce (at most 64)";
         case MHIP_ERR_UNSUPPORTED_BLOCK: return "unsupported fp8 scale block (must be 1024)";
+        case MHIP_ERR_BUFFER_TOO_SMALL: return "remote buffer is smaller than the transfer";
+        case MHIP_ERR_MESH_DIM_LENGTH_MISMATCH: return "dimension of destination device_mesh has a different length than the source tensor";
+        case MHIP_ERR_MESH_DIM_MISSING: return "destination mesh does not have a dimension of the source tensor";
         default: break;
     }
     if (status > 0 && status < 10000) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -118,7 +121,7 @@ int mhip_memset(void* dst, int value, size_t bytes, mhip_stream_t stream) {
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     return launch_in_pieces(wgs, kFillThreads, 1, [&](uint64_t wg0, uint32_t count) {
-        hipLaunchKernelGGL(fill_kernel, dim3(count), dim3(kFillThreads), 0, hs, static_cast<unsigned char*>(dst), word,
+        MHIP_LAUNCH(fill_kernel, dim3(count), dim3(kFillThreads), 0, hs, static_cast<unsigned char*>(dst), word,
                            (uint64_t)bytes, head, nvec, wg0);
     });
 }

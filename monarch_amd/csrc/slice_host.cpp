@@ -1,7 +1,9 @@
-// Host-side Slice algebra and DeviceMesh membership behind the C ABI.
-// Mirrors ndslice::Slice (ndslice/src/slice.rs) and DeviceMesh
-// (monarch_tensor_worker/src/device_mesh.rs); pure integer work, no GPU calls.
+// Host-side Slice algebra, DeviceMesh membership and SendTensor routing behind the C ABI.
+// Mirrors ndslice::Slice (ndslice/src/slice.rs), DeviceMesh (monarch_tensor_worker/src/device_mesh.rs),
+// WorkerActor::send_tensor's rank pairing (monarch_tensor_worker/src/lib.rs:722-731) and Tensor.to_mesh's
+// checks (python/monarch/common/tensor.py:417-438); pure integer work, no GPU calls.
 #include <algorithm>
+#include <cstring>
 #include <numeric>
 #include <utility>
 #include <vector>
@@ -91,6 +93,8 @@ static int coordinates(const mhip_slice_t& s, uint64_t value, uint64_t* out) {
         const uint32_t d = order[r];
         uint64_t c = 0;
         if (s.sizes[d] > 1) {
+            // Slice::new never yields a zero stride on a dimension longer than 1; a caller-built struct can
+            if (s.strides[d] == 0) return MHIP_ERR_INVALID_ARGUMENT;
             c = pos / s.strides[d];
             pos %= s.strides[d];
         }
@@ -174,7 +178,7 @@ int mhip_slice_iter(const mhip_slice_t* s, uint64_t start, uint64_t count, uint6
         uint64_t coord[MHIP_MAX_DIMS];
         unravel(s->sizes, s->ndim, start, coord);
         uint64_t loc = s->offset + dot(coord, s->strides, s->ndim);
-        const uint64_t stop = std::min(len, start + count);
+        const uint64_t stop = start + std::min(count, len - start);  // start + count may not fit 64 bits
         for (uint64_t i = start; i < stop; ++i) {
             locs[n++] = loc;
             for (uint32_t k = s->ndim; k-- > 0;) {
@@ -226,7 +230,7 @@ int mhip_slice_subview(const mhip_slice_t* s, const uint64_t* starts, uint32_t n
     if (bad(s) || !out_offset || (nstarts && !starts) || (nlens && !lens)) return MHIP_ERR_INVALID_ARGUMENT;
     if (nstarts != s->ndim || nlens != s->ndim) return MHIP_ERR_INVALID_DIMS;
     for (uint32_t d = 0; d < s->ndim; ++d)
-        if (starts[d] + lens[d] > s->sizes[d]) return MHIP_ERR_INDEX_OUT_OF_RANGE;
+        if (starts[d] > s->sizes[d] || lens[d] > s->sizes[d] - starts[d]) return MHIP_ERR_INDEX_OUT_OF_RANGE;  // no wrap
     *out_offset = s->offset + dot(starts, s->strides, s->ndim);
     return MHIP_SUCCESS;
 }
@@ -310,6 +314,63 @@ int mhip_mesh_ranks_for_dims(const mhip_slice_t* ranks, uint64_t rank, const uin
     uint64_t n = 0;
     mhip_slice_iter(&group, 0, total, out, &n);
     *count = n;
+    return MHIP_SUCCESS;
+}
+
+int mhip_send_tensor_route(const mhip_slice_t* from_ranks, const mhip_slice_t* to_ranks, uint64_t rank,
+                           uint64_t* from_rank, uint64_t* to_rank) {
+    if (bad(from_ranks) || bad(to_ranks) || !from_rank || !to_rank) return MHIP_ERR_INVALID_ARGUMENT;
+    // lib.rs:722-731: the i-th sender pairs with the i-th receiver; a rank outside a slice, or an index
+    // past the other slice's length, leaves that side empty
+    auto pair = [rank](const mhip_slice_t* mine, const mhip_slice_t* other) -> uint64_t {
+        uint64_t index = 0, peer = 0;
+        if (mhip_slice_index(mine, rank, &index) != MHIP_SUCCESS) return MHIP_NO_RANK;
+        if (mhip_slice_get(other, index, &peer) != MHIP_SUCCESS) return MHIP_NO_RANK;
+        return peer;
+    };
+    *to_rank = pair(from_ranks, to_ranks);
+    *from_rank = pair(to_ranks, from_ranks);
+    return MHIP_SUCCESS;
+}
+
+int mhip_to_mesh_from_ranks(const char* const* slicing_names, const mhip_slice_t* slicing,
+                            const char* const* mesh_names, const uint64_t* mesh_sizes, uint32_t mesh_ndim,
+                            uint64_t* out_sizes, uint64_t* out_strides, uint32_t* out_ndim,
+                            uint32_t* broadcast_dims, uint32_t* n_broadcast, uint32_t* culprit) {
+    if (bad(slicing) || !out_ndim || !n_broadcast || mesh_ndim > MHIP_MAX_DIMS) return MHIP_ERR_INVALID_ARGUMENT;
+    if ((slicing->ndim && (!slicing_names || !out_sizes || !out_strides)) ||
+        (mesh_ndim && (!mesh_names || !mesh_sizes || !broadcast_dims)))
+        return MHIP_ERR_INVALID_ARGUMENT;
+    uint32_t kept = 0, bcast = 0;
+    // tensor.py:417-433: walk the destination mesh's dimensions in its order
+    for (uint32_t m = 0; m < mesh_ndim; ++m) {
+        uint32_t index = slicing->ndim;
+        for (uint32_t k = 0; k < slicing->ndim; ++k)
+            if (std::strcmp(slicing_names[k], mesh_names[m]) == 0) { index = k; break; }  // list.index: first match
+        if (index == slicing->ndim) {
+            broadcast_dims[bcast++] = m;
+            continue;
+        }
+        if (slicing->sizes[index] != mesh_sizes[m]) {
+            if (culprit) *culprit = m;
+            return MHIP_ERR_MESH_DIM_LENGTH_MISMATCH;
+        }
+        if (kept == slicing->ndim) return MHIP_ERR_INVALID_ARGUMENT;  // a name repeated in the destination mesh
+        out_sizes[kept] = mesh_sizes[m];
+        out_strides[kept++] = slicing->strides[index];
+    }
+    if (kept != slicing->ndim) {  // tensor.py:435-437
+        if (culprit) {
+            for (uint32_t k = 0; k < slicing->ndim; ++k) {
+                bool found = false;
+                for (uint32_t m = 0; m < mesh_ndim; ++m) found = found || std::strcmp(slicing_names[k], mesh_names[m]) == 0;
+                if (!found) { *culprit = k; break; }
+            }
+        }
+        return MHIP_ERR_MESH_DIM_MISSING;
+    }
+    *out_ndim = kept;
+    *n_broadcast = bcast;
     return MHIP_SUCCESS;
 }
 

@@ -479,20 +479,20 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
             a.wg0 = wg0;
             const dim3 grid(count);
             switch (unit) {
-                case 1: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-                case 2: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                case 2: MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
                 case 4:
-                    if (big) hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a);
-                    else hipLaunchKernelGGL((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a);
+                    if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a);
+                    else MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a);
                     break;
-                default: hipLaunchKernelGGL((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+                default: MHIP_LAUNCH((slice_transpose_vec_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
             }
         });
         return true;
     }
     if (unit != 16) return false;
     const uint64_t cap = max_workgroups(kThreads);  // grid-stride kernel
-    hipLaunchKernelGGL((slice_transpose_kernel<uint4, 32, PACK>), dim3((uint32_t)(a.ntiles < cap ? a.ntiles : cap)), dim3(kThreads), 0,
+    MHIP_LAUNCH((slice_transpose_kernel<uint4, 32, PACK>), dim3((uint32_t)(a.ntiles < cap ? a.ntiles : cap)), dim3(kThreads), 0,
                        stream, a);
     *rc = launch_status();
     return true;

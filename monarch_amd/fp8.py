@@ -21,6 +21,23 @@ BLOCK = 1024
 FP8_MAX = 448.0
 
 
+def _nblocks(n: int) -> int:
+    return (n + BLOCK - 1) // BLOCK
+
+
+def _check_payload(q: torch.Tensor, scales: torch.Tensor, n: int, device: torch.device) -> None:
+    """Caller-supplied code and scale buffers: on ``device``, contiguous, one byte per element for ``n`` elements
+    and one fp32 scale per 1024-element block.  A short buffer would be an out-of-bounds device write."""
+    for t in (q, scales):
+        _torch.require_contiguous(t)
+        if t.device != device:
+            raise ValueError(f"buffer is on {t.device}, the data on {device}")
+    if q.element_size() != 1 or q.numel() != n:
+        raise ValueError(f"q must hold {n} one-byte codes, got {q.numel()} elements of {q.element_size()} bytes")
+    if scales.dtype != torch.float32 or scales.numel() != _nblocks(n):
+        raise ValueError(f"scales must hold {_nblocks(n)} fp32 values, got {scales.numel()} of {scales.dtype}")
+
+
 class FlatBucket:
     """Offsets table and device pointer table for a list of ragged tensors."""
 
@@ -41,33 +58,62 @@ class FlatBucket:
         self.total = self.offsets[-1]
         # device-resident tables, uploaded once and reused by every pack / unpack
         self.d_offsets = torch.tensor(self.offsets, dtype=torch.int64, device=self.device)
+        self._tables = {}
         self.d_ptrs = self.pointer_table(tensors)
+
+    # Launches read a pointer table asynchronously, possibly on a stream torch's allocator does not know about, so a
+    # table must not go back to the allocator while a launch may still be queued.  Tables are kept per set of
+    # tensors (uploading is a host-synchronous copy, so a cached table is complete before any launch uses it);
+    # the cache holds the tensors too, so a cached address cannot be handed to another tensor meanwhile.
+    _MAX_TABLES = 8
 
     def pointer_table(self, tensors: Sequence[torch.Tensor]) -> torch.Tensor:
         if [t.numel() for t in tensors] != self.sizes:
             raise ValueError("tensor sizes do not match the bucket")
-        return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, device=self.device)
+        key = tuple(t.data_ptr() for t in tensors)
+        hit = self._tables.get(key)
+        if hit is None:
+            if len(self._tables) >= self._MAX_TABLES:   # retire the oldest once everything queued so far has run
+                torch.cuda.synchronize(self.device)
+                self._tables.pop(next(iter(self._tables)))
+            hit = (torch.tensor(key, dtype=torch.int64, device=self.device), list(tensors))
+            self._tables[key] = hit
+        return hit[0]
 
     def pack(self, flat: torch.Tensor = None, d_ptrs: torch.Tensor = None, stream=None) -> torch.Tensor:
         """flat[offsets[t] + j] = tensors[t][j]"""
         if flat is None:
             flat = torch.empty(self.total, dtype=self.dtype, device=self.device)
+        else:
+            self._check_flat(flat, self.dtype)
         ptrs = self.d_ptrs if d_ptrs is None else d_ptrs
+        if ptrs.dtype != torch.int64 or ptrs.numel() != len(self.sizes) or ptrs.device != self.device:
+            raise ValueError("the pointer table must hold one int64 device pointer per tensor of the bucket")
         check(lib().mhip_flat_pack(flat.data_ptr(), ptrs.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
-                                   self.total, flat.element_size(), _torch.stream_handle(stream)))
+                                   self.total, self.tensors[0].element_size(), _torch.stream_handle(stream)))
         return flat
+
+    def _check_flat(self, flat: torch.Tensor, dtype: torch.dtype) -> None:
+        _torch.require_contiguous(flat)
+        if flat.device != self.device:
+            raise ValueError(f"flat buffer is on {flat.device}, the bucket on {self.device}")
+        if flat.dtype != dtype or flat.numel() != self.total:
+            raise ValueError(f"flat buffer must hold {self.total} elements of {dtype}, got {flat.numel()} of {flat.dtype}")
 
     def unpack(self, flat: torch.Tensor, outs: Sequence[torch.Tensor], stream=None) -> None:
         """outs[t][j] = flat[offsets[t] + j]; ``flat`` may have any dtype of the outs' element size."""
+        _torch.require_contiguous(flat)
+        if flat.numel() != self.total or flat.device != self.device:
+            raise ValueError(f"flat buffer must hold {self.total} elements on {self.device}")
         for t in outs:
             _torch.require_contiguous(t)
             if t.element_size() != flat.element_size():
                 raise ValueError("element size mismatch")
+            if t.device != self.device:
+                raise ValueError(f"output is on {t.device}, the bucket on {self.device}")
         ptrs = self.pointer_table(outs)
         check(lib().mhip_flat_unpack(ptrs.data_ptr(), flat.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
                                      self.total, flat.element_size(), _torch.stream_handle(stream)))
-        # the launch reads the table asynchronously: keep it (and the outputs) alive
-        self._last_unpack = (ptrs, list(outs))
 
 
 def quantize_bucket(bucket: FlatBucket, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None):
@@ -78,7 +124,8 @@ def quantize_bucket(bucket: FlatBucket, q: torch.Tensor = None, scales: torch.Te
     if q is None:
         q = torch.empty(n, dtype=torch.uint8, device=bucket.device)
     if scales is None:
-        scales = torch.empty((n + BLOCK - 1) // BLOCK, dtype=torch.float32, device=bucket.device)
+        scales = torch.empty(_nblocks(n), dtype=torch.float32, device=bucket.device)
+    _check_payload(q, scales, n, bucket.device)
     check(lib().mhip_fp8_quantize_bucket(q.data_ptr(), scales.data_ptr(), bucket.d_ptrs.data_ptr(),
                                          bucket.d_offsets.data_ptr(), len(bucket.sizes), n, BLOCK,
                                          _torch.stream_handle(stream)))
@@ -89,10 +136,7 @@ def dequant_accumulate_bucket(bucket: FlatBucket, q: torch.Tensor, scales: torch
     """``tensor_t[j] += float(q[off_t + j]) * scale`` on the bucket's own fp32 tensors."""
     if bucket.dtype != torch.float32:
         raise ValueError("dequant_accumulate_bucket expects a bucket of fp32 accumulators")
-    for t in (q, scales):
-        _torch.require_contiguous(t)
-    if q.numel() != bucket.total or scales.numel() != (bucket.total + BLOCK - 1) // BLOCK:
-        raise ValueError("size mismatch between the bucket, q and scales")
+    _check_payload(q, scales, bucket.total, bucket.device)
     check(lib().mhip_fp8_dequant_accumulate_bucket(bucket.d_ptrs.data_ptr(), q.data_ptr(), scales.data_ptr(),
                                                    bucket.d_offsets.data_ptr(), len(bucket.sizes), bucket.total, BLOCK,
                                                    _torch.stream_handle(stream)))
@@ -104,11 +148,11 @@ def quantize(flat_bf16: torch.Tensor, q: torch.Tensor = None, scales: torch.Tens
     if flat_bf16.dtype != torch.bfloat16:
         raise ValueError("quantize expects a bf16 buffer")
     n = flat_bf16.numel()
-    nb = (n + BLOCK - 1) // BLOCK
     if q is None:
         q = torch.empty(n, dtype=torch.uint8, device=flat_bf16.device)
     if scales is None:
-        scales = torch.empty(nb, dtype=torch.float32, device=flat_bf16.device)
+        scales = torch.empty(_nblocks(n), dtype=torch.float32, device=flat_bf16.device)
+    _check_payload(q, scales, n, flat_bf16.device)
     check(lib().mhip_fp8_quantize(q.data_ptr(), scales.data_ptr(), flat_bf16.data_ptr(), n, BLOCK,
                                   _torch.stream_handle(stream)))
     return q, scales
@@ -116,12 +160,10 @@ def quantize(flat_bf16: torch.Tensor, q: torch.Tensor = None, scales: torch.Tens
 
 def dequant_accumulate(acc: torch.Tensor, q: torch.Tensor, scales: torch.Tensor, stream=None) -> None:
     """acc[i] += float(q[i]) * scales[i // 1024] (fp32, product rounded before the add)."""
-    for t in (acc, q, scales):
-        _torch.require_contiguous(t)
-    if acc.dtype != torch.float32 or scales.dtype != torch.float32 or q.element_size() != 1:
-        raise ValueError("acc and scales must be fp32 and q one byte per element")
-    if acc.numel() != q.numel() or scales.numel() != (q.numel() + BLOCK - 1) // BLOCK:
-        raise ValueError("size mismatch between acc, q and scales")
+    _torch.require_contiguous(acc)
+    if acc.dtype != torch.float32:
+        raise ValueError("acc must be fp32")
+    _check_payload(q, scales, acc.numel(), acc.device)
     check(lib().mhip_fp8_dequant_accumulate(acc.data_ptr(), q.data_ptr(), scales.data_ptr(), q.numel(), BLOCK,
                                             _torch.stream_handle(stream)))
 
@@ -138,12 +180,7 @@ def dequant_accumulate_many(acc: torch.Tensor, qs: Sequence[torch.Tensor], scale
         raise ValueError("acc must be fp32")
     n = acc.numel()
     for q, s in zip(qs, scales):
-        _torch.require_contiguous(q)
-        _torch.require_contiguous(s)
-        if q.element_size() != 1 or s.dtype != torch.float32:
-            raise ValueError("codes must be one byte per element and scales fp32")
-        if q.numel() != n or s.numel() != (n + BLOCK - 1) // BLOCK:
-            raise ValueError("size mismatch between acc, q and scales")
+        _check_payload(q, s, n, acc.device)
     check(lib().mhip_fp8_dequant_accumulate_many(acc.data_ptr(), ptr_array([q.data_ptr() for q in qs]),
                                                  ptr_array([s.data_ptr() for s in scales]), len(qs), n, BLOCK,
                                                  1 if overwrite else 0, _torch.stream_handle(stream)))
@@ -157,12 +194,7 @@ def dequant_accumulate_bucket_many(bucket: FlatBucket, qs: Sequence[torch.Tensor
     if len(qs) == 0 or len(qs) != len(scales):
         raise ValueError("one scales tensor per code tensor, at least one peer")
     for q, s in zip(qs, scales):
-        _torch.require_contiguous(q)
-        _torch.require_contiguous(s)
-        if q.element_size() != 1 or s.dtype != torch.float32:
-            raise ValueError("codes must be one byte per element and scales fp32")
-        if q.numel() != bucket.total or s.numel() != (bucket.total + BLOCK - 1) // BLOCK:
-            raise ValueError("size mismatch between the bucket, q and scales")
+        _check_payload(q, s, bucket.total, bucket.device)
     check(lib().mhip_fp8_dequant_accumulate_bucket_many(
         bucket.d_ptrs.data_ptr(), ptr_array([q.data_ptr() for q in qs]), ptr_array([s.data_ptr() for s in scales]),
         len(qs), bucket.d_offsets.data_ptr(), len(bucket.sizes), bucket.total, BLOCK, _torch.stream_handle(stream)))

@@ -133,11 +133,6 @@ def check_reduce_args(mesh_names: Sequence[str], mesh_sizes: Dict[str, int], sha
     return dims, tuple(result)
 
 
-def _flat_copy(dst_ptr: int, src_ptr: int, nbytes: int, stream) -> None:
-    flat = Slice.new_row_major([nbytes])
-    check(lib().mhip_slice_pack(dst_ptr, src_ptr, C.byref(flat.c), 1, _torch.stream_handle(stream)))
-
-
 def all_reduce(out: torch.Tensor, group: Sequence[torch.Tensor], op: ReduceOp, stream=None) -> None:
     """Local combine of ``Communicator::all_reduce`` (torch-sys-cuda/src/nccl.rs:464-489):
     ``out = op(group)``; ``out`` may be one of the group's tensors (the in-place form)."""
@@ -205,21 +200,29 @@ def stream_reduce(group: Sequence[Optional[torch.Tensor]], rank: int, factory: F
     group = [factory.zeros() if t is None else t for t in group]
     local = group[rank]
     if reduction.is_stack:
+        for t in group:
+            _torch.require_contiguous(t)
+            if t.dtype != local.dtype or t.numel() != local.numel():
+                raise MhipError(_lib.ERR_TYPE_MISMATCH, "all group members must share dtype and size")
+        ptrs = ptr_array([t.data_ptr() for t in group])
         if scatter:  # all_to_all_single, stream.rs:1381-1399
             output = local if in_place else (out if out is not None else torch.empty_like(local))
-            src = [t.clone() for t in group] if in_place else group  # peers read the pre-exchange values
-            c = local.numel() // n
-            eb = local.element_size()
-            for g in range(n):
-                _flat_copy(output.data_ptr() + g * c * eb, src[g].data_ptr() + rank * c * eb, c * eb, stream)
+            _torch.require_contiguous(output)
+            if output.numel() != local.numel() or output.dtype != local.dtype:
+                raise MhipError(_lib.ERR_OUTPUT_SIZE_MISMATCH, "output tensor must match the input tensor")
+            check(lib().mhip_stack_scatter(output.data_ptr(), ptrs, n, rank, local.numel(), local.element_size(),
+                                           _torch.stream_handle(stream)))
             return output
         if in_place:
             raise ValueError("in-place, non-scatter not supported for stack reduce")
         output = out if out is not None else torch.empty((n, *factory.size), dtype=factory.dtype, device=local.device)
-        eb = local.element_size() * local.numel()
-        for g in range(n):  # all_gather_into_tensor, stream.rs:1408-1417
-            _torch.require_contiguous(group[g])
-            _flat_copy(output.data_ptr() + g * eb, group[g].data_ptr(), eb, stream)
+        _torch.require_contiguous(output)
+        if output.numel() != n * local.numel() or output.dtype != local.dtype:
+            raise MhipError(_lib.ERR_OUTPUT_SIZE_MISMATCH,
+                            "output tensor size must be equal to world size times input tensor size")
+        # all_gather_into_tensor, stream.rs:1408-1417
+        check(lib().mhip_stack(output.data_ptr(), ptrs, n, local.numel(), local.element_size(),
+                               _torch.stream_handle(stream)))
         return output
     op = reduction.op
     if scatter:

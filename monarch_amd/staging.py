@@ -15,7 +15,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from . import _torch
-from ._lib import check, lib, ptr_array
+from ._lib import RdmaBufferC, check, lib, ptr_array
 from .ndslice import Slice, slice_array
 
 
@@ -38,6 +38,15 @@ def _check_view_fits(base: torch.Tensor, s: Slice) -> None:
         raise ValueError(f"slice reaches element {hi} but the storage holds {storage_elems}")
 
 
+def _check_staging(buf: torch.Tensor, nbytes: int, device: torch.device) -> None:
+    """A caller-supplied staging buffer: on the device of the tensor, contiguous, exactly ``nbytes`` long."""
+    _torch.require_device(buf)
+    if buf.device != device:
+        raise ValueError(f"staging buffer is on {buf.device}, the tensor on {device}")
+    if not buf.is_contiguous() or buf.numel() * buf.element_size() != nbytes:
+        raise ValueError("staging buffer must be contiguous and hold exactly len(slice) elements")
+
+
 def pack(base: torch.Tensor, s: Slice, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
     """``out[i] = storage(base)[s.get(i)]``; returns a 1-D tensor of ``base.dtype``."""
     _torch.require_device(base)
@@ -45,8 +54,8 @@ def pack(base: torch.Tensor, s: Slice, out: Optional[torch.Tensor] = None, strea
     n = len(s)
     if out is None:
         out = torch.empty(n, dtype=base.dtype, device=base.device)
-    elif out.numel() * out.element_size() != n * base.element_size() or not out.is_contiguous():
-        raise ValueError("staging buffer must be contiguous and hold exactly len(slice) elements")
+    else:
+        _check_staging(out, n * base.element_size(), base.device)
     check(lib().mhip_slice_pack(out.data_ptr(), _torch.storage_ptr(base), C.byref(s.c), base.element_size(),
                                 _torch.stream_handle(stream)))
     return out
@@ -55,10 +64,8 @@ def pack(base: torch.Tensor, s: Slice, out: Optional[torch.Tensor] = None, strea
 def unpack(base: torch.Tensor, s: Slice, src: torch.Tensor, stream=None) -> None:
     """``storage(base)[s.get(i)] = src[i]``; elements outside the view keep their values."""
     _torch.require_device(base)
-    _torch.require_contiguous(src)
     _check_view_fits(base, s)
-    if src.numel() * src.element_size() != len(s) * base.element_size():
-        raise ValueError("staging buffer must hold exactly len(slice) elements")
+    _check_staging(src, len(s) * base.element_size(), base.device)
     check(lib().mhip_slice_unpack(_torch.storage_ptr(base), src.data_ptr(), C.byref(s.c), base.element_size(),
                                   _torch.stream_handle(stream)))
 
@@ -71,6 +78,10 @@ def pack_many(base: torch.Tensor, views: Sequence[Slice], outs: Optional[List[to
         _check_view_fits(base, s)
     if outs is None:
         outs = [torch.empty(len(s), dtype=base.dtype, device=base.device) for s in views]
+    elif len(outs) != len(views):
+        raise ValueError(f"{len(views)} views need {len(views)} staging buffers, got {len(outs)}")
+    for s, o in zip(views, outs):
+        _check_staging(o, len(s) * base.element_size(), base.device)
     arr = slice_array(views)
     check(lib().mhip_slice_pack_many(ptr_array([o.data_ptr() for o in outs]), _torch.storage_ptr(base), arr,
                                      len(views), base.element_size(), _torch.stream_handle(stream)))
@@ -79,32 +90,28 @@ def pack_many(base: torch.Tensor, views: Sequence[Slice], outs: Optional[List[to
 
 def unpack_many(base: torch.Tensor, views: Sequence[Slice], srcs: Sequence[torch.Tensor], stream=None) -> None:
     _torch.require_device(base)
+    if len(srcs) != len(views):
+        raise ValueError(f"{len(views)} views need {len(views)} staging buffers, got {len(srcs)}")
     for s, src in zip(views, srcs):
         _check_view_fits(base, s)
-        _torch.require_contiguous(src)
-        if src.numel() * src.element_size() != len(s) * base.element_size():
-            raise ValueError("staging buffer must hold exactly len(slice) elements")
+        _check_staging(src, len(s) * base.element_size(), base.device)
     arr = slice_array(views)
     check(lib().mhip_slice_unpack_many(_torch.storage_ptr(base), ptr_array([t.data_ptr() for t in srcs]), arr,
                                        len(views), base.element_size(), _torch.stream_handle(stream)))
 
 
 # One RDMA work request carries its length in a 32-bit field of the scatter/gather entry
-# (monarch_rdma/src/rdma_components.rs:1041,1063 cast the size with ``as u32``), so a transfer of
-# 4 GiB or more has to be cut into several requests.  Segments are multiples of 16 bytes.
+# (monarch_rdma/src/rdma_components.rs:1041,1063 cast the size with ``as u32``), so the library cuts a
+# transfer of 4 GiB or more into several requests (``mhip_buffer_transfer``).  Segments are multiples of 16 bytes.
 MAX_SEGMENT_BYTES = (1 << 32) - 16
 
 
-def transfer_segments(nbytes: int, max_bytes: Optional[int] = None):
-    """``(offset, length)`` pairs that cover ``nbytes`` with every length <= ``max_bytes``."""
-    limit = MAX_SEGMENT_BYTES if max_bytes is None else max_bytes
-    if limit <= 0:
-        raise ValueError("segments must hold at least one byte")
-    done = 0
-    while done < nbytes:
-        step = min(limit, nbytes - done)
-        yield done, step
-        done += step
+def transfer(dst_ptr: int, src_ptr: int, nbytes: int, max_segment_bytes: int = 0, stream=None) -> int:
+    """Moves ``nbytes`` bytes as one device copy per work request; returns the number of requests posted."""
+    posted = C.c_uint32()
+    check(lib().mhip_buffer_transfer(dst_ptr, src_ptr, nbytes, max_segment_bytes, _torch.stream_handle(stream),
+                                     C.byref(posted)))
+    return posted.value
 
 
 class RDMABuffer:
@@ -112,7 +119,9 @@ class RDMABuffer:
 
     On one GPU the transport is a flat device copy; the names keep the reference's
     direction: ``buf.read_into(dst)`` copies the buffer's bytes into ``dst`` and
-    ``buf.write_from(src)`` copies ``src`` into the buffer.
+    ``buf.write_from(src)`` copies ``src`` into the buffer.  As in the reference's binding
+    (monarch_rdma/extension/lib.rs:135-190) the tensor becomes a local ``RdmaBuffer`` and the library's
+    ``write_from`` / ``read_into`` run on it with this buffer as the remote side.
     """
 
     def __init__(self, data: torch.Tensor) -> None:
@@ -126,28 +135,27 @@ class RDMABuffer:
     def data(self) -> torch.Tensor:
         return self._data
 
-    def _copy(self, dst_ptr: int, src_ptr: int, nbytes: int, stream) -> None:
-        for offset, length in transfer_segments(nbytes):  # one "work request" per segment
-            flat = Slice.new_row_major([length])
-            check(lib().mhip_slice_pack(dst_ptr + offset, src_ptr + offset, C.byref(flat.c), 1,
-                                        _torch.stream_handle(stream)))
+    def _remote(self, offset: int) -> RdmaBufferC:
+        return RdmaBufferC(self.addr + offset, self.size - offset)
 
     def read_into(self, dst: torch.Tensor, offset: int = 0, stream=None) -> int:
         _assert_tensor_is_1d_contiguous_uint8(dst)
         _torch.require_device(dst)
         size = dst.numel()
-        if offset + size > self.size:
+        if offset < 0 or offset + size > self.size:
             raise ValueError(f"offset + size ({offset + size}) must be <= buffer size ({self.size})")
-        self._copy(dst.data_ptr(), self.addr + offset, size, stream)
+        local = RdmaBufferC(dst.data_ptr(), size)
+        check(lib().mhip_buffer_write_from(C.byref(local), C.byref(self._remote(offset)), _torch.stream_handle(stream)))
         return size
 
     def write_from(self, src: torch.Tensor, offset: int = 0, stream=None) -> None:
         _assert_tensor_is_1d_contiguous_uint8(src)
         _torch.require_device(src)
         size = src.numel()
-        if size + offset > self.size:
+        if offset < 0 or size + offset > self.size:
             raise ValueError(f"size + offset ({size + offset}) must be <= buffer size ({self.size})")
-        self._copy(self.addr + offset, src.data_ptr(), size, stream)
+        local = RdmaBufferC(src.data_ptr(), size)
+        check(lib().mhip_buffer_read_into(C.byref(local), C.byref(self._remote(offset)), _torch.stream_handle(stream)))
 
 
 class TensorBuffer:

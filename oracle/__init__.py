@@ -259,6 +259,63 @@ def reduce(ins: Sequence[np.ndarray], op: int = SUM, out: np.ndarray | None = No
     return out
 
 
+PROD, MAX, MIN = 1, 2, 3
+_DTYPE_CODES = {"uint8": 0, "int8": 1, "int32": 3, "int64": 4, "float32": 6, "float64": 7}
+
+
+def reduce_op(ins: Sequence[np.ndarray], op: int, kind: str | None = None) -> np.ndarray:
+    """Any ReduceOp (SUM, PROD, MAX, MIN, AVG) over ``ins``.  uint16 arrays are bit patterns: ``kind`` says
+    whether of bf16 (default) or of IEEE half ("f16")."""
+    ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
+    dt = ins[0].dtype
+    code = (5 if kind == "f16" else 15) if dt == np.uint16 else _DTYPE_CODES[dt.name]
+    out = np.empty_like(ins[0])
+    ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+    rc = lib().o_reduce_op(_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint64(ins[0].size), C.c_int(code), C.c_int(op))
+    assert rc == 0
+    return out
+
+
+def stack(ins: Sequence[np.ndarray]) -> np.ndarray:
+    """Reduction::Stack without scatter: ``out[g] = ins[g]``, shape ``[n, numel]``."""
+    ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]
+    out = np.empty((len(ins), ins[0].size), dtype=ins[0].dtype)
+    ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+    lib().o_stack(_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint64(ins[0].size), C.c_uint32(ins[0].itemsize))
+    return out
+
+
+def stack_scatter(ins: Sequence[np.ndarray], rank: int, out: np.ndarray | None = None) -> np.ndarray:
+    """Reduction::Stack with scatter (all_to_all_single) as member ``rank`` sees it; ``out`` may be ``ins[rank]``."""
+    assert all(x.flags.c_contiguous for x in ins)
+    if out is None:
+        out = np.empty_like(ins[0].reshape(-1))
+    ptrs = (C.c_void_p * len(ins))(*[x.ctypes.data for x in ins])
+    rc = lib().o_stack_scatter(_ptr(out), ptrs, C.c_uint32(len(ins)), C.c_uint32(rank), C.c_uint64(ins[0].size),
+                               C.c_uint32(ins[0].itemsize))
+    if rc:
+        raise ValueError("numel must be a multiple of the group size and rank inside the group")
+    return out
+
+
+NO_RANK = (1 << 64) - 1
+
+
+def send_tensor_route(from_ranks: OSlice, to_ranks: OSlice, rank: int):
+    """``(from_rank, to_rank)`` of ``rank``, ``None`` where the reference has ``Option::None``."""
+    fr, to = C.c_uint64(), C.c_uint64()
+    lib().o_send_tensor_route(C.byref(from_ranks.c), C.byref(to_ranks.c), C.c_uint64(rank), C.byref(fr), C.byref(to))
+    return (None if fr.value == NO_RANK else fr.value, None if to.value == NO_RANK else to.value)
+
+
+def send_tensor(src_base: np.ndarray, view: OSlice) -> np.ndarray:
+    """The receiver's contiguous result for a sender holding ``view`` of the flat storage ``src_base``."""
+    src_base = np.ascontiguousarray(src_base).reshape(-1)
+    out = np.empty(len(view), dtype=src_base.dtype)
+    lib().o_send_tensor(_ptr(out), _ptr(src_base), C.byref(view.c), C.c_uint32(src_base.itemsize))
+    return out
+
+
 def reduce_scatter(ins: Sequence[np.ndarray], in_view: OSlice, out_views: Sequence[OSlice],
                    op: int = SUM) -> List[np.ndarray]:
     ins = [np.ascontiguousarray(x).reshape(-1) for x in ins]

@@ -16,8 +16,16 @@
  *     round-trip and tiling invariants.
  *   reduce sum (f32, exact-integer cases)          pinned: torch-sys-cuda/src/nccl.rs:850-873,
  *     1033-1065, python/tests/test_controller.py:188-254 closed forms.
- *   reduce avg, bf16 rounding                      pinned against torch's CPU cast/sum (a library
- *     routine) only; the reference holds no bf16 or avg vector: PARITY UNPINNED in the reference.
+ *   reduce avg, bf16 / f16 rounding, f64, reduce-scatter (f32 and bf16, Sum and Avg)
+ *                                                  pinned against explicit member-order adds in numpy / torch
+ *     (library routines) with n_in != n_out and strided input views; the reference holds no bf16, f64
+ *     or avg vector: PARITY UNPINNED in the reference.
+ *   reduce prod / max / min                        pinned against numpy multiply / fmax / fmin chains; the NaN and
+ *     signed-zero rule is NCCL's, which is outside the reference tree: PARITY UNPINNED in the reference.
+ *   stack (all_gather / all_to_all)                pinned: torch-sys-cuda/src/nccl.rs:927-959, 996-1031 vectors,
+ *     torch.stack / chunk.
+ *   send_tensor routing and result                 pinned: closed forms on the reference's mesh shapes
+ *     (python/tests/test_controller.py to_mesh cases), torch .contiguous().
  *   DeviceMesh members                             pinned: monarch_tensor_worker/src/device_mesh.rs:184-244.
  *   fp8 e4m3fn block-scaled codec                  no counterpart in the reference (fp8 reductions are
  *     refused, torch-sys-cuda/src/nccl.rs:474-476): PARITY UNPINNED in the reference; the encode/decode
@@ -446,6 +454,8 @@ void o_reduce_i64(int64_t* out, const int64_t* const* in, uint32_t n, uint64_t n
     }
 }
 
+static float o_combine_f32(float acc, float x, int op); /* defined with the other ops below */
+
 /* ---- Reduce with scatter ----
  * reduced[i] = op_g in[g][in_view.get(i)] over the logical index space of in_view;
  * outs[k][j] = reduced[out_views[k].get(j)].  With in_view contiguous [n*c] and
@@ -460,7 +470,7 @@ void o_reduce_scatter_f32(float* const* outs, const o_slice_t* out_views, uint32
             o_slice_get(&out_views[k], j, &i);
             o_slice_get(in_view, i, &loc);
             float acc = in[0][loc];
-            for (uint32_t g = 1; g < n_in; g++) acc += in[g][loc];
+            for (uint32_t g = 1; g < n_in; g++) acc = o_combine_f32(acc, in[g][loc], op);
             if (op == 4) acc = acc / (float)n_in;
             outs[k][j] = acc;
         }
@@ -476,11 +486,159 @@ void o_reduce_scatter_bf16(uint16_t* const* outs, const o_slice_t* out_views, ui
             o_slice_get(&out_views[k], j, &i);
             o_slice_get(in_view, i, &loc);
             float acc = bf16_to_f32(in[0][loc]);
-            for (uint32_t g = 1; g < n_in; g++) acc += bf16_to_f32(in[g][loc]);
+            for (uint32_t g = 1; g < n_in; g++) acc = o_combine_f32(acc, bf16_to_f32(in[g][loc]), op);
             if (op == 4) acc = acc / (float)n_in;
             outs[k][j] = f32_to_bf16_rne(acc);
         }
     }
+}
+
+/* ---- The other ReduceOps (torch-sys-cuda/src/nccl.rs:285-292: Prod = 1, Max = 2, Min = 3) ----
+ * Same shape as the Sum loops above: accumulate in member order in fp32 (f64 for f64, the integer
+ * type for integers), round once.  Max / Min are written out as comparisons so that every case is
+ * fixed: the accumulator is kept on ties (the first of +0 / -0 in member order wins) and a NaN operand
+ * is skipped unless all operands are NaN - the result fmaxf / fminf give, which is how NCCL's kernels
+ * compute ncclMax / ncclMin.  NCCL itself is not part of the reference tree and the reference holds no
+ * vector for these ops: PARITY UNPINNED against the reference; pinned against numpy (fmax / fmin /
+ * multiply) only.  Integer Prod wraps, as integer Sum does (parameter_server.rs:202). */
+static float o_combine_f32(float acc, float x, int op) {
+    switch (op) {
+        case 1: return acc * x;
+        case 2: return (x > acc || acc != acc) ? x : acc;
+        case 3: return (x < acc || acc != acc) ? x : acc;
+        default: return acc + x;
+    }
+}
+static double o_combine_f64(double acc, double x, int op) {
+    switch (op) {
+        case 1: return acc * x;
+        case 2: return (x > acc || acc != acc) ? x : acc;
+        case 3: return (x < acc || acc != acc) ? x : acc;
+        default: return acc + x;
+    }
+}
+#define O_INT_COMBINE(NAME, T, UT)                                 \
+    static T NAME(T acc, T x, int op) {                            \
+        switch (op) {                                              \
+            case 1: return (T)(UT)((UT)acc * (UT)x);               \
+            case 2: return x > acc ? x : acc;                      \
+            case 3: return x < acc ? x : acc;                      \
+            default: return (T)(UT)((UT)acc + (UT)x);              \
+        }                                                          \
+    }
+O_INT_COMBINE(o_combine_u8, uint8_t, uint8_t)
+O_INT_COMBINE(o_combine_i8, int8_t, uint8_t)
+O_INT_COMBINE(o_combine_i32, int32_t, uint32_t)
+O_INT_COMBINE(o_combine_i64, int64_t, uint64_t)
+
+/* out = op over the n inputs for any ReduceOp; dtype in c10::ScalarType numbering
+ * (0 u8, 1 i8, 3 i32, 4 i64, 5 f16, 6 f32, 7 f64, 15 bf16).  Returns 0, or -1 for an unknown dtype. */
+int o_reduce_op(void* out, const void* const* in, uint32_t n, uint64_t numel, int dtype, int op) {
+    for (uint64_t i = 0; i < numel; i++) {
+        switch (dtype) {
+            case 6: {
+                float acc = ((const float*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_f32(acc, ((const float*)in[r])[i], op);
+                if (op == 4) acc = acc / (float)n;
+                ((float*)out)[i] = acc;
+                break;
+            }
+            case 15: {
+                float acc = bf16_to_f32(((const uint16_t*)in[0])[i]);
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_f32(acc, bf16_to_f32(((const uint16_t*)in[r])[i]), op);
+                if (op == 4) acc = acc / (float)n;
+                ((uint16_t*)out)[i] = f32_to_bf16_rne(acc);
+                break;
+            }
+            case 5: {
+                float acc = f16_to_f32(((const uint16_t*)in[0])[i]);
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_f32(acc, f16_to_f32(((const uint16_t*)in[r])[i]), op);
+                if (op == 4) acc = acc / (float)n;
+                ((uint16_t*)out)[i] = f32_to_f16_rne(acc);
+                break;
+            }
+            case 7: {
+                double acc = ((const double*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_f64(acc, ((const double*)in[r])[i], op);
+                if (op == 4) acc = acc / (double)n;
+                ((double*)out)[i] = acc;
+                break;
+            }
+            case 0: {
+                uint8_t acc = ((const uint8_t*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_u8(acc, ((const uint8_t*)in[r])[i], op);
+                ((uint8_t*)out)[i] = acc;
+                break;
+            }
+            case 1: {
+                int8_t acc = ((const int8_t*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_i8(acc, ((const int8_t*)in[r])[i], op);
+                ((int8_t*)out)[i] = acc;
+                break;
+            }
+            case 3: {
+                int32_t acc = ((const int32_t*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_i32(acc, ((const int32_t*)in[r])[i], op);
+                ((int32_t*)out)[i] = acc;
+                break;
+            }
+            case 4: {
+                int64_t acc = ((const int64_t*)in[0])[i];
+                for (uint32_t r = 1; r < n; r++) acc = o_combine_i64(acc, ((const int64_t*)in[r])[i], op);
+                ((int64_t*)out)[i] = acc;
+                break;
+            }
+            default: return -1;
+        }
+    }
+    return 0;
+}
+
+/* ---- Reduction::Stack ----
+ * Without scatter: all_gather_into_tensor (monarch_tensor_worker/src/stream.rs:1408-1417), result
+ * [n, *shape]: out[g*numel + i] = in[g][i]; the reference's vector is torch-sys-cuda/src/nccl.rs:927-959. */
+void o_stack(void* out, const void* const* in, uint32_t n, uint64_t numel, uint32_t elem_size) {
+    for (uint32_t g = 0; g < n; g++)
+        for (uint64_t b = 0; b < numel * elem_size; b++)
+            ((uint8_t*)out)[(uint64_t)g * numel * elem_size + b] = ((const uint8_t*)in[g])[b];
+}
+/* With scatter: all_to_all_single (stream.rs:1381-1399; nccl.rs:760-812: count = numel / world_size,
+ * chunk r of the send buffer goes to rank r, the chunk received from rank r lands at chunk r) as
+ * member `rank` sees it: out[g*c + i] = in[g][rank*c + i].  Vector: nccl.rs:996-1031.  `out` is written
+ * through a temporary so that the in-place form (out == in[rank]) reads pre-exchange values. */
+int o_stack_scatter(void* out, const void* const* in, uint32_t n, uint32_t rank, uint64_t numel,
+                    uint32_t elem_size) {
+    if (n == 0 || numel % n != 0 || rank >= n) return -1;
+    uint64_t chunk = numel / n * elem_size;
+    uint8_t* tmp = (uint8_t*)malloc(chunk * n + 1);
+    if (!tmp) return -2;
+    for (uint32_t g = 0; g < n; g++) memcpy(tmp + g * chunk, (const uint8_t*)in[g] + rank * chunk, chunk);
+    memcpy(out, tmp, chunk * n);
+    free(tmp);
+    return 0;
+}
+
+/* ---- SendTensor ----
+ * Routing, monarch_tensor_worker/src/lib.rs:722-731: to_rank = to_ranks.get(from_ranks.index(rank)),
+ * from_rank = from_ranks.get(to_ranks.index(rank)); UINT64_MAX stands for None. */
+void o_send_tensor_route(const o_slice_t* from_ranks, const o_slice_t* to_ranks, uint64_t rank,
+                         uint64_t* from_rank, uint64_t* to_rank) {
+    uint64_t index, peer;
+    *to_rank = *from_rank = UINT64_MAX;
+    if (o_slice_index(from_ranks, rank, &index) == O_OK && o_slice_get(to_ranks, index, &peer) == O_OK)
+        *to_rank = peer;
+    if (o_slice_index(to_ranks, rank, &index) == O_OK && o_slice_get(from_ranks, index, &peer) == O_OK)
+        *from_rank = peer;
+}
+/* What StreamActor::send_tensor (stream.rs:1470-1560) leaves on the receiver: a fresh contiguous tensor
+ * of factory.size holding the sender's elements in logical (row-major, Slice::iter) order.  The sender's
+ * view goes through staging bytes, the transfer is a byte copy. */
+void o_send_tensor(void* result, const void* src_base, const o_slice_t* src_view, uint32_t elem_size) {
+    uint64_t bytes = o_slice_len(src_view) * elem_size;
+    uint8_t* staging = (uint8_t*)malloc(bytes ? bytes : 1);
+    o_slice_pack(staging, src_base, src_view, elem_size);
+    memcpy(result, staging, bytes);
+    free(staging);
 }
 
 /* ---- DeviceMesh, monarch_tensor_worker/src/device_mesh.rs:71-102 ----

@@ -181,6 +181,71 @@ int main(void) {
             }
     }
 
+    /* 5. RdmaBuffer transfers in several work requests, max of the 8 buffers, stack, and a column block sent
+     *    through staging memory (SendTensor) */
+    {
+        mhip_rdma_buffer_t local = {d[0], M * sizeof(uint16_t)}, remote = {dout, M * sizeof(uint16_t)};
+        CHECK(mhip_buffer_read_into(&local, &remote, stream));            /* d[0] -> dout */
+        uint32_t posted = 0;
+        CHECK(mhip_buffer_transfer(d[1], dout, M * sizeof(uint16_t), 4096, stream, &posted)); /* dout -> d[1] */
+        CHECK(mhip_memcpy_dtoh(out, d[1], M * sizeof(uint16_t), stream));
+        CHECK(mhip_stream_synchronize(stream));
+        if (posted != (M * sizeof(uint16_t) + 4095) / 4096 || memcmp(out, h[0], M * sizeof(uint16_t)) != 0) {
+            fprintf(stderr, "segmented buffer transfer failed (%u requests)\n", posted);
+            return 1;
+        }
+        memcpy(h[1], h[0], M * sizeof(uint16_t));
+        mhip_rdma_buffer_t small = {dq, 16};
+        if (mhip_buffer_read_into(&local, &small, stream) != MHIP_ERR_BUFFER_TOO_SMALL) {
+            fprintf(stderr, "a write past the remote buffer was not refused\n");
+            return 1;
+        }
+        CHECK(mhip_reduce(dout, dptr, G, M, MHIP_DTYPE_BF16, MHIP_OP_MAX, stream));
+        CHECK(mhip_memcpy_dtoh(out, dout, M * sizeof(uint16_t), stream));
+        CHECK(mhip_stream_synchronize(stream));
+        for (int i = 0; i < M; ++i) {
+            float best = bf16_to_f32(h[0][i]);
+            for (int g = 1; g < G; ++g) best = bf16_to_f32(h[g][i]) > best ? bf16_to_f32(h[g][i]) : best;
+            if (bf16_to_f32(out[i]) != best) {
+                fprintf(stderr, "max mismatch at %d\n", i);
+                return 1;
+            }
+        }
+        void* dstack;
+        CHECK(mhip_malloc(&dstack, (size_t)G * M * sizeof(uint16_t)));
+        CHECK(mhip_stack(dstack, dptr, G, M, sizeof(uint16_t), stream));
+        uint16_t* stacked = malloc((size_t)G * M * sizeof(uint16_t));
+        CHECK(mhip_memcpy_dtoh(stacked, dstack, (size_t)G * M * sizeof(uint16_t), stream));
+        CHECK(mhip_stream_synchronize(stream));
+        for (int g = 0; g < G; ++g)
+            if (memcmp(stacked + (size_t)g * M, h[g], M * sizeof(uint16_t)) != 0) {
+                fprintf(stderr, "stack mismatch in member %d\n", g);
+                return 1;
+            }
+        /* columns [64, 192) of the [1024, 256] f32 matrix at the start of x, sent as a [1024, 128] tensor */
+        const uint64_t csizes[2] = {1024, 128}, cstrides[2] = {256, 1};
+        const mhip_slice_t col = {64, 2, csizes, cstrides};
+        uint64_t from_rank = 0, to_rank = 0;
+        const uint64_t one = 1;
+        const mhip_slice_t from_ranks = {0, 1, &one, &one}, to_ranks = {1, 1, &one, &one};
+        CHECK(mhip_send_tensor_route(&from_ranks, &to_ranks, 1, &from_rank, &to_rank));
+        if (from_rank != 0 || to_rank != MHIP_NO_RANK) {
+            fprintf(stderr, "send_tensor routing: from %llu to %llu\n", (unsigned long long)from_rank, (unsigned long long)to_rank);
+            return 1;
+        }
+        CHECK(mhip_send_tensor(db, 1024 * 128 * sizeof(float), dx, &col, sizeof(float), dp, stream));
+        CHECK(mhip_memcpy_dtoh(back, db, 1024 * 128 * sizeof(float), stream));
+        CHECK(mhip_stream_synchronize(stream));
+        for (int r = 0; r < 1024; ++r)
+            for (int c = 0; c < 128; ++c)
+                if (back[r * 128 + c] != x[r * 256 + 64 + c]) {
+                    fprintf(stderr, "send_tensor mismatch at row %d column %d\n", r, c);
+                    return 1;
+                }
+        CHECK(mhip_free(dstack));
+        free(stacked);
+    }
+
     for (int g = 0; g < G; ++g) CHECK(mhip_free(d[g]));
     CHECK(mhip_free(dx)); CHECK(mhip_free(dp)); CHECK(mhip_free(db)); CHECK(mhip_free(dout));
     CHECK(mhip_free(dt)); CHECK(mhip_free(dq)); CHECK(mhip_free(dsc)); CHECK(mhip_free(dacc));

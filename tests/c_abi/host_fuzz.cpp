@@ -191,6 +191,82 @@ int main() {
             }
         }
     }
+    // caller-built structs that Slice::new would never produce, and extreme arguments: a status comes back, nothing
+    // divides by zero, wraps or reads out of bounds
+    {
+        case_no = 100000;
+        uint64_t out[4] = {0, 0, 0, 0}, w = 99;
+        const uint64_t four = 4, zero = 0, one = 1;
+        const mhip_slice_t zero_stride{0, 1, &four, &zero};
+        CHECK(mhip_slice_coordinates(&zero_stride, 2, out) == MHIP_ERR_INVALID_ARGUMENT);
+        CHECK(mhip_slice_index(&zero_stride, 0, out) == MHIP_ERR_INVALID_ARGUMENT);
+        CHECK(mhip_slice_enforce_embedding(&zero_stride, &zero_stride) == MHIP_ERR_INVALID_ARGUMENT);
+        uint64_t members[4];
+        CHECK(mhip_mesh_dim_members(&zero_stride, 0, 0, members, out) == MHIP_ERR_INVALID_ARGUMENT);
+        const mhip_slice_t plain{0, 1, &four, &one};
+        const uint64_t huge = ~0ull, two = 2;
+        CHECK(mhip_slice_subview(&plain, &huge, 1, &two, 1, out) == MHIP_ERR_INDEX_OUT_OF_RANGE);   // starts + lens wraps to 1
+        CHECK(mhip_slice_subview(&plain, &two, 1, &huge, 1, out) == MHIP_ERR_INDEX_OUT_OF_RANGE);
+        CHECK(mhip_slice_subview(&plain, &two, 1, &two, 1, out) == MHIP_SUCCESS && out[0] == 2);
+        uint64_t locs[4] = {7, 7, 7, 7};
+        CHECK(mhip_slice_iter(&plain, 1, huge, locs, &w) == MHIP_SUCCESS && w == 3 && locs[0] == 1 && locs[2] == 3);  // start + count wraps
+        CHECK(mhip_slice_iter(&plain, huge, huge, locs, &w) == MHIP_SUCCESS && w == 0);
+        const mhip_slice_t too_deep{0, MHIP_MAX_DIMS + 1, &four, &one};
+        CHECK(mhip_slice_len(&too_deep, out) == MHIP_ERR_INVALID_ARGUMENT);
+        const mhip_slice_t null_arrays{0, 2, nullptr, nullptr};
+        CHECK(mhip_slice_get(&null_arrays, 0, out) == MHIP_ERR_INVALID_ARGUMENT);
+    }
+
+    // SendTensor routing: the i-th sender pairs with the i-th receiver; to_mesh checks on random name lists
+    for (case_no = 200000; case_no < 202000; ++case_no) {
+        const uint64_t n_from = 1 + below(6), n_to = 1 + below(6), s_from = 1 + below(3), s_to = 1 + below(3);
+        const uint64_t o_from = below(10), o_to = below(30);
+        const mhip_slice_t from{o_from, 1, &n_from, &s_from}, to{o_to, 1, &n_to, &s_to};
+        for (uint64_t rank = 0; rank < 50; ++rank) {
+            uint64_t fr = 1, tr = 1;
+            CHECK(mhip_send_tensor_route(&from, &to, rank, &fr, &tr) == MHIP_SUCCESS);
+            uint64_t want_to = MHIP_NO_RANK, want_from = MHIP_NO_RANK;
+            if (rank >= o_from && (rank - o_from) % s_from == 0 && (rank - o_from) / s_from < n_from) {
+                const uint64_t i = (rank - o_from) / s_from;
+                if (i < n_to) want_to = o_to + i * s_to;
+            }
+            if (rank >= o_to && (rank - o_to) % s_to == 0 && (rank - o_to) / s_to < n_to) {
+                const uint64_t i = (rank - o_to) / s_to;
+                if (i < n_from) want_from = o_from + i * s_from;
+            }
+            CHECK(fr == want_from && tr == want_to);
+        }
+        const char* pool[] = {"host", "gpu", "replica", "pp"};
+        const uint32_t nm = (uint32_t)below(5), ns = (uint32_t)below(4);
+        const char* mesh_names[4];
+        const char* slicing_names[4];
+        uint64_t mesh_sizes[4], sl_sizes[4], sl_strides[4];
+        uint32_t perm[4] = {0, 1, 2, 3};
+        for (uint32_t k = 4; k > 1; --k) std::swap(perm[k - 1], perm[below(k)]);
+        for (uint32_t m = 0; m < nm; ++m) { mesh_names[m] = pool[perm[m]]; mesh_sizes[m] = 1 + below(3); }
+        uint32_t perm2[4] = {0, 1, 2, 3};
+        for (uint32_t k = 4; k > 1; --k) std::swap(perm2[k - 1], perm2[below(k)]);
+        for (uint32_t k = 0; k < ns; ++k) { slicing_names[k] = pool[perm2[k]]; sl_sizes[k] = 1 + below(3); sl_strides[k] = 1 + below(9); }
+        const mhip_slice_t slicing{below(5), ns, sl_sizes, sl_strides};
+        uint64_t osz[4], ost[4];
+        uint32_t ond = 77, bc[4], nbc = 77, culprit = 77;
+        const int rc = mhip_to_mesh_from_ranks(slicing_names, &slicing, mesh_names, mesh_sizes, nm, osz, ost, &ond, bc, &nbc, &culprit);
+        // by the definition (tensor.py:417-437)
+        int want = MHIP_SUCCESS;
+        uint32_t kept = 0, nb = 0;
+        for (uint32_t m = 0; m < nm && want == MHIP_SUCCESS; ++m) {
+            uint32_t idx = ns;
+            for (uint32_t k = 0; k < ns; ++k) if (slicing_names[k] == mesh_names[m]) idx = k;   // pool strings are unique objects
+            if (idx == ns) { ++nb; continue; }
+            if (sl_sizes[idx] != mesh_sizes[m]) { want = MHIP_ERR_MESH_DIM_LENGTH_MISMATCH; break; }
+            CHECK(rc != MHIP_SUCCESS || (osz[kept] == mesh_sizes[m] && ost[kept] == sl_strides[idx]));
+            ++kept;
+        }
+        if (want == MHIP_SUCCESS && kept != ns) want = MHIP_ERR_MESH_DIM_MISSING;
+        CHECK(rc == want);
+        if (rc == MHIP_SUCCESS) CHECK(ond == kept && nbc == nb);
+    }
+
     std::printf("ok: %" PRIu64 " valid and %" PRIu64 " invalid slices\n", n_valid, n_invalid);
     return 0;
 }

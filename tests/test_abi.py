@@ -45,7 +45,8 @@ def test_status_text_and_host_only_calls():
     one = (C.c_void_p * 1)(16)
     assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F8E4M3FN, 0, None) == _lib.ERR_FLOAT8_REDUCTION
     assert lib.mhip_reduce(16, one, 1, 4, 2, 0, None) == _lib.ERR_INVALID_DATA_TYPE
-    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F32, 2, None) == _lib.ERR_UNSUPPORTED_OP
+    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F32, 5, None) == _lib.ERR_UNSUPPORTED_OP
+    assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_F32, -1, None) == _lib.ERR_UNSUPPORTED_OP
     assert lib.mhip_reduce(16, one, 1, 4, _lib.DTYPE_I32, 4, None) == _lib.ERR_UNSUPPORTED_OP
     assert lib.mhip_reduce(16, one, 0, 4, _lib.DTYPE_F32, 0, None) == _lib.ERR_INVALID_ARGUMENT
     many = (C.c_void_p * 65)(*([16] * 65))
@@ -121,7 +122,8 @@ _RUST_TYPE = {
     "mhip_event_t*": "*mut mhip_event_t", "mhip_stream_t": "mhip_stream_t", "mhip_stream_t*": "*mut mhip_stream_t",
     "size_t": "usize", "size_t*": "*mut usize", "uint32_t": "u32", "uint64_t": "u64", "uint64_t*": "*mut u64",
     "uint8_t*": "*mut u8", "void*": "*mut c_void", "void* const*": "*const *mut c_void", "void**": "*mut *mut c_void",
-    "const char*": "*const c_char",
+    "const char*": "*const c_char", "const char* const*": "*const *const c_char", "uint32_t*": "*mut u32",
+    "const mhip_rdma_buffer_t*": "*const mhip_rdma_buffer_t",
 }
 
 

@@ -5,6 +5,7 @@ import torch
 
 import oracle
 from monarch_amd import Slice, staging
+from monarch_amd._lib import MhipError
 from util import valid_slices, bits, fuzz_slices, oslice, span, sync
 
 pytestmark = pytest.mark.gpu
@@ -355,12 +356,21 @@ def test_tensor_buffer_round_trip():
         buf.read_into(torch.zeros(buf.size + 1, dtype=torch.uint8, device=DEV))
 
 
-def test_rdma_buffer_transfer_in_segments(monkeypatch):
-    # a transfer longer than one work request can carry goes out as several segments
-    monkeypatch.setattr(staging, "MAX_SEGMENT_BYTES", 1008)
+def test_rdma_buffer_transfer_in_segments():
+    # a transfer longer than one work request can carry goes out as several requests (the length field of a
+    # scatter/gather entry is 32 bits, rdma_components.rs:1041,1063); here with the request size lowered
     g = torch.Generator().manual_seed(3)
     host = torch.randint(0, 256, (5003,), dtype=torch.uint8, generator=g)
-    buf = staging.RDMABuffer(host.to(DEV))
+    src = host.to(DEV)
+    for limit, nbytes, so, do in ((1008, 4000, 1001, 0), (16, 100, 3, 5), (4096, 4096, 0, 0), (0, 5003, 0, 0), (1, 37, 11, 2)):
+        dst = torch.zeros(nbytes + 16, dtype=torch.uint8, device=DEV)
+        posted = staging.transfer(dst.data_ptr() + do, src.data_ptr() + so, nbytes, limit)
+        sync()
+        assert posted == (1 if limit == 0 else -(-nbytes // limit))
+        want = torch.zeros(nbytes + 16, dtype=torch.uint8)
+        want[do: do + nbytes] = host[so: so + nbytes]
+        assert torch.equal(dst.cpu(), want)
+    buf = staging.RDMABuffer(src)
     dst = torch.zeros(4000, dtype=torch.uint8, device=DEV)
     assert buf.read_into(dst, offset=1001) == 4000
     sync()
@@ -370,6 +380,71 @@ def test_rdma_buffer_transfer_in_segments(monkeypatch):
     want = host.clone()
     want[7:3007] = 9
     assert torch.equal(buf.data.cpu(), want)
+    # the library's own RdmaBuffer calls: local.size bytes, in the direction the name says
+    import ctypes as C
+    from monarch_amd._lib import RdmaBufferC, lib
+    a = torch.arange(64, dtype=torch.uint8, device=DEV)
+    b = torch.zeros(100, dtype=torch.uint8, device=DEV)
+    la, rb = RdmaBufferC(a.data_ptr(), 64), RdmaBufferC(b.data_ptr(), 100)
+    assert lib().mhip_buffer_read_into(C.byref(la), C.byref(rb), None) == 0        # a -> b (put)
+    sync()
+    assert torch.equal(b[:64].cpu(), a.cpu()) and torch.count_nonzero(b[64:]) == 0
+    b[:64] = 7
+    assert lib().mhip_buffer_write_from(C.byref(la), C.byref(rb), None) == 0       # b -> a (get)
+    sync()
+    assert torch.all(a == 7)
+
+
+def test_staging_buffers_are_validated_before_launch():
+    x = torch.zeros(8, 8, device=DEV)
+    s = Slice(offset=0, sizes=[8, 4], strides=[8, 1])
+    with pytest.raises(ValueError, match="exactly len"):
+        staging.pack(x, s, out=torch.empty(31, device=DEV))
+    with pytest.raises(MhipError):
+        staging.pack(x, s, out=torch.empty(32))                      # host memory
+    with pytest.raises(ValueError, match="exactly len"):
+        staging.pack_many(x, [s, s], outs=[torch.empty(32, device=DEV), torch.empty(16, device=DEV)])
+    with pytest.raises(ValueError, match="staging buffers"):
+        staging.pack_many(x, [s, s], outs=[torch.empty(32, device=DEV)])
+    with pytest.raises(ValueError, match="contiguous"):
+        staging.unpack(x, s, torch.empty(32, 2, device=DEV)[:, 0])
+
+
+def test_config3_reshard_end_to_end():
+    # to_mesh of a column-sharded weight: [4096, 14336] bf16 -> 8 column-block views -> 8 staging buffers ->
+    # buffer transfer (several requests each) -> 8 receiver tensors [4096, 1792]; and back into a zeroed weight
+    from monarch_amd.reduce import Factory
+    from monarch_amd.send_tensor import route, stream_send_tensor
+    rows, cols, k = 4096, 14336, 8
+    w = cols // k
+    g = torch.Generator(device=DEV).manual_seed(3000)
+    x = (torch.randn(rows, cols, generator=g, device=DEV) * 0.02).bfloat16()
+    views = [Slice(offset=j * w, sizes=[rows, w], strides=[cols, 1]) for j in range(k)]
+    area = staging.StagingArea(k, rows * w * 2, DEV)
+    bufs = [area.slot(j) for j in range(k)]
+    staging.pack_many(x, views, outs=[b.view(torch.bfloat16) for b in bufs])
+    recv = [torch.empty(rows, w, dtype=torch.bfloat16, device=DEV) for _ in range(k)]
+    for j in range(k):
+        posted = staging.transfer(recv[j].data_ptr(), bufs[j].data_ptr(), rows * w * 2, 4 << 20)
+        assert posted == 4                                    # 14 MiB in requests of 4 MiB
+    sync()
+    hx = bits(x).reshape(-1)
+    for j in (0, 3, 7):
+        want = oracle.send_tensor(hx, oslice(views[j]))
+        assert np.array_equal(bits(recv[j]).reshape(-1), want), j
+    for j in range(k):
+        assert torch.equal(recv[j], x[:, j * w:(j + 1) * w])
+    back = torch.zeros_like(x)
+    staging.unpack_many(back, views, [r.view(-1) for r in recv])
+    sync()
+    assert torch.equal(back.view(torch.int16), x.view(torch.int16))
+    # the same through the SendTensor entry point, one message per destination rank
+    from_ranks, to_ranks = Slice(offset=0, sizes=[1], strides=[1]), Slice(offset=5, sizes=[1], strides=[1])
+    assert route(from_ranks, to_ranks, 5) == (0, None) and route(from_ranks, to_ranks, 0) == (None, 5)
+    col = x[:, 5 * w: 6 * w]                                   # the sender's (non-contiguous) tensor
+    got = stream_send_tensor({0: col}, 5, 0, None, Factory.of(col), staging_bytes=bufs[5])
+    sync()
+    assert got.is_contiguous() and np.array_equal(bits(got).reshape(-1), oracle.send_tensor(hx, oslice(views[5])))
 
 
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64, torch.complex128])

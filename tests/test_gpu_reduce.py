@@ -128,9 +128,8 @@ def test_reduce_argument_errors():
     with pytest.raises(MhipError) as e:
         R.all_reduce(out, [x] * 65, R.ReduceOp.Sum)
     assert e.value.name == "TooManyInputs"
-    with pytest.raises(MhipError) as e:
-        R.all_reduce(out, [x], R.ReduceOp.Max)
-    assert e.value.name == "UnsupportedOp"
+    rc = _lib.lib().mhip_reduce(out.data_ptr(), _lib.ptr_array([x.data_ptr()]), 1, 16, _lib.DTYPE_F32, 5, None)
+    assert rc == _lib.ERR_UNSUPPORTED_OP          # outside ncclRedOp_t, nccl.rs:285-292
     with pytest.raises(MhipError) as e:
         R.all_reduce(out, [x.double()], R.ReduceOp.Sum)
     assert e.value.name == "TypeMismatch"
@@ -505,3 +504,136 @@ def test_stream_reduce_placement_and_errors():
     b = R.reduce(ones, m2, ("x", "y"), "sum")
     sync()
     assert torch.all(a == 2.0) and torch.all(b == 4.0)
+
+
+# ---------------- Prod / Max / Min, Reduction::Stack ----------------
+
+_OTHER = ((R.ReduceOp.Prod, oracle.PROD), (R.ReduceOp.Max, oracle.MAX), (R.ReduceOp.Min, oracle.MIN))
+
+
+def _obits(t):
+    """Host array as the oracle's reduce_op wants it: signed integers keep their sign, bf16 / f16 become bits."""
+    return bits(t)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16, torch.float64, torch.uint8, torch.int8,
+                                   torch.int32, torch.int64])
+@pytest.mark.parametrize("n", [1, 2, 3, 8, 9, 17])
+def test_reduce_prod_max_min_bit_exact(dtype, n):
+    for numel in (1, 7, 1000, 4099, (1 << 17) + 5):
+        hosts = [_rand(dtype, numel, 900 * n + r) for r in range(n)]
+        if dtype in (torch.bfloat16, torch.float16):
+            hosts = [h * 60 for h in hosts]      # products of values around 1, not around 0.02^n
+        devs = [h.to(DEV) for h in hosts]
+        for op, code in _OTHER:
+            out = torch.empty_like(devs[0])
+            R.all_reduce(out, devs, op)
+            sync()
+            want = oracle.reduce_op([_obits(h) for h in hosts], code, kind="f16" if dtype == torch.float16 else None)
+            assert np.array_equal(_obits(out), want), (dtype, n, numel, op)
+
+
+def test_reduce_max_min_nan_zero_rule_and_in_place():
+    nan, inf = float("nan"), float("inf")
+    a = torch.tensor([1.0, nan, nan, 3.0, nan, -0.0, 0.0, -inf, 5.0])
+    b = torch.tensor([nan, 2.0, nan, nan, -5.0, 0.0, -0.0, inf, 5.0])
+    c = torch.tensor([0.5, nan, nan, 4.0, nan, -0.0, -0.0, 0.0, -5.0])
+    for dtype in (torch.float32, torch.bfloat16, torch.float16, torch.float64):
+        hs = [t.to(dtype) for t in (a, b, c)]
+        for op, code in _OTHER[1:]:
+            work = [h.to(DEV) for h in hs]
+            R.all_reduce(work[1], work, op)          # in place on member 1
+            sync()
+            want = oracle.reduce_op([_obits(h) for h in hs], code, kind="f16" if dtype == torch.float16 else None)
+            got = _obits(work[1])
+            if dtype in (torch.float32, torch.float64):
+                assert np.array_equal(np.isnan(got), np.isnan(want))
+                ok = ~np.isnan(want)
+                assert np.array_equal(got[ok], want[ok]) and np.array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+            else:
+                assert np.array_equal(got, want)     # bit patterns, NaN canonical on both sides
+
+
+def test_reduce_scatter_other_ops():
+    rng = np.random.default_rng(12)
+    hosts = [rng.uniform(-2, 2, size=(6, 40)).astype(np.float32) for _ in range(3)]
+    devs = [torch.from_numpy(h).to(DEV) for h in hosts]
+    in_view = Slice(offset=0, sizes=[6, 40], strides=[40, 1])
+    for views in ([Slice(offset=10 * k, sizes=[6, 10], strides=[40, 1]) for k in range(4)],      # vector form
+                  [Slice(offset=k, sizes=[6, 13], strides=[40, 3]) for k in range(3)]):           # element form
+        for op, code in _OTHER:
+            outs = [torch.empty(len(v), device=DEV) for v in views]
+            R.reduce_scatter_views(outs, views, devs, in_view, op)
+            sync()
+            want = oracle.reduce_scatter([h.reshape(-1) for h in hosts], oslice(in_view), [oslice(v) for v in views], code)
+            for o, w in zip(outs, want):
+                assert np.array_equal(o.cpu().numpy(), w), op
+    hb = [torch.from_numpy(h).bfloat16() for h in hosts]
+    db = [h.to(DEV) for h in hb]
+    views = [Slice(offset=k * 7, sizes=[6, 7], strides=[40, 1]) for k in range(5)]                # ragged rows
+    for op, code in _OTHER:
+        outs = [torch.empty(len(v), dtype=torch.bfloat16, device=DEV) for v in views]
+        R.reduce_scatter_views(outs, views, db, in_view, op)
+        sync()
+        want = oracle.reduce_scatter([bits(h).reshape(-1) for h in hb], oslice(in_view), [oslice(v) for v in views], code)
+        for o, w in zip(outs, want):
+            assert np.array_equal(bits(o), w), op
+
+
+def test_stack_reference_vectors():
+    # all_gather_into_tensor, torch-sys-cuda/src/nccl.rs:927-959
+    group = [torch.full((2, 2), float(i), device=DEV) for i in range(2)]
+    for rank in range(2):
+        out = R.stream_reduce(group, rank, R.Factory.of(group[0]), R.Reduction.from_str("stack"), False, False)
+        sync()
+        assert out.shape == (2, 2, 2) and torch.equal(out, torch.stack(group))
+    # all_to_all_single, nccl.rs:996-1031
+    group = [torch.tensor([0.0, 1.0], device=DEV), torch.tensor([2.0, 3.0], device=DEV)]
+    want = [[0.0, 2.0], [1.0, 3.0]]
+    for rank in range(2):
+        out = R.stream_reduce(group, rank, R.Factory.of(group[0]), R.Reduction.from_str("stack"), True, False)
+        sync()
+        assert out.cpu().tolist() == want[rank]
+    with pytest.raises(ValueError, match="in-place, non-scatter not supported for stack reduce"):   # stream.rs:1403-1406
+        R.stream_reduce(group, 0, R.Factory.of(group[0]), R.Reduction.from_str("stack"), False, True)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.float64])
+@pytest.mark.parametrize("n", [1, 2, 5, 8, 64])
+def test_stack_and_stack_scatter_against_oracle(dtype, n):
+    import ctypes as C
+    lib = _lib.lib()
+    es = torch.empty(0, dtype=dtype).element_size()
+    for per in (1, 3, 8, 1000, 4099, 65536 + 24):
+        numel = per * n
+        hosts = [_rand(dtype, numel + 3, 31 * n + r) for r in range(n)]
+        for skew in (0, 1):                                # element-aligned only when skewed
+            devs = [h.to(DEV)[skew: skew + numel] for h in hosts]
+            hs = [bits(h)[skew: skew + numel] for h in hosts]
+            out = torch.zeros(n * numel + 2, dtype=dtype, device=DEV)
+            ov = out[skew: skew + n * numel]
+            rc = lib.mhip_stack(ov.data_ptr(), _lib.ptr_array([d.data_ptr() for d in devs]), n, numel, es, None)
+            assert rc == 0
+            sync()
+            assert np.array_equal(bits(ov), oracle.stack(hs).reshape(-1)), (dtype, n, per, skew)
+            assert bits(out)[-1] == 0 and (skew == 0 or bits(out)[0] == 0)
+            for rank in sorted({0, n // 2, n - 1}):
+                o2 = torch.zeros(numel + 2, dtype=dtype, device=DEV)
+                rc = lib.mhip_stack_scatter(o2[1: 1 + numel].data_ptr(), _lib.ptr_array([d.data_ptr() for d in devs]), n,
+                                            rank, numel, es, None)
+                assert rc == 0
+                sync()
+                assert np.array_equal(bits(o2)[1: 1 + numel], oracle.stack_scatter(hs, rank)), (dtype, n, per, rank)
+                assert bits(o2)[0] == 0 and bits(o2)[-1] == 0
+    # in place on the member's own tensor (stream.rs:1383-1384)
+    per = 517
+    hosts = [_rand(dtype, per * n, 77 + r) for r in range(n)]
+    devs = [h.to(DEV) for h in hosts]
+    rank = n - 1
+    out = R.stream_reduce(devs, rank, R.Factory.of(devs[0]), R.Reduction.from_str("stack"), True, True)
+    sync()
+    assert out.data_ptr() == devs[rank].data_ptr()
+    assert np.array_equal(bits(out), oracle.stack_scatter([bits(h) for h in hosts], rank))
+    for g in range(n):
+        if g != rank:
+            assert np.array_equal(bits(devs[g]), bits(hosts[g]))       # peers untouched

@@ -316,15 +316,84 @@ def test_send_tensor_routing_and_to_mesh_checks():
         check_to_mesh(["host", "gpu"], slicing, ["gpu"], [8])
 
 
-def test_transfer_segments_cover_the_range():
-    # lengths fit the 32-bit field of a scatter/gather entry (rdma_components.rs:1041,1063)
-    from monarch_amd.staging import MAX_SEGMENT_BYTES, transfer_segments
+def test_transfer_and_stack_argument_checks_without_a_gpu():
+    # everything that is refused before a launch: lengths fit the 32-bit field of a scatter/gather entry
+    # (rdma_components.rs:1041,1063), buffers must be large enough, stack chunks must divide evenly
+    import ctypes as C
+    from monarch_amd import _lib
+    from monarch_amd._lib import RdmaBufferC
+    from monarch_amd.staging import MAX_SEGMENT_BYTES
+    lib = _lib.lib()
     assert MAX_SEGMENT_BYTES < 2**32 and MAX_SEGMENT_BYTES % 16 == 0
-    assert list(transfer_segments(0)) == []
-    assert list(transfer_segments(100)) == [(0, 100)]
-    assert list(transfer_segments(10, max_bytes=4)) == [(0, 4), (4, 4), (8, 2)]
-    big = list(transfer_segments(3 * 2**32 + 5))
-    assert [o for o, _ in big] == [0, MAX_SEGMENT_BYTES, 2 * MAX_SEGMENT_BYTES, 3 * MAX_SEGMENT_BYTES]
-    assert sum(n for _, n in big) == 3 * 2**32 + 5 and all(n <= MAX_SEGMENT_BYTES for _, n in big)
-    with pytest.raises(ValueError):
-        list(transfer_segments(1, max_bytes=0))
+    posted = C.c_uint32(7)
+    assert lib.mhip_buffer_transfer(None, None, 0, 0, None, C.byref(posted)) == 0 and posted.value == 0
+    assert lib.mhip_buffer_transfer(None, 16, 32, 0, None, None) == _lib.ERR_UNDEFINED_TENSOR
+    small, big = RdmaBufferC(4096, 100), RdmaBufferC(8192, 101)
+    assert lib.mhip_buffer_read_into(C.byref(big), C.byref(small), None) == _lib.ERR_BUFFER_TOO_SMALL
+    assert lib.mhip_buffer_write_from(C.byref(big), C.byref(small), None) == _lib.ERR_BUFFER_TOO_SMALL
+    assert lib.mhip_buffer_read_into(None, C.byref(small), None) == _lib.ERR_INVALID_ARGUMENT
+    empty = RdmaBufferC(None, 0)
+    assert lib.mhip_buffer_read_into(C.byref(empty), C.byref(small), None) == 0     # nothing to move
+    one = (C.c_void_p * 2)(4096, 8192)
+    assert lib.mhip_stack_scatter(4096, one, 2, 0, 7, 4, None) == _lib.ERR_INPUT_SIZE_MISMATCH   # 7 elements, 2 members
+    assert lib.mhip_stack_scatter(4096, one, 2, 2, 8, 4, None) == _lib.ERR_INDEX_OUT_OF_RANGE
+    assert lib.mhip_stack(4096, one, 0, 8, 4, None) == _lib.ERR_INVALID_ARGUMENT
+    assert lib.mhip_stack(None, one, 2, 8, 4, None) == _lib.ERR_UNDEFINED_TENSOR
+    assert lib.mhip_stack(4096, one, 2, 0, 4, None) == 0
+    many = (C.c_void_p * 65)(*([4096] * 65))
+    assert lib.mhip_stack(4096, many, 65, 8, 4, None) == _lib.ERR_TOO_MANY_INPUTS
+    assert lib.mhip_stack(4098, one, 2, 8, 4, None) == _lib.ERR_INVALID_ARGUMENT     # not element-aligned
+    s = Slice(offset=0, sizes=[4, 6], strides=[6, 1])
+    assert lib.mhip_send_tensor(4096, 95, 8192, C.byref(s.c), 4, None, None) == _lib.ERR_OUTPUT_SIZE_MISMATCH
+    assert lib.mhip_send_tensor(None, 96, 8192, C.byref(s.c), 4, None, None) == _lib.ERR_UNDEFINED_TENSOR
+    bad = Slice(offset=0, sizes=[2, 2], strides=[2, 2], _validate=False)
+    assert lib.mhip_send_tensor(4096, 16, 8192, C.byref(bad.c), 4, None, None) == _lib.ERR_NONUNIQUE_STRIDES
+
+
+def test_send_tensor_routing_matches_reference_cases_and_oracle():
+    import random
+    import oracle
+    from monarch_amd.send_tensor import check_to_mesh, route
+    # monarch_tensor_worker/src/comm.rs:1493-1537: from_ranks {0,[1],[1]}, to_ranks {1,[1],[1]} on ranks 0 and 1;
+    # comm.rs:1662 (send_tensor_local): both slices {0,[1],[1]}
+    one = lambda off: Slice(offset=off, sizes=[1], strides=[1])
+    assert route(one(0), one(1), 0) == (None, 1) and route(one(0), one(1), 1) == (0, None)
+    assert route(one(0), one(0), 0) == (0, 0)
+    # python/tests/test_controller.py:311-323 (test_movement) on a 2 x 2 mesh {0,[2,2],[2,1]}: host 0 -> host 1
+    sm0, sm1 = Slice(offset=0, sizes=[2], strides=[1]), Slice(offset=2, sizes=[2], strides=[1])
+    fr, bc = check_to_mesh(["gpu"], sm0, ["gpu"], [2])
+    assert fr == sm0 and bc == []
+    assert [route(fr, sm1, r) for r in range(4)] == [(None, 2), (None, 3), (0, None), (1, None)]
+    # test_controller.py:325-338 (test_broadcast_one): host=1 submesh to the whole mesh broadcasts along host
+    fr, bc = check_to_mesh(["gpu"], sm1, ["host", "gpu"], [2, 2])
+    assert fr == sm1 and bc == ["host"]
+    # test_controller.py:340-352 (test_broadcast_two): a single device (no named dims left) to the whole mesh
+    fr, bc = check_to_mesh([], Slice(offset=3, sizes=[], strides=[]), ["host", "gpu"], [2, 2])
+    assert fr == Slice(offset=3, sizes=[], strides=[]) and bc == ["host", "gpu"]
+    assert route(fr, one(0), 3) == (None, 0) and route(fr, one(0), 0) == (3, None)
+    # random rank slices: the library's routing and the oracle's agree on every rank, senders and receivers pair up
+    gen = random.Random(7)
+    for _ in range(200):
+        nd = gen.randrange(1, 4)
+        sizes = [gen.randrange(1, 4) for _ in range(nd)]
+        strides, acc = [], 1
+        for z in reversed(sizes):
+            strides.insert(0, acc)
+            acc *= z * gen.randrange(1, 3)
+        a = Slice(offset=gen.randrange(5), sizes=sizes, strides=strides)
+        kind = gen.randrange(3)
+        if kind == 0:      # same shape elsewhere
+            b = Slice(offset=gen.randrange(40), sizes=sizes, strides=strides)
+        elif kind == 1:    # same number of ranks, another shape
+            rm = Slice.new_row_major(sizes[::-1])
+            b = Slice(offset=gen.randrange(40), sizes=rm.sizes, strides=rm.strides)
+        else:              # fewer or more receivers than senders
+            b = Slice(offset=gen.randrange(40), sizes=[gen.randrange(1, 7)], strides=[gen.randrange(1, 3)])
+        oa, ob = oracle.OSlice.unchecked(a.offset, a.sizes, a.strides), oracle.OSlice.unchecked(b.offset, b.sizes, b.strides)
+        senders, receivers = list(a), list(b)
+        for rank in range(0, 80):
+            got = route(a, b, rank)
+            assert got == oracle.send_tensor_route(oa, ob, rank), (a, b, rank)
+            want_to = receivers[senders.index(rank)] if rank in senders and senders.index(rank) < len(receivers) else None
+            want_from = senders[receivers.index(rank)] if rank in receivers and receivers.index(rank) < len(senders) else None
+            assert got == (want_from, want_to)

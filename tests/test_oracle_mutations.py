@@ -3,11 +3,14 @@ copy of ``oracle/monarch_oracle.c`` (a wrong divisor, a rounding per add, a drop
 transposed index chain), builds it, puts it in the oracle's place and expects the named pin test to
 fail.  A pin that passes on the mutated build pins nothing."""
 import os
+import re
 import subprocess
 
+import numpy as np
 import pytest
 
 import oracle
+import test_oracle_collectives as K
 import test_oracle_numeric as T
 
 SRC = os.path.join(os.path.dirname(oracle.__file__), "monarch_oracle.c")
@@ -18,10 +21,10 @@ MUTATIONS = [
      lambda: T.test_reduce_scatter_bf16_member_order(T.AVG, 3, 2)),
     ("scatter_f32_divides_by_n_out", "o_reduce_scatter_f32", "acc = acc / (float)n_in", "acc = acc / (float)n_out",
      lambda: T.test_reduce_scatter_f32_avg_member_order(3, 2)),
-    ("scatter_bf16_rounds_per_add", "o_reduce_scatter_bf16", "acc += bf16_to_f32(in[g][loc])",
+    ("scatter_bf16_rounds_per_add", "o_reduce_scatter_bf16", "acc = o_combine_f32(acc, bf16_to_f32(in[g][loc]), op)",
      "acc = bf16_to_f32(f32_to_bf16_rne(acc + bf16_to_f32(in[g][loc])))",
      lambda: T.test_reduce_scatter_bf16_member_order(T.SUM, 5, 4)),
-    ("scatter_bf16_drops_last_member", "o_reduce_scatter_bf16", "g < n_in; g++) acc += bf16", "g + 1 < n_in; g++) acc += bf16",
+    ("scatter_bf16_drops_last_member", "o_reduce_scatter_bf16", "g < n_in; g++) acc = o_combine_f32(acc, bf16", "g + 1 < n_in; g++) acc = o_combine_f32(acc, bf16",
      lambda: T.test_reduce_scatter_bf16_member_order(T.SUM, 3, 2)),
     ("scatter_f32_skips_in_view", "o_reduce_scatter_f32", "o_slice_get(in_view, i, &loc)", "loc = i",
      lambda: T.test_reduce_scatter_f32_avg_member_order(5, 4)),
@@ -33,11 +36,30 @@ MUTATIONS = [
      "double acc = in[0][i];\n        for (uint32_t r = 1; r < n; r++) acc += in[r][i];",
      "double acc = in[n - 1][i];\n        for (uint32_t r = n - 1; r-- > 0;) acc += in[r][i];",
      lambda: T.test_reduce_f64_left_to_right(7)),
+    ("max_propagates_nan", "o_combine_f32", "case 2: return (x > acc || acc != acc) ? x : acc;",
+     "case 2: return (x > acc || x != x) ? x : acc;", K.test_max_min_nan_and_signed_zero_rule),
+    ("min_takes_the_later_zero", "o_combine_f32", "case 3: return (x < acc || acc != acc) ? x : acc;",
+     "case 3: return (x <= acc || acc != acc) ? x : acc;", K.test_max_min_nan_and_signed_zero_rule),
+    ("int8_max_compares_unsigned", "o_reduce_op", "int8_t acc = ((const int8_t*)in[0])[i];\n                for (uint32_t r = 1; r < n; r++) acc = o_combine_i8(acc, ((const int8_t*)in[r])[i], op);",
+     "uint8_t acc = ((const uint8_t*)in[0])[i];\n                for (uint32_t r = 1; r < n; r++) acc = o_combine_u8(acc, ((const uint8_t*)in[r])[i], op);",
+     lambda: K.test_integer_prod_wraps_and_max_min_follow_the_sign(np.int8)),
+    ("bf16_prod_rounds_per_step", "o_reduce_op", "acc = o_combine_f32(acc, bf16_to_f32(((const uint16_t*)in[r])[i]), op);",
+     "acc = bf16_to_f32(f32_to_bf16_rne(o_combine_f32(acc, bf16_to_f32(((const uint16_t*)in[r])[i]), op)));",
+     lambda: K.test_bf16_and_f16_other_ops_accumulate_in_fp32_and_round_once(K.PROD)),
+    ("all_to_all_sends_own_chunk_index", "o_stack_scatter", "(const uint8_t*)in[g] + rank * chunk", "(const uint8_t*)in[g] + g * chunk",
+     K.test_stack_scatter_matches_reference_all_to_all_vector),
+    ("all_to_all_in_place_reads_overwritten_chunks", "o_stack_scatter",
+     "memcpy(tmp + g * chunk, (const uint8_t*)in[g] + rank * chunk, chunk);\n    memcpy(out, tmp, chunk * n);",
+     "memcpy((uint8_t*)out + g * chunk, (const uint8_t*)in[(g + 1) % n] + rank * chunk, chunk);\n    for (uint32_t g = 0; g < n; g++) memcpy((uint8_t*)out + g * chunk, (const uint8_t*)in[g] + rank * chunk, chunk);",
+     K.test_stack_scatter_matches_reference_all_to_all_vector),
+    ("send_route_swaps_the_sides", "o_send_tensor_route", "        *to_rank = peer;", "        *from_rank = peer;",
+     K.test_send_tensor_result_is_the_contiguous_view),
 ]
 
 
 def _mutate(text, func, old, new):
-    start = text.index(func + "(")
+    # the definition: a line at top level that names the function and opens a body
+    start = re.search(r"^[A-Za-z_][\w \*]*\b" + func + r"\([^;{]*\)\s*\{", text, flags=re.M).start()
     end = text.index("\n}\n", start)
     body = text[start:end]
     assert body.count(old) == 1, (func, old, body.count(old))
