@@ -297,7 +297,7 @@ int mhip_send_tensor(void* result, size_t result_bytes, const void* src_base,
  * reductions, torch-sys-cuda/src/nccl.rs:275-278,474-476).  Per `block` consecutive
  * elements of a flat bf16 buffer (last block may be short):
  *   absmax = max|x| (NaN ignored) clamped to [2^-40, FLT_MAX];  scales[b] = absmax / 448
- *   q[i] = e4m3fn_rne(clamp(x[i] * (448 / absmax), -448, 448)), NaN -> fp8 NaN
+ *   q[i] = e4m3fn_rne(clamp(x[i] * (448 / absmax), -448, 448)), NaN -> the fp8 NaN code with x[i]'s sign
  * block must be 1024 (MHIP_ERR_UNSUPPORTED_BLOCK otherwise). */
 int mhip_fp8_quantize(uint8_t* q, float* scales, const void* x_bf16, uint64_t numel,
                       uint32_t block, mhip_stream_t stream);

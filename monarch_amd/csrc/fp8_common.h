@@ -46,6 +46,9 @@ __device__ __forceinline__ int quant_pair(uint32_t w, float inv, int old) {
 }
 
 __device__ __forceinline__ uint8_t quant_one_careful(uint32_t h, float inv) {
+    // NaN -> the fp8 NaN code with the input's sign, whatever its payload.  Taken from the bits: the multiply
+    // below quiets a signalling NaN, and the sign of what the conversion then produces is not the input's.
+    if ((h & 0x7fffu) > 0x7f80u) return (uint8_t)(((h >> 8) & 0x80u) | 0x7fu);
     float y = __uint_as_float(h << 16) * inv;
     y = y > kFp8Max ? kFp8Max : y;    // comparisons are false for NaN: it passes through
     y = y < -kFp8Max ? -kFp8Max : y;

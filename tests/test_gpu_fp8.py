@@ -23,9 +23,7 @@ def _check_quant(x: torch.Tensor):
     sync()
     wq, ws = oracle.fp8_quantize(bits(x), 1024)
     gq = q.cpu().numpy()
-    nan = (wq & 0x7F) == 0x7F
-    assert np.array_equal((gq & 0x7F) == 0x7F, nan)
-    assert np.array_equal(gq[~nan], wq[~nan])
+    assert np.array_equal(gq, wq)                      # every code, the sign bit of NaN codes included
     assert np.array_equal(s.cpu().numpy().view(np.uint32), ws.view(np.uint32))
     return q, s
 
