@@ -26,16 +26,33 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 METRIC = "pack/unpack + reduce GB/s on 1 MI355X, % of HBM peak, vs host-CPU path"
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/);
-# None until a counter run exists for the workload.
-MEASURED_TRAFFIC = {  # profiles/bench_workloads_all_kernels.md, column "scaled traffic B"
-    "c2": 452_868_627, "c2_inplace": 452_868_813, "c2_separate": 452_867_743, "c2p_pack": 100_663_296,
-    "c2p_unpack": 100_663_323, "c3_pack": 234_865_257, "c3_unpack": 234_865_222, "c4": 603_819_720,
-    "c4_slots": 603_821_319, "c5_flat_pack": 3_166_109_361, "c5_quantize": 2_384_059_401,
-    "c5_dequant": 7_127_817_329, "c5_flat_unpack": 6_014_978_770, "c5_dequant_many8": 12_779_870_515,
-    "c5_quantize_bucket": 2_374_361_487, "c5_dequant_bucket": 7_176_519_083, "tr_f32_pack": 536_870_344,
-    "tr_f32_unpack": 536_870_553, "tr_bf16_pack": 268_487_701, "tr_bf16_unpack": 268_483_118,
-}
+# HBM bytes per launch come from the committed rocprofv3 counter summary (FETCH_SIZE / WRITE_SIZE runs, scaled by what the
+# same counters read for a plain copy of known size): the table is read from the file, so a figure here is always the
+# one the profile states.  A workload without a row reports null.
+TRAFFIC_SOURCE = os.path.join("profiles", "bench_workloads_all_kernels.md")
+
+
+def measured_traffic(path: str = None) -> dict:
+    """workload -> {"traffic": scaled HBM bytes per launch, "algorithmic": bytes per launch} from the summary's table."""
+    path = path or os.path.join(ROOT, TRAFFIC_SOURCE)
+    table = {}
+    if not os.path.exists(path):
+        return table
+    header = None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if "scaled traffic B" in cells and "workload" in cells:
+            header = cells
+            continue
+        if header and len(cells) == len(header) and not set(cells[0]) <= set("-: "):
+            row = dict(zip(header, cells))
+            try:
+                table[row["workload"]] = {"traffic": int(row["scaled traffic B"]), "algorithmic": int(row["algorithmic B"])}
+            except ValueError:
+                continue
+        elif header and not line.strip().startswith("|"):
+            header = None
+    return table
 
 
 def _load():
@@ -369,6 +386,94 @@ def wl_c3(torch, unpack=False, sets=3):
     return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 
 
+def wl_c3_reshard(torch, sets=3):
+    """Configuration 3 end to end (SendTensor / to_mesh of a column-sharded weight): the 8 column blocks are packed
+    into 8 staging buffers in one launch, and each buffer is transferred into its receiver's contiguous tensor.
+    Bytes per step: pack reads and writes 117 MB, the transfers read and write them again."""
+    from monarch_amd import Slice, staging
+    from monarch_amd._lib import ptr_array
+    from monarch_amd.ndslice import slice_array
+    g = torch.Generator(device="cuda:0").manual_seed(3000)
+    rows, cols, k = 4096, 14336, 8
+    w = cols // k
+    views = [Slice(offset=j * w, sizes=[rows, w], strides=[cols, 1]) for j in range(k)]
+    arr = slice_array(views)
+    bufs = []
+    for _ in range(sets):
+        x = (torch.randn(rows, cols, generator=g, device="cuda:0") * 0.02).bfloat16()
+        area = staging.StagingArea(k, rows * w * 2)
+        recv = [torch.empty(rows, w, dtype=torch.bfloat16, device="cuda:0") for _ in range(k)]
+        staging.pack_many(x, views, [area.slot(j, torch.bfloat16) for j in range(k)])
+        bufs.append((x, area, recv))
+    nbytes = 4 * rows * cols * 2
+    seqs = []
+    for x, area, recv in bufs:
+        seq = [prepared("mhip_slice_pack_many", ptr_array([area.slot(j).data_ptr() for j in range(k)]), x.data_ptr(), arr, k, 2,
+                        STREAM())]
+        seq += [prepared("mhip_buffer_transfer", recv[j].data_ptr(), area.slot(j).data_ptr(), rows * w * 2, 0, STREAM(), None)
+                for j in range(k)]
+        seqs.append(seq)
+
+    def launch(i):
+        rc = 0
+        for f in seqs[i % sets]:
+            rc |= f()
+        return rc
+
+    def cpu():
+        import oracle
+        h = bufs[0][0].cpu().view(torch.uint16).numpy().reshape(-1)
+        v = oracle.OSlice(views[0].offset, views[0].sizes, views[0].strides)
+        t0 = time.perf_counter()
+        oracle.send_tensor(h, v)
+        dt = (time.perf_counter() - t0) * k
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "1 of the 8 column blocks through the oracle's send_tensor (Slice::get walk + byte copy), scaled x8"}
+
+    return "c3_reshard_end_to_end", nbytes, launch, cpu, "slice_copy_kernel<16> + 8 x contiguous_copy_kernel", "u8"
+
+
+def wl_stack(torch, scatter=False, sets=2):
+    """Reduction::Stack of the C2 bucket's 8 chunks in one launch: all_gather_into_tensor (out[g] = in[g]) or, with
+    scatter, all_to_all_single as member 3 sees it (out chunk g = chunk 3 of member g)."""
+    from monarch_amd import staging
+    from monarch_amd._lib import ptr_array
+    n, numel = 8, 25_165_824
+    g = torch.Generator(device="cuda:0").manual_seed(2002)
+    bufs = []
+    for _ in range(sets):
+        area = staging.StagingArea(n, numel * 2)
+        ins = area.slots(torch.bfloat16)
+        for t in ins:
+            t.copy_((torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16())
+        out = torch.empty((1 if scatter else n) * numel, dtype=torch.bfloat16, device="cuda:0")
+        bufs.append((area, ins, out))
+    nbytes = 2 * (1 if scatter else n) * numel * 2
+    if scatter:
+        calls = [prepared("mhip_stack_scatter", out.data_ptr(), ptr_array([t.data_ptr() for t in ins]), n, 3, numel, 2, STREAM())
+                 for _, ins, out in bufs]
+    else:
+        calls = [prepared("mhip_stack", out.data_ptr(), ptr_array([t.data_ptr() for t in ins]), n, numel, 2, STREAM())
+                 for _, ins, out in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import oracle
+        hs = [t.cpu().view(torch.uint16).numpy() for t in bufs[0][1]]
+        t0 = time.perf_counter()
+        if scatter:
+            oracle.stack_scatter(hs, 3)
+        else:
+            oracle.stack(hs)
+        dt = time.perf_counter() - t0
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "full workload, 1 pass of the oracle's byte loops"}
+
+    return ("stack_scatter_bf16_8" if scatter else "stack_bf16_8"), nbytes, launch, cpu, "stack_copy_kernel", "u8"
+
+
 def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
     from monarch_amd import Slice, staging
     n = int(os.environ.get("MONARCH_BENCH_TRANSPOSE_N", "8192"))
@@ -446,35 +551,63 @@ def wl_c4(torch, sets=2, slots=False):
         t0 = time.perf_counter()
         oracle.reduce_scatter([hx[gi * pitch:] for gi in range(G)], ov, [o0], oracle.SUM)
         dt = (time.perf_counter() - t0) * K
+        # the library path of the same work on the host: sum over the gpu axis, then 8 contiguous column slices
+        # (the shape rule of python/monarch/common/tensor.py:494-503 followed by the column-block scatter)
+        if slots:
+            ht = torch.stack([torch.from_numpy(hx[i * pitch: i * pitch + slab]) for i in range(H * G)]).view(H, G, Rr, Cc)
+        else:
+            ht = torch.from_numpy(hx).view(H, G, Rr, Cc)
+        ht.sum(1)
+        t1 = time.perf_counter()
+        red = ht.sum(1)
+        cols = [red[:, :, k * w:(k + 1) * w].contiguous() for k in range(K)]
+        dt_torch = time.perf_counter() - t1
+        del cols
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "1 of the 8 scatter outputs through the oracle, scaled x8"}
+                "sample": "1 of the 8 scatter outputs through the oracle, scaled x8",
+                "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                              "sample": "one pass of x.sum(1) and 8 .contiguous() column slices on the full tensor"}}
 
     name = "c4_mesh_dim_reduce_scatter_f32" + ("_staging_slots" if slots else "")
     return name, nbytes, launch, cpu, "reduce_scatter_kernel<f32,vec>", "f32"
 
 
+_C5 = {}
+
+
 def _c5_setup(torch):
-    import numpy as np
-    from monarch_amd import fp8
-    rng = np.random.default_rng(5000)
-    sizes = np.round(np.exp(rng.uniform(np.log(2**10), np.log(2**22), size=1500))).astype(np.int64).tolist()
-    total = sum(sizes)
-    g = torch.Generator(device="cuda:0").manual_seed(5001)
-    x = torch.randn(total, generator=g, device="cuda:0")
-    x = torch.where(torch.rand(total, generator=g, device="cuda:0") < 1e-3, x * 50, x).bfloat16()
-    offs = np.concatenate([[0], np.cumsum(sizes)])
-    tensors = [x[offs[i]: offs[i + 1]].clone() for i in range(1500)]
-    del x
-    bucket = fp8.FlatBucket(tensors)
-    return fp8, bucket, tensors, sizes, total
+    """The bucket of configuration 5, built once per process: its stages share the tensors, the flat buffer and the payload."""
+    if not _C5:
+        import numpy as np
+        from monarch_amd import fp8
+        rng = np.random.default_rng(5000)
+        sizes = np.round(np.exp(rng.uniform(np.log(2**10), np.log(2**22), size=1500))).astype(np.int64).tolist()
+        total = sum(sizes)
+        g = torch.Generator(device="cuda:0").manual_seed(5001)
+        x = torch.randn(total, generator=g, device="cuda:0")
+        x = torch.where(torch.rand(total, generator=g, device="cuda:0") < 1e-3, x * 50, x).bfloat16()
+        offs = np.concatenate([[0], np.cumsum(sizes)])
+        tensors = [x[offs[i]: offs[i + 1]].clone() for i in range(1500)]
+        del x
+        bucket = fp8.FlatBucket(tensors)
+        flat = bucket.pack()
+        q, s = fp8.quantize(flat)
+        _C5.update(fp8=fp8, bucket=bucket, tensors=tensors, sizes=sizes, total=total, flat=flat, q=q, s=s)
+    c = _C5
+    return c["fp8"], c["bucket"], c["tensors"], c["sizes"], c["total"], c["flat"], c["q"], c["s"]
+
+
+def release_shared():
+    _C5.clear()
 
 
 def wl_c5(torch, stage="quantize"):
-    fp8, bucket, tensors, sizes, total = _c5_setup(torch)
+    fp8, bucket, tensors, sizes, total, flat, q, s = _c5_setup(torch)
     nblk = (total + 1023) // 1024
-    flat = bucket.pack()
-    q, s = fp8.quantize(flat)
-    acc = torch.zeros(total, device="cuda:0")
+    acc = torch.zeros(total, device="cuda:0") if "dequant" in stage or stage == "flat_unpack" else None
+    if stage in ("flat_pack", "quantize", "quantize_bucket"):   # these write the shared buffers: give them their own
+        flat = torch.empty_like(flat) if stage == "flat_pack" else flat
+        q, s = (torch.empty_like(q), torch.empty_like(s)) if stage != "flat_pack" else (q, s)
     outs = [torch.empty(n, device="cuda:0") for n in sizes] if stage == "flat_unpack" else None
     if stage == "flat_pack":
         nbytes, kern = 4 * total, "flat_copy_kernel<pack>"
@@ -553,8 +686,19 @@ def wl_c5(torch, stage="quantize"):
             else:
                 oracle.flat_unpack(np.zeros(sample, dtype=np.float32), offs)
         dt = (time.perf_counter() - t0) * (total / sample)
-        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": f"first {sample} elements of the flat buffer through the oracle, scaled to {total}"}
+        rec = {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+               "sample": f"first {sample} elements of the flat buffer through the oracle, scaled to {total}"}
+        if stage in ("quantize", "quantize_bucket"):
+            # the library path of the same codec on the host: per-block absmax, scale, clamp to +-448, torch's e4m3fn cast
+            ht = torch.from_numpy(h[: sample // 1024 * 1024].view(np.int16)).view(torch.bfloat16)
+            t1 = time.perf_counter()
+            xf = ht.float().view(-1, 1024)
+            amax = xf.abs().amax(1, keepdim=True).clamp_min(2.0**-40)
+            (xf * (448.0 / amax)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+            dt_torch = (time.perf_counter() - t1) * (total / ht.numel())
+            rec["torch_cpu"] = {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                                "sample": f"absmax / scale / clamp / to(float8_e4m3fn) over the first {ht.numel()} elements, scaled"}
+        return rec
 
     return f"c5_fp8_{stage}", nbytes, launch, cpu, kern, "bf16->f8e4m3fn"
 
@@ -584,6 +728,9 @@ WORKLOADS = {
     "c2p_unpack": lambda t: wl_c2p(t, True),
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
+    "c3_reshard_e2e": wl_c3_reshard,
+    "stack8": lambda t: wl_stack(t, False),
+    "stack_scatter8": lambda t: wl_stack(t, True),
     "c4": wl_c4,
     "c4_slots": lambda t: wl_c4(t, slots=True),
     "tr_f32_pack": lambda t: wl_transpose(t, "f32", False),
@@ -602,9 +749,19 @@ WORKLOADS = {
 }
 
 
-def run(workload: str, steps: int, warmup: int, cpu_baseline: bool):
-    torch, lib, _ = _load()
-    torch.cuda.set_device(0)
+# The default run reports these beside the headline workload, measured in the same process:
+# workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
+SUMMARY = {
+    "c2": 0.75, "c2_inplace": 0.75, "c2_separate": 0.75, "c2p_pack": 0.75, "c2p_unpack": 0.75,
+    "c3_pack": 0.60, "c3_unpack": 0.60, "c3_reshard_e2e": 0.60, "c4": 0.60, "c4_slots": 0.60,
+    "c5_flat_pack": 0.60, "c5_quantize": 0.60, "c5_dequant": 0.60, "c5_flat_unpack": 0.60,
+    "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
+    "stack8": None, "stack_scatter8": None,
+    "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
+}
+
+
+def measure(torch, lib, workload: str, steps: int, warmup: int):
     name, nbytes, launch, cpu, kernel, dtype = WORKLOADS[workload](torch)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = 0
@@ -618,22 +775,66 @@ def run(workload: str, steps: int, warmup: int, cpu_baseline: bool):
         rc |= launch(i)
     kernel_ms = ev.stop_ms() / steps
     if rc != 0:
-        sys.exit(f"a launch returned status {rc}")
+        sys.exit(f"a launch of {workload} returned status {rc}")
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+    return dict(name=name, nbytes=nbytes, cpu=cpu, kernel=kernel, dtype=dtype, kernel_ms=kernel_ms, wall_ms=wall_ms,
+                keep=launch)
+
+
+def run(workload: str, steps: int, warmup: int, cpu_baseline: bool, summary: bool = False):
+    torch, lib, _ = _load()
+    torch.cuda.set_device(0)
+    traffic = measured_traffic()
+    m = measure(torch, lib, workload, steps, warmup)
+    nbytes = m["nbytes"]
+    achieved = nbytes / (m["kernel_ms"] * 1e-3) / 1e9
     rec = {
-        "metric": METRIC, "value": nbytes / (wall_ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
-        "steps": steps, "warmup": warmup, "ms_per_step": wall_ms, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
-        "config": {"workload": name, "algorithmic_bytes_per_step": nbytes, "kernel": kernel,
+        "metric": METRIC, "value": nbytes / (m["wall_ms"] * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": m["wall_ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": m["dtype"], "data": "synthetic",
+        "config": {"workload": m["name"], "algorithmic_bytes_per_step": nbytes, "kernel": m["kernel"],
                    **({"layout": LAYOUT[workload]} if workload in LAYOUT else {})},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC.get(workload)},
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic.get(workload, {}).get("traffic"),
+                     "traffic_source": TRAFFIC_SOURCE},
     }
     if cpu_baseline:
-        rec["cpu_baseline"] = cpu()
+        rec["cpu_baseline"] = m["cpu"]()
         rec["cpu_baseline"]["host_cpus"] = os.cpu_count()
+    if summary:
+        # every other class of the path, same process, same method (HIP events on the launch stream, rotating buffer
+        # sets), fewer launches; the CPU legs here are the short ones (the headline's own leg runs above)
+        import gc
+        k_steps, k_warm = max(5, min(steps, 60)), max(2, min(warmup, 10))
+        cpu_legs = ("c2p_pack", "c3_pack", "c3_reshard_e2e", "c4", "c5_quantize", "c5_dequant", "stack8")
+
+        def entry(w, mm, with_cpu):
+            ach = mm["nbytes"] / (mm["kernel_ms"] * 1e-3) / 1e9
+            e = {"workload": mm["name"], "kernel": mm["kernel"], "ms": mm["kernel_ms"], "achieved": ach,
+                 "frac": ach / HBM_PEAK_GBS, "target": SUMMARY[w], "algorithmic_bytes": mm["nbytes"],
+                 "traffic": traffic.get(w, {}).get("traffic")}
+            if with_cpu:
+                e["cpu_baseline"] = mm["cpu"]()
+            return e
+
+        out = {}
+        if workload in SUMMARY:
+            out[workload] = entry(workload, m, False)
+        m = None
+        for w in SUMMARY:
+            if w in out:
+                continue
+            gc.collect()
+            torch.cuda.empty_cache()  # the previous workload's buffer sets go back before the next ones are made
+            mm = measure(torch, lib, w, k_steps, k_warm)
+            out[w] = entry(w, mm, cpu_baseline and w in cpu_legs)
+            mm = None
+        out = {w: out[w] for w in SUMMARY}
+        rec["workloads"] = out
+        rec["config"]["workloads_note"] = (f"each entry of `workloads`: {k_steps} launches after {k_warm} warm-up launches, HIP events "
+                                           "on the launch stream; target = fraction of HBM peak asked of the class")
+    release_shared()
     return rec
 
 
@@ -642,18 +843,22 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
-    ap.add_argument("--all", action="store_true", help="also run every other workload; their lines go to stderr")
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
+    ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    headline = args.workload or "c2"
     if args.all:
         for w in sorted(WORKLOADS):
-            if w != args.workload:
+            if w != headline:
                 rec = run(w, args.steps, args.warmup, not args.no_cpu_baseline)
                 print(json.dumps(rec), file=sys.stderr, flush=True)
-    print(json.dumps(run(args.workload, args.steps, args.warmup, not args.no_cpu_baseline)), flush=True)
+    # a named workload is a single measurement (what the profiler runs); the default run adds the summary
+    summary = args.workload is None and not args.no_summary
+    print(json.dumps(run(headline, args.steps, args.warmup, not args.no_cpu_baseline, summary)), flush=True)
 
 
 if __name__ == "__main__":

@@ -14,6 +14,23 @@ def test_more_than_one_gpu_is_refused():
     assert r.returncode != 0 and "one GPU" in (r.stdout + r.stderr)
 
 
+def test_traffic_figures_come_from_the_committed_profile_summary():
+    sys.path.insert(0, ROOT)
+    import bench
+    table = bench.measured_traffic()
+    text = open(os.path.join(ROOT, bench.TRAFFIC_SOURCE)).read()
+    assert "rocprofv3 --pmc FETCH_SIZE" in text and "rocprofv3 --pmc WRITE_SIZE" in text    # the commands that made it
+    for w, target in bench.SUMMARY.items():
+        assert w in bench.WORKLOADS
+        if target is not None:
+            assert w in table, f"{w}: a workload with a roofline target needs a counter row in {bench.TRAFFIC_SOURCE}"
+    for w, row in table.items():
+        assert w in bench.WORKLOADS, w
+        assert f"| {row['traffic']} |" in text                      # the very figure the summary states
+        assert 0.9 < row["traffic"] / row["algorithmic"] < 1.1, (w, row)   # no wasted re-reads anywhere
+    assert table["c2"]["algorithmic"] == 9 * 25_165_824 * 2 and table["c3_pack"]["algorithmic"] == 2 * 4096 * 14336 * 2
+
+
 @pytest.mark.gpu
 def test_default_bench_line():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "1", "--steps", "10", "--warmup", "3"],
@@ -38,3 +55,16 @@ def test_default_bench_line():
     assert cpu["sample"] and cpu["all_cores"]["cores"] >= 1
     # wall-clock throughput cannot exceed the kernel-time throughput by more than timer noise
     assert rec["value"] <= roof["achieved"] * 1.10
+    # every class of the path is reported in the same line, measured in the same process
+    sys.path.insert(0, ROOT)
+    import bench
+    wl = rec["workloads"]
+    assert list(wl) == list(bench.SUMMARY)
+    for w, e in wl.items():
+        assert e["ms"] > 0 and abs(e["frac"] - e["achieved"] / 8000.0) < 1e-9 and 0.2 < e["frac"] < 1.0, (w, e)
+        assert e["target"] == bench.SUMMARY[w] and e["algorithmic_bytes"] > 0
+        if e["traffic"] is not None:
+            assert 0.9 < e["traffic"] / e["algorithmic_bytes"] < 1.1, (w, e)
+    assert wl["c2"]["frac"] == roof["frac"]
+    for w in ("c4", "c5_quantize"):
+        assert wl[w]["cpu_baseline"]["torch_cpu"]["value"] > 0
