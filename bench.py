@@ -749,6 +749,71 @@ WORKLOADS = {
 }
 
 
+def sweep_transpose_walks(dtypes, reps=5, launches=30):
+    """A/B of the transposing kernel's tile walks (--sweep transpose_walks): every variant is switched in turn inside
+    one process through MONARCH_HIP_TRANSPOSE_WALK, medians of `reps` alternations of `launches` launches, three
+    rotating buffer sets.  Prints one Markdown table per element size: fraction of HBM peak per variant."""
+    torch, lib, _ = _load()
+    from monarch_amd import Slice
+    torch.cuda.set_device(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    libc = C.CDLL(None)
+
+    def setenv(v):
+        if v is None:
+            libc.unsetenv(b"MONARCH_HIP_TRANSPOSE_WALK")
+        else:
+            libc.setenv(b"MONARCH_HIP_TRANSPOSE_WALK", v.encode(), 1)
+
+    types = {"u8": (torch.uint8, 1), "bf16": (torch.bfloat16, 2), "f32": (torch.float32, 4), "f64": (torch.float64, 8)}
+    # (batch, rows, cols, pitch): of a [batch, rows, pitch] tensor the part [:, :, :cols] is packed transposed
+    shapes = [(1, 8192, 8192, 8192), (1, 4096, 4096, 4096), (4, 4096, 4096, 4096), (1, 16384, 8192, 8192),
+              (1, 8192, 16384, 16384), (1, 8192, 4096, 4096), (1, 4096, 8192, 8192), (8, 2048, 8192, 8192),
+              (1, 8064, 8064, 8064), (1, 8200, 8200, 8200), (1, 8192, 8192, 8320), (1, 8192, 8192, 8256),
+              (1, 6144, 6144, 6144), (1, 12288, 12288, 12288), (1, 5000, 7000, 7000)]
+    variants = {"library": None, "blocked 4": "0,1,4,0", "blocked 4 rot": "0,1,4,1", "blocked 8": "0,1,8,0",
+                "blocked 8 rot": "0,1,8,1", "blocked 16": "0,1,16,0", "packed fastest": "1,0", "memory fastest": "2,0",
+                "diagonal, XCD ranges": "3,1", "diagonal": "3,0"}
+    for name in dtypes:
+        dt, es = types[name]
+        print(f"\n### {name} ({es}-byte elements)\n")
+        print("| batch, rows, cols, pitch | direction | " + " | ".join(variants) + " | best |")
+        print("|---|---|" + "---:|" * len(variants) + "---|")
+        for (b, r, c, pitch) in shapes:
+            if b * r * pitch * es > (3 << 30):
+                continue
+            bufs = []
+            for _ in range(3):
+                x = torch.empty(b, r, pitch, dtype=dt, device="cuda:0")
+                x.view(torch.uint8).random_(0, 255)
+                bufs.append((x, torch.empty(b * r * c, dtype=dt, device="cuda:0")))
+            s = Slice.of_tensor(bufs[0][0][:, :, :c].transpose(1, 2))
+            for sym in ("mhip_slice_pack", "mhip_slice_unpack"):
+                if sym.endswith("unpack"):
+                    calls = [prepared(sym, x.data_ptr(), st.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+                else:
+                    calls = [prepared(sym, st.data_ptr(), x.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+                res = {k: [] for k in variants}
+                for _ in range(reps):
+                    for k, v in variants.items():
+                        setenv(v)
+                        for i in range(4):
+                            assert calls[i % 3]() == 0
+                        torch.cuda.synchronize()
+                        ev = Events(lib, stream)
+                        ev.start()
+                        for i in range(launches):
+                            calls[i % 3]()
+                        res[k].append(2 * b * r * c * es / (ev.stop_ms() / launches) / 1e6 / HBM_PEAK_GBS)
+                setenv(None)
+                med = {k: sorted(v)[len(v) // 2] for k, v in res.items()}
+                best = max(med, key=med.get)
+                print(f"| {b}, {r}, {c}, {pitch} | {sym[11:]} | " + " | ".join(f"{med[k]:.3f}" for k in variants) + f" | {best} |",
+                      flush=True)
+            del bufs, calls
+            torch.cuda.empty_cache()
+
+
 # The default run reports these beside the headline workload, measured in the same process:
 # workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
 SUMMARY = {
@@ -847,9 +912,14 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep", choices=["transpose_walks"], help="print an A/B table instead of the bench line")
+    ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep == "transpose_walks":
+        sweep_transpose_walks(args.dtypes.split(","))
+        return
     headline = args.workload or "c2"
     if args.all:
         for w in sorted(WORKLOADS):

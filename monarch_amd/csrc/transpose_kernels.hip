@@ -7,12 +7,18 @@
 // tile: it reads rows that are contiguous along c, parks them in LDS, and writes rows
 // that are contiguous along q, so that both HBM sides see coalesced wavefront accesses
 // (the direct gather would fetch a whole 64-byte sector per element on one side).
-// The LDS tile is padded by one element per row: the transposed read then walks
-// consecutive banks instead of hitting one bank 64 times.
+// Elements of 1, 2, 4 and 8 bytes use slice_transpose_vec_kernel (256- or 512-byte tile rows, 16 bytes per lane
+// on both HBM sides, LDS rows XOR-permuted in 16-byte groups); only the 16-byte-element variant,
+// slice_transpose_kernel, uses a 32 x 32 tile padded by one element per row.
+#include <cstdio>
+
 #include "mhip_device.h"
 #include "pack_internal.h"
 
 namespace mhip {
+
+// Orders in which the workgroups of the vector kernel take tiles.
+enum : uint32_t { kWalkBlocked = 0, kWalkPackedFastest = 1, kWalkMemoryFastest = 2, kWalkDiagonal = 3 };
 
 struct TransArgs {
     char* base;
@@ -22,6 +28,8 @@ struct TransArgs {
     uint32_t Sc, Q;    // extent along c and along q
     uint32_t ctiles, qtiles;
     uint64_t wg0;      // workgroups of this copy launched before this grid (a multiple of 8)
+    uint32_t walk;      // kWalk*: the order in which workgroups take tiles (chosen on the host, see choose_walk)
+    uint32_t xcd_ranges;  // 1: each XCD (workgroup index mod 8) owns a contiguous eighth of the walk; 0: workgroup i takes tile i
     uint32_t rotate;    // rotate the c-groups of each eighth of the walk against the previous one (see the host side)
     uint32_t qgroups;   // ceil(qtiles / group)
     uint64_t rows_per_eighth;  // ceil(nbatch * qgroups / 8)
@@ -191,25 +199,45 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
     T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
     const uint64_t per_batch = (uint64_t)a.cgroups * ((a.qtiles + a.group - 1) / a.group) * a.group * a.group;
 
-    // XCD-contiguous tile ranges: workgroup w runs on XCD w % 8
+    // workgroup w runs on XCD w % 8
     const uint64_t per_xcd = (a.ntiles + 7) / 8;
     const uint64_t wg = a.wg0 + blockIdx.x;
-    const uint64_t tile_id = (wg % 8) * per_xcd + wg / 8;
+    const uint64_t tile_id = a.xcd_ranges ? (wg % 8) * per_xcd + wg / 8 : wg;
     if (tile_id >= a.ntiles) return;
 
-    const uint64_t b = tile_id / per_batch;
-    const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
-    const uint32_t gsz = a.group * a.group;
-    const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
-    const uint32_t gq = grp / a.cgroups;
-    uint32_t gc = grp - gq * a.cgroups;
-    if (a.rotate) {
-        // a function of the row of groups alone, so that every row still visits each of its c-groups once
-        const uint32_t eighth = (uint32_t)((b * a.qgroups + gq) / a.rows_per_eighth);  // 0..7: the XCD, when ranges hold whole rows
-        gc = (gc + eighth * a.cgroups / 8) % a.cgroups;
+    uint64_t b;
+    uint32_t qt, ct;
+    if (a.walk == kWalkBlocked) {
+        b = tile_id / per_batch;
+        const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
+        const uint32_t gsz = a.group * a.group;
+        const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
+        const uint32_t gq = grp / a.cgroups;
+        uint32_t gc = grp - gq * a.cgroups;
+        if (a.rotate) {
+            // a function of the row of groups alone, so that every row still visits each of its c-groups once
+            const uint32_t eighth = (uint32_t)((b * a.qgroups + gq) / a.rows_per_eighth);  // 0..7: the XCD, when ranges hold whole rows
+            gc = (gc + eighth * a.cgroups / 8) % a.cgroups;
+        }
+        qt = gq * a.group + within / a.group;
+        ct = gc * a.group + within % a.group;
+        if (qt >= a.qtiles || ct >= a.ctiles) return;  // padding of the blocked walk (uniform per workgroup)
+    } else {
+        const uint64_t plain = (uint64_t)a.qtiles * a.ctiles;
+        b = tile_id / plain;
+        const uint32_t t = (uint32_t)(tile_id - b * plain);
+        if (a.walk == kWalkPackedFastest) {          // neighbours write neighbouring pieces of the same packed rows
+            ct = t / a.qtiles;
+            qt = t - ct * a.qtiles;
+        } else if (a.walk == kWalkMemoryFastest) {   // neighbours read neighbouring pieces of the same memory rows
+            qt = t / a.ctiles;
+            ct = t - qt * a.ctiles;
+        } else {                                     // kWalkDiagonal: neighbours differ in both coordinates
+            const uint32_t d = t / a.qtiles;
+            qt = t - d * a.qtiles;
+            ct = (d + qt) % a.ctiles;
+        }
     }
-    const uint32_t qt = gq * a.group + within / a.group, ct = gc * a.group + within % a.group;
-    if (qt >= a.qtiles || ct >= a.ctiles) return;  // padding of the blocked walk (uniform per workgroup)
     // A tile that would hang over the edge is moved back inside when the extent allows it: it
     // then overlaps its neighbour, and both write the same bytes to the overlap.
     uint32_t q0 = qt * TQ, c0 = ct * TC;
@@ -390,6 +418,45 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
     }
 }
 
+// Which walk a launch takes.  Measured on MI355X over fifteen shapes, both directions and four element sizes, every
+// variant switched in turn inside one process (the table is profiles/transpose_walk_ab.md):
+//   * when every row pitch of both sides is a multiple of 4 KiB (power-of-two matrices and the like), the rows of a
+//     tile all fall on the same few positions of HBM's address interleave, and so do the tiles of a block of the
+//     blocked walk.  The diagonal walk - consecutive workgroups step one tile along q AND along c, no XCD ranges -
+//     keeps the workgroups in flight spread over all positions on both sides: 1/2/4-byte elements +0.025 to +0.037
+//     of peak on average over the shapes of that class (-0.05 to +0.12 on single shapes); 8-byte elements lose
+//     0.03 with it and keep the blocked walk;
+//   * at every other pitch the rows of a tile spread by themselves, neighbouring tiles share partial cache lines, and
+//     the blocked XCD-contiguous walk wins (the diagonal one loses 0.02 to 0.10 there).
+// MONARCH_HIP_TRANSPOSE_WALK overrides the choice (a tuning aid, read at every call so that variants can be
+// switched in turn inside one process): "<walk>[,<xcd_ranges>[,<group>[,<rotate>]]]" with walk 0 blocked,
+// 1 packed side fastest, 2 memory side fastest, 3 diagonal.
+static void choose_walk(TransArgs* a, uint32_t unit, uint64_t nbatch) {
+    bool interleave_aligned = unit <= 4 && ((uint64_t)a->Q * unit) % 4096 == 0;
+    for (int k = 0; interleave_aligned && k < a->n_inner; ++k)
+        if ((a->inner_stride[k] * unit) % 4096 != 0) interleave_aligned = false;
+    if (interleave_aligned) {
+        a->walk = kWalkDiagonal;
+        a->xcd_ranges = 0;
+        a->rotate = 0;
+    }
+    if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_WALK")) {
+        unsigned walk = 0, ranges = 1, group = a->group, rotate = 0;
+        const int n = std::sscanf(e, "%u,%u,%u,%u", &walk, &ranges, &group, &rotate);
+        if (n >= 1 && walk <= kWalkDiagonal) {
+            a->walk = walk;
+            a->xcd_ranges = n >= 2 ? (ranges ? 1 : 0) : 1;
+            a->rotate = n >= 4 ? (rotate ? 1 : 0) : 0;
+        }
+        if (n >= 3 && group >= 1 && group <= 64) {
+            a->group = group;
+            a->cgroups = (a->ctiles + group - 1) / group;
+            a->qgroups = (a->qtiles + group - 1) / group;
+            a->rows_per_eighth = (nbatch * a->qgroups + 7) / 8;
+        }
+    }
+}
+
 template <bool PACK>
 bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t unit, hipStream_t stream, int* rc) {
     if (c.run != 1 || c.ndim < 2 || c.ndim > kMaxCanonDims) return false;
@@ -439,7 +506,9 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     // (8 workgroups per CU of 4-byte tiles, 4 of 2-byte tiles), so that the eight XCDs each stream
     // runs of group * 256 bytes on both sides.  Measured at 8192^2 fp32 pack: group 1 0.47, 4 0.52,
     // 16 0.65 of peak; 2-byte elements do best at 8.
-    a.group = big ? 8 : (unit == 4 || unit == 8) ? 16 : vec ? 8 : 4;
+    // 1-byte elements (256 x 256 tiles, two workgroups per CU) do best at 4: 8200^2 0.40 -> 0.47, 5000 x 7000 0.51 -> 0.57,
+    // never lower than 8 on the shapes of the walk table.
+    a.group = big ? 8 : (unit == 4 || unit == 8) ? 16 : unit == 2 ? 8 : 4;
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
     if (vec) {
         // 16-byte stores land on 16-byte boundaries when the rows of the side that is written do
@@ -462,7 +531,8 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         // power-of-two shapes from 4096^2 to 16384^2, both directions, switched on and off in turn on one GPU:
         // 2-byte elements +0.023 of peak on average (-0.01 to +0.09; four 4096^2 matrices 0.45 -> 0.54), 4-byte
         // elements +0.005 (-0.03 to +0.05), which is why only the narrow elements use it.  At other pitches the rows of a tile spread by themselves and a rotation
-        // costs up to 0.08.
+        // costs up to 0.08.  (When the packed side's rows are 4 KiB multiples as well, choose_walk replaces the blocked
+        // walk by the diagonal one and this rotation does not apply.)
         bool camped = unit <= 2;
         for (int k = 0; camped && k < a.n_inner; ++k)
             if ((a.inner_stride[k] * unit) % 8192 != 0) camped = false;
@@ -471,7 +541,10 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     const uint64_t qgroups = (a.qtiles + a.group - 1) / a.group;
     a.qgroups = (uint32_t)qgroups;
     a.rows_per_eighth = (nbatch * qgroups + 7) / 8;
-    a.ntiles = nbatch * a.cgroups * qgroups * a.group * a.group;
+    a.walk = kWalkBlocked;
+    a.xcd_ranges = 1;
+    if (vec) choose_walk(&a, unit, nbatch);
+    a.ntiles = a.walk == kWalkBlocked ? nbatch * a.cgroups * a.qgroups * a.group * a.group : nbatch * (uint64_t)a.qtiles * a.ctiles;
     if (vec) {
         const uint64_t nblocks = 8 * ((a.ntiles + 7) / 8);  // one tile per workgroup, eight XCD ranges
         const uint32_t lanes = unit == 8 ? 256 : big ? 1024 : 512;
