@@ -604,6 +604,9 @@ def release_shared():
 def wl_c5(torch, stage="quantize"):
     fp8, bucket, tensors, sizes, total, flat, q, s = _c5_setup(torch)
     nblk = (total + 1023) // 1024
+    # the fused bucket forms run with the bucket's block index unless the stage name ends in "_search"
+    index = None if stage.endswith("_search") else bucket.block_index().data_ptr()
+    stage = stage[: -len("_search")] if stage.endswith("_search") else stage
     acc = torch.zeros(total, device="cuda:0") if "dequant" in stage or stage == "flat_unpack" else None
     if stage in ("flat_pack", "quantize", "quantize_bucket"):   # these write the shared buffers: give them their own
         flat = torch.empty_like(flat) if stage == "flat_pack" else flat
@@ -619,13 +622,13 @@ def wl_c5(torch, stage="quantize"):
     elif stage == "quantize_bucket":
         nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_bucket_kernel"
         launch = prepared("mhip_fp8_quantize_bucket", q.data_ptr(), s.data_ptr(), bucket.d_ptrs.data_ptr(),
-                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, STREAM())
+                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, index, STREAM())
     elif stage == "dequant_bucket":
         nbytes, kern = 9 * total + 4 * nblk, "fp8_dequant_accumulate_bucket_kernel"
         accs = [torch.zeros(n, device="cuda:0") for n in sizes]
         aptrs = bucket.pointer_table(accs)
         launch = prepared("mhip_fp8_dequant_accumulate_bucket", aptrs.data_ptr(), q.data_ptr(), s.data_ptr(),
-                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, STREAM())
+                          bucket.d_offsets.data_ptr(), len(sizes), total, 1024, index, STREAM())
         launch.keep = accs
     elif stage == "dequant_bucket_many8":
         qs = [q] + [(q ^ (r + 1)).contiguous() for r in range(1, 8)]
@@ -636,7 +639,7 @@ def wl_c5(torch, stage="quantize"):
         from monarch_amd._lib import ptr_array
         launch = prepared("mhip_fp8_dequant_accumulate_bucket_many", aptrs.data_ptr(), ptr_array([t.data_ptr() for t in qs]),
                           ptr_array([t.data_ptr() for t in ss]), 8, bucket.d_offsets.data_ptr(), len(sizes), total, 1024,
-                          STREAM())
+                          index, STREAM())
         launch.keep = (accs, qs, ss)
     elif stage in ("dequant_many8", "dequant_many8_overwrite"):
         # 8 peers' payloads (the same codes perturbed per peer) into one accumulator in one pass
@@ -700,7 +703,8 @@ def wl_c5(torch, stage="quantize"):
                                 "sample": f"absmax / scale / clamp / to(float8_e4m3fn) over the first {ht.numel()} elements, scaled"}
         return rec
 
-    return f"c5_fp8_{stage}", nbytes, launch, cpu, kern, "bf16->f8e4m3fn"
+    return f"c5_fp8_{stage}" + ("_table_search" if index is None and "bucket" in stage else ""), nbytes, launch, cpu, kern, \
+        "bf16->f8e4m3fn"
 
 
 LAYOUT = {  # where a workload's inputs live, when that is the library's choice
@@ -742,6 +746,8 @@ WORKLOADS = {
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
     "c5_quantize_bucket": lambda t: wl_c5(t, "quantize_bucket"),
     "c5_dequant_bucket": lambda t: wl_c5(t, "dequant_bucket"),
+    "c5_quantize_bucket_search": lambda t: wl_c5(t, "quantize_bucket_search"),
+    "c5_dequant_bucket_search": lambda t: wl_c5(t, "dequant_bucket_search"),
     "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
     "c5_dequant_many8": lambda t: wl_c5(t, "dequant_many8"),
     "c5_dequant_many8_overwrite": lambda t: wl_c5(t, "dequant_many8_overwrite"),

@@ -134,9 +134,11 @@ extern "C" {
     pub fn mhip_fp8_quantize(q: *mut u8, scales: *mut f32, x_bf16: *const c_void, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate(acc: *mut f32, q: *const u8, scales: *const f32, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_many(acc: *mut f32, q: *const *const u8, scales: *const *const f32, n: u32, numel: u64, block: u32, overwrite: c_int, stream: mhip_stream_t) -> c_int;
-    pub fn mhip_fp8_quantize_bucket(q: *mut u8, scales: *mut f32, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *const *mut c_void, q: *const u8, scales: *const f32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
-    pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *const *mut c_void, q: *const *const u8, scales: *const *const f32, n: u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_quantize_bucket(q: *mut u8, scales: *mut f32, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *const *mut c_void, q: *const u8, scales: *const f32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *const *mut c_void, q: *const *const u8, scales: *const *const f32, n: u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_bucket_index_bytes(total: u64, block: u32, bytes: *mut usize) -> c_int;
+    pub fn mhip_bucket_index_build(d_index: *mut u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_device_count(count: *mut c_int) -> c_int;
     pub fn mhip_set_device(device: c_int) -> c_int;
     pub fn mhip_device_synchronize() -> c_int;

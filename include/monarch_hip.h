@@ -318,14 +318,17 @@ int mhip_fp8_dequant_accumulate_many(float* acc, const uint8_t* const* q, const 
  * mhip_flat_pack (bf16) + mhip_fp8_quantize, resp. to mhip_fp8_dequant_accumulate on a flat
  * fp32 accumulator + mhip_flat_unpack, without materialising the flat buffers.  Blocks are
  * still counted over the bucket's flat index space.  d_tensors: bf16 inputs;
- * d_acc_tensors: fp32 accumulators, updated in place. */
+ * d_acc_tensors: fp32 accumulators, updated in place.
+ * d_index is the bucket's block index (mhip_bucket_index_build) or NULL.  Without it every wavefront
+ * searches the offsets table for the tensors of its span; with it that is one load.  Results are the
+ * same bits either way. */
 int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_tensors,
                              const uint64_t* d_offsets, uint32_t ntensors, uint64_t total,
-                             uint32_t block, mhip_stream_t stream);
+                             uint32_t block, const uint32_t* d_index, mhip_stream_t stream);
 int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t* q,
                                        const float* scales, const uint64_t* d_offsets,
                                        uint32_t ntensors, uint64_t total, uint32_t block,
-                                       mhip_stream_t stream);
+                                       const uint32_t* d_index, mhip_stream_t stream);
 
 /* mhip_fp8_dequant_accumulate_bucket for n peers in one pass (q and scales: host tables of n device
  * pointers, n <= 64): bit-identical to n single-peer calls in peer order, the accumulators cross
@@ -333,7 +336,15 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
 int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const uint8_t* const* q,
                                             const float* const* scales, uint32_t n,
                                             const uint64_t* d_offsets, uint32_t ntensors, uint64_t total,
-                                            uint32_t block, mhip_stream_t stream);
+                                            uint32_t block, const uint32_t* d_index, mhip_stream_t stream);
+
+/* Block index of a bucket, a workspace of the fused forms above that depends on the offsets table
+ * only (build it once per bucket): d_index[b] = the tensor holding flat element b * block for
+ * b < ceil(total / block), and one closing entry.  *bytes = 4 * (ceil(total / block) + 1) is the
+ * device memory the caller provides.  No counterpart in the reference. */
+int mhip_bucket_index_bytes(uint64_t total, uint32_t block, size_t* bytes);
+int mhip_bucket_index_build(uint32_t* d_index, const uint64_t* d_offsets, uint32_t ntensors,
+                            uint64_t total, uint32_t block, mhip_stream_t stream);
 
 /* ====================================================================== */
 /* Runtime pass-through (the cuda-sys / nccl-sys symbols this path uses)   */

@@ -139,9 +139,11 @@ SIGNATURES = {
     "mhip_fp8_quantize": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int, _vp]),
-    "mhip_fp8_quantize_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
-    "mhip_fp8_dequant_accumulate_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
-    "mhip_fp8_dequant_accumulate_bucket_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
+    "mhip_fp8_quantize_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
+    "mhip_fp8_dequant_accumulate_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
+    "mhip_fp8_dequant_accumulate_bucket_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
+    "mhip_bucket_index_bytes": (C.c_int, [C.c_uint64, C.c_uint32, C.POINTER(C.c_size_t)]),
+    "mhip_bucket_index_build": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
     "mhip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
     "mhip_set_device": (C.c_int, [C.c_int]),
     "mhip_device_synchronize": (C.c_int, []),

@@ -19,10 +19,34 @@ namespace mhip {
 struct BucketArgs {
     char* const* tensors;     // device table of ntensors pointers
     const uint64_t* offsets;  // device table of ntensors + 1 element offsets
+    const uint32_t* index;    // block index (see bucket_index_kernel), or null: search the offsets table
     uint64_t total;           // elements in the bucket
     uint64_t nblocks;
     uint32_t ntensors;
 };
+
+// Block index of a bucket: index[b] = the tensor that holds flat element b * 1024 for b < nblocks, and
+// index[nblocks] = ntensors - 1.  Built once per bucket (the offsets do not change between steps), it replaces the
+// table search every wavefront otherwise does per span: one load instead of two dependent probe rounds.
+__global__ __launch_bounds__(kThreads) void bucket_index_kernel(uint32_t* __restrict__ index, const uint64_t* __restrict__ offsets,
+                                                                uint32_t ntensors, uint64_t nblocks) {
+    const uint64_t stride = (uint64_t)gridDim.x * kThreads;
+    for (uint64_t b = (uint64_t)blockIdx.x * kThreads + threadIdx.x; b <= nblocks; b += stride)
+        index[b] = b < nblocks ? find_tensor(offsets, 1, 0, ntensors, b * kBlock) : ntensors - 1;
+}
+
+// Tensors of the first and the last element of [begin, end), begin a block start.  With an index, *t_hi is exact
+// when it equals *t_lo and an upper bound otherwise (the tensor-by-tensor walks skip the empty segments).
+// All 64 lanes call it with the same arguments.
+__device__ __forceinline__ void span_tensors(const BucketArgs& a, uint64_t begin, uint64_t end, uint32_t* t_lo, uint32_t* t_hi) {
+    if (a.index != nullptr) {
+        const uint32_t lo = a.index[begin / kBlock];
+        *t_lo = lo;
+        *t_hi = a.offsets[lo + 1] >= end ? lo : a.index[(end + kBlock - 1) / kBlock];
+    } else {
+        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, t_lo, t_hi);
+    }
+}
 
 // Careful path for one block that straddles tensors, holds NaN / Inf, or is the short last block of
 // the bucket, whole wavefront.  [t_lo, t_hi] are the tensors of its first and last element.  The block
@@ -129,7 +153,7 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_quantize_bucket_kernel(uin
         const uint64_t span_end = span_begin + (uint64_t)kBucketBlocks * kBlock < a.total
                                       ? span_begin + (uint64_t)kBucketBlocks * kBlock : a.total;
         uint32_t t_first, t_last;
-        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, span_begin, span_end - 1, &t_first, &t_last);
+        span_tensors(a, span_begin, span_end, &t_first, &t_last);
         if (t_first != t_last || span_end - span_begin != (uint64_t)kBucketBlocks * kBlock) {  // wave-uniform, rare
             quantize_bucket_span_slow(q, scales, a.tensors, a.offsets, a.total, a.nblocks, t_first, t_last, b0, lane);
             continue;
@@ -170,7 +194,7 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_
         const uint64_t begin = b * kBlock;
         const uint64_t end = begin + kBlock < a.total ? begin + kBlock : a.total;
         uint32_t t_lo, t_hi;
-        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, &t_lo, &t_hi);
+        span_tensors(a, begin, end, &t_lo, &t_hi);
         const float s = scales[b];
         if (t_lo == t_hi && end - begin == kBlock) {
             // the whole block lies in one tensor: 4 steps of 256 elements, all loads first
@@ -229,7 +253,7 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_
         const uint64_t begin = b * kBlock;
         const uint64_t end = begin + kBlock < a.total ? begin + kBlock : a.total;
         uint32_t t_lo, t_hi;
-        wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, &t_lo, &t_hi);
+        span_tensors(a, begin, end, &t_lo, &t_hi);
         if (t_lo == t_hi && end - begin == kBlock) {
             float* dst = reinterpret_cast<float*>(a.tensors[t_lo]) + (begin - a.offsets[t_lo]);
             float v[4][4];
@@ -286,44 +310,89 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_
     }
 }
 
-}  // namespace mhip
-
-using namespace mhip;
-
-extern "C" {
-
-int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_tensors, const uint64_t* d_offsets,
-                             uint32_t ntensors, uint64_t total, uint32_t block, mhip_stream_t stream) {
-    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
-    if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
-    if (!q || !scales || !d_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
-    if ((uintptr_t)scales & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+// shared by the entry points that quantise a bucket: `index` is a device pointer or null
+static int quantize_bucket(uint8_t* q, float* scales, const void* const* d_tensors, const uint64_t* d_offsets,
+                           uint32_t ntensors, uint64_t total, const uint32_t* index, hipStream_t hs) {
     BucketArgs a{};
     a.tensors = reinterpret_cast<char* const*>(const_cast<void* const*>(reinterpret_cast<const void* const*>(d_tensors)));
     a.offsets = d_offsets;
+    a.index = index;
     a.total = total;
     a.nblocks = (total + kBlock - 1) / kBlock;
     a.ntensors = ntensors;
     const uint64_t per_wg = (kBucketThreads / 64) * kBucketBlocks;
     const uint64_t wgs = (a.nblocks + per_wg - 1) / per_wg;
     const uint64_t cap = max_workgroups(kBucketThreads);
-    hipStream_t hs = static_cast<hipStream_t>(stream);
-    DeviceGuard guard(hs);
     MHIP_LAUNCH(fp8_quantize_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0, hs, q,
                        scales, a);
     return launch_status();
 }
 
+static int build_bucket_index(uint32_t* index, const uint64_t* d_offsets, uint32_t ntensors, uint64_t total, hipStream_t hs) {
+    const uint64_t nblocks = (total + kBlock - 1) / kBlock;
+    const uint64_t wgs = (nblocks + 1 + kThreads - 1) / kThreads;
+    const uint64_t cap = max_workgroups(kThreads);
+    MHIP_LAUNCH(bucket_index_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kThreads), 0, hs, index, d_offsets, ntensors,
+                nblocks);
+    return launch_status();
+}
+
+static int check_quantize_bucket_args(const void* q, const float* scales, const void* d_tensors, const void* d_offsets,
+                                      uint32_t block) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (!q || !scales || !d_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
+    if ((uintptr_t)scales & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+    return MHIP_SUCCESS;
+}
+
+}  // namespace mhip
+
+using namespace mhip;
+
+extern "C" {
+
+int mhip_bucket_index_bytes(uint64_t total, uint32_t block, size_t* bytes) {
+    if (!bytes) return MHIP_ERR_INVALID_ARGUMENT;
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (total > (1ull << 62)) return MHIP_ERR_INVALID_ARGUMENT;
+    *bytes = (size_t)(((total + kBlock - 1) / kBlock + 1) * sizeof(uint32_t));
+    return MHIP_SUCCESS;
+}
+
+int mhip_bucket_index_build(uint32_t* d_index, const uint64_t* d_offsets, uint32_t ntensors, uint64_t total, uint32_t block,
+                            mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (ntensors == 0) return MHIP_ERR_INVALID_ARGUMENT;
+    if (!d_index || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
+    if ((uintptr_t)d_index & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    return build_bucket_index(d_index, d_offsets, ntensors, total, hs);
+}
+
+int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_tensors, const uint64_t* d_offsets,
+                             uint32_t ntensors, uint64_t total, uint32_t block, const uint32_t* d_index, mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
+    if (int rc = check_quantize_bucket_args(q, scales, d_tensors, d_offsets, block)) return rc;
+    if ((uintptr_t)d_index & 3u) return MHIP_ERR_INVALID_ARGUMENT;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    return quantize_bucket(q, scales, d_tensors, d_offsets, ntensors, total, d_index, hs);
+}
+
 int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t* q, const float* scales,
                                        const uint64_t* d_offsets, uint32_t ntensors, uint64_t total, uint32_t block,
-                                       mhip_stream_t stream) {
+                                       const uint32_t* d_index, mhip_stream_t stream) {
     if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
     if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
     if (!q || !scales || !d_acc_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
     if ((uintptr_t)scales & 3u) return MHIP_ERR_INVALID_ARGUMENT;
     BucketArgs a{};
+    if ((uintptr_t)d_index & 3u) return MHIP_ERR_INVALID_ARGUMENT;
     a.tensors = reinterpret_cast<char* const*>(d_acc_tensors);
     a.offsets = d_offsets;
+    a.index = d_index;
     a.total = total;
     a.nblocks = (total + kBlock - 1) / kBlock;
     a.ntensors = ntensors;
@@ -338,7 +407,8 @@ int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t
 
 int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const uint8_t* const* q,
                                             const float* const* scales, uint32_t n, const uint64_t* d_offsets,
-                                            uint32_t ntensors, uint64_t total, uint32_t block, mhip_stream_t stream) {
+                                            uint32_t ntensors, uint64_t total, uint32_t block, const uint32_t* d_index,
+                                            mhip_stream_t stream) {
     if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
     if (!q || !scales || n == 0) return MHIP_ERR_INVALID_ARGUMENT;
     if (n > (uint32_t)kMaxBucketPeers) return MHIP_ERR_TOO_MANY_INPUTS;
@@ -352,8 +422,10 @@ int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const ui
         p.scales[r] = scales[r];
     }
     p.n = n;
+    if ((uintptr_t)d_index & 3u) return MHIP_ERR_INVALID_ARGUMENT;
     p.b.tensors = reinterpret_cast<char* const*>(d_acc_tensors);
     p.b.offsets = d_offsets;
+    p.b.index = d_index;
     p.b.total = total;
     p.b.nblocks = (total + kBlock - 1) / kBlock;
     p.b.ntensors = ntensors;

@@ -320,3 +320,53 @@ def test_config5_full_size_properties():
     fp8.dequant_accumulate_bucket(ab, q, s)
     sync()
     assert torch.equal(torch.cat(accs), acc)
+
+
+@pytest.mark.parametrize("ntensors", [1, 2, 7, 66, 700, 4226])
+def test_block_index_forms_match_table_search(ntensors):
+    # the bucket's block index against its definition, and the fused forms with and without it, bit for bit
+    g = torch.Generator().manual_seed(1000 + ntensors)
+    if ntensors <= 7:
+        sizes = torch.randint(1, 9000, (ntensors,), generator=g).tolist()
+    else:
+        sizes = torch.randint(0, 3000 if ntensors < 1000 else 40, (ntensors,), generator=g).tolist()
+        sizes[ntensors // 3] = 5000       # whole blocks inside one tensor next to blocks that span dozens
+        sizes[0] = 0
+    total = sum(sizes)
+    offs = np.concatenate([[0], np.cumsum(sizes)])
+    big = _c5_like(total, seed=ntensors)
+    big[total // 2] = float("nan")
+    dbig = big.to(DEV)
+    dev = [dbig[offs[i]: offs[i + 1]].clone() for i in range(ntensors)]
+    bucket = fp8.FlatBucket(dev)
+    q0, s0 = fp8.quantize_bucket(bucket, indexed=False)
+    index = bucket.block_index()
+    sync()
+    nblocks = (total + 1023) // 1024
+    starts = np.arange(nblocks, dtype=np.int64) * 1024
+    want = np.searchsorted(offs, starts, side="right") - 1        # the last tensor whose offset is <= the block start
+    got = index.cpu().numpy()
+    assert got.size == nblocks + 1 and np.array_equal(got[:nblocks], want) and got[nblocks] == ntensors - 1
+    q1, s1 = fp8.quantize_bucket(bucket)                          # picks the index up now that it exists
+    sync()
+    assert torch.equal(q0, q1) and torch.equal(s0.view(torch.int32), s1.view(torch.int32))
+    wq, ws = oracle.fp8_quantize(bits(big), 1024)
+    assert np.array_equal(q1.cpu().numpy(), wq) and np.array_equal(s1.cpu().numpy(), ws)
+    qf = q1.clone()
+    qf[(qf & 0x7F) == 0x7F] = 0x11
+    rng = np.random.default_rng(ntensors)
+    init = torch.from_numpy(rng.normal(size=total).astype(np.float32)).to(DEV)
+    results = []
+    for indexed in (False, True):
+        accs = [init[offs[i]: offs[i + 1]].clone() for i in range(ntensors)]
+        ab = fp8.FlatBucket(accs)
+        fp8.dequant_accumulate_bucket(ab, qf, s1, indexed=indexed)
+        fp8.dequant_accumulate_bucket_many(ab, [qf, qf & 0xF7, qf], [s1, s1 * 0.5, s1], indexed=indexed)
+        sync()
+        results.append(torch.cat(accs))
+    assert torch.equal(results[0].view(torch.int32), results[1].view(torch.int32))
+    acc_h = init.cpu().numpy().copy()
+    hq = qf.cpu().numpy()
+    for hq_r, hs_r in ((hq, ws), (hq, ws), (hq & 0xF7, ws * np.float32(0.5)), (hq, ws)):  # clearing a bit never makes a NaN code
+        oracle.fp8_dequant_accumulate(acc_h, hq_r, hs_r, 1024)
+    assert np.array_equal(results[1].cpu().numpy().view(np.uint32), acc_h.view(np.uint32))

@@ -75,6 +75,9 @@ def test_fp8_bucket_round_trip_replays():
     q = torch.empty(total, dtype=torch.uint8, device=DEV)
     scales = torch.empty((total + 1023) // 1024, dtype=torch.float32, device=DEV)
 
+    src.block_index()   # built before the capture: the captured calls then use the indexed kernels and allocate nothing
+    dst.block_index()
+
     def pipeline():
         fp8.quantize_bucket(src, q, scales)
         fp8.dequant_accumulate_bucket(dst, q, scales)
