@@ -66,6 +66,7 @@ pub mod status {
     pub const TOO_MANY_INPUTS: i32 = 10203;
     pub const UNSUPPORTED_BLOCK: i32 = 10204;
     pub const BUFFER_TOO_SMALL: i32 = 10205;
+    pub const SCRATCH_TOO_SMALL: i32 = 10206;
     pub const MESH_DIM_LENGTH_MISMATCH: i32 = 10301;
     pub const MESH_DIM_MISSING: i32 = 10302;
 }
@@ -137,6 +138,7 @@ extern "C" {
     pub fn mhip_fp8_quantize_bucket(q: *mut u8, scales: *mut f32, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_bucket(d_acc_tensors: *const *mut c_void, q: *const u8, scales: *const f32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_bucket_many(d_acc_tensors: *const *mut c_void, q: *const *const u8, scales: *const *const f32, n: u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_fp8_quantize_bucket_static(q: *mut u8, scales: *mut f32, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_bucket_index_bytes(total: u64, block: u32, bytes: *mut usize) -> c_int;
     pub fn mhip_bucket_index_build(d_index: *mut u32, d_offsets: *const u64, ntensors: u32, total: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_device_count(count: *mut c_int) -> c_int;

@@ -61,6 +61,7 @@ enum {
     MHIP_ERR_TOO_MANY_INPUTS = 10203,
     MHIP_ERR_UNSUPPORTED_BLOCK = 10204,
     MHIP_ERR_BUFFER_TOO_SMALL = 10205,
+    MHIP_ERR_SCRATCH_TOO_SMALL = 10206,
     /* Tensor.to_mesh checks, python/monarch/common/tensor.py:426-437 */
     MHIP_ERR_MESH_DIM_LENGTH_MISMATCH = 10301,
     MHIP_ERR_MESH_DIM_MISSING = 10302
@@ -345,6 +346,18 @@ int mhip_fp8_dequant_accumulate_bucket_many(void* const* d_acc_tensors, const ui
 int mhip_bucket_index_bytes(uint64_t total, uint32_t block, size_t* bytes);
 int mhip_bucket_index_build(uint32_t* d_index, const uint64_t* d_offsets, uint32_t ntensors,
                             uint64_t total, uint32_t block, mhip_stream_t stream);
+
+/* mhip_fp8_quantize_bucket with the block index kept by the library: for callers that cannot allocate the
+ * d_index workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The index is built into a static device array of 2^20 entries (4 MiB on every GPU
+ * the library runs on) and used by the same kernel; the call allocates nothing and gives the same bits as
+ * mhip_fp8_quantize_bucket.  total > (2^20 - 1) * 1024 elements -> MHIP_ERR_SCRATCH_TOO_SMALL.  All calls on one GPU
+ * share that array: calls that overlap in time on one GPU (different streams, different threads) race and must
+ * be ordered by the caller. */
+#define MHIP_STATIC_INDEX_MAX_ELEMENTS ((((uint64_t)1 << 20) - 1) * 1024)
+int mhip_fp8_quantize_bucket_static(uint8_t* q, float* scales, const void* const* d_tensors,
+                                    const uint64_t* d_offsets, uint32_t ntensors, uint64_t total,
+                                    uint32_t block, mhip_stream_t stream);
 
 /* ====================================================================== */
 /* Runtime pass-through (the cuda-sys / nccl-sys symbols this path uses)   */

@@ -40,6 +40,7 @@ ERR_UNSUPPORTED_OP = 10202
 ERR_TOO_MANY_INPUTS = 10203
 ERR_UNSUPPORTED_BLOCK = 10204
 ERR_BUFFER_TOO_SMALL = 10205
+ERR_SCRATCH_TOO_SMALL = 10206
 ERR_MESH_DIM_LENGTH_MISMATCH = 10301
 ERR_MESH_DIM_MISSING = 10302
 NO_RANK = (1 << 64) - 1
@@ -56,7 +57,7 @@ STATUS_NAMES = {
     ERR_INPUT_SIZE_MISMATCH: "InputSizeMismatch", ERR_UNDEFINED_TENSOR: "UndefinedTensor",
     ERR_INVALID_ARGUMENT: "InvalidArgument", ERR_UNSUPPORTED_OP: "UnsupportedOp",
     ERR_TOO_MANY_INPUTS: "TooManyInputs", ERR_UNSUPPORTED_BLOCK: "UnsupportedBlock",
-    ERR_BUFFER_TOO_SMALL: "BufferTooSmall", ERR_MESH_DIM_LENGTH_MISMATCH: "MeshDimLengthMismatch",
+    ERR_BUFFER_TOO_SMALL: "BufferTooSmall", ERR_SCRATCH_TOO_SMALL: "ScratchTooSmall", ERR_MESH_DIM_LENGTH_MISMATCH: "MeshDimLengthMismatch",
     ERR_MESH_DIM_MISSING: "MeshDimMissing",
 }
 
@@ -142,6 +143,7 @@ SIGNATURES = {
     "mhip_fp8_quantize_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
     "mhip_fp8_dequant_accumulate_bucket": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
     "mhip_fp8_dequant_accumulate_bucket_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
+    "mhip_fp8_quantize_bucket_static": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
     "mhip_bucket_index_bytes": (C.c_int, [C.c_uint64, C.c_uint32, C.POINTER(C.c_size_t)]),
     "mhip_bucket_index_build": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
     "mhip_device_count": (C.c_int, [C.POINTER(C.c_int)]),

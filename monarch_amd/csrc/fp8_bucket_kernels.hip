@@ -12,6 +12,8 @@
 // the offsets table; a span inside one tensor (the common case: tensors are >= 1K
 // elements) then costs nothing extra; a block that straddles tensors is walked tensor by
 // tensor, the lanes taking consecutive elements of each segment.
+#include <mutex>
+
 #include "fp8_common.h"
 
 namespace mhip {
@@ -345,6 +347,34 @@ static int check_quantize_bucket_args(const void* q, const float* scales, const 
     return MHIP_SUCCESS;
 }
 
+// ---- block index kept by the library, for callers that cannot allocate the workspace ----
+// mhip_fp8_quantize_bucket_static builds the bucket's block index into this array instead of into caller memory.
+// Every GPU the library runs on holds its own copy (4 MiB) until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress: the device address is looked up once per device, with that device
+// current, and kernels are given that address.
+constexpr uint64_t kStaticIndexEntries = 1ull << 20;  // blocks of 1024 elements, plus the closing entry
+static __device__ __align__(256) uint32_t scratch[kStaticIndexEntries];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static uint32_t* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until looked up
+
+// Address of the current device's copy of `scratch`; the caller has made the launch device current.
+static int static_index_for_current_device(uint32_t** out) {
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return MHIP_ERR_INVALID_DEVICE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        uint32_t* ptr = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
+        if (ptr == nullptr) return MHIP_ERR_INVALID_DEVICE;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MHIP_SUCCESS;
+}
+
 }  // namespace mhip
 
 using namespace mhip;
@@ -379,6 +409,22 @@ int mhip_fp8_quantize_bucket(uint8_t* q, float* scales, const void* const* d_ten
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     return quantize_bucket(q, scales, d_tensors, d_offsets, ntensors, total, d_index, hs);
+}
+
+int mhip_fp8_quantize_bucket_static(uint8_t* q, float* scales, const void* const* d_tensors, const uint64_t* d_offsets,
+                                    uint32_t ntensors, uint64_t total, uint32_t block, mhip_stream_t stream) {
+    if (block != kBlock) return MHIP_ERR_UNSUPPORTED_BLOCK;
+    // the index needs ceil(total / 1024) + 1 entries
+    if (total > (kStaticIndexEntries - 1) * kBlock) return MHIP_ERR_SCRATCH_TOO_SMALL;
+    if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
+    if (int rc = check_quantize_bucket_args(q, scales, d_tensors, d_offsets, block)) return rc;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    DeviceGuard guard(hs);
+    uint32_t* index = nullptr;
+    if (int rc = static_index_for_current_device(&index)) return rc;
+    // every entry the quantiser reads is rewritten by this build, so nothing of an earlier call has to be cleared
+    if (int rc = build_bucket_index(index, d_offsets, ntensors, total, hs)) return rc;
+    return quantize_bucket(q, scales, d_tensors, d_offsets, ntensors, total, index, hs);
 }
 
 int mhip_fp8_dequant_accumulate_bucket(void* const* d_acc_tensors, const uint8_t* q, const float* scales,
