@@ -596,3 +596,30 @@ def test_stream_send_tensor_semantics():
         stream_send_tensor(world, 0, None, None, f)
     fr, to = Slice(offset=0, sizes=[2], strides=[1]), Slice(offset=2, sizes=[2], strides=[1])
     assert route(fr, to, 3) == (1, None)
+
+
+@pytest.mark.parametrize("walk", ["0,1,4,0", "0,1,4,1", "0,1,16,1", "0,0,8,0", "1,0", "1,1", "2,0", "2,1", "3,0", "3,1"])
+def test_every_tile_walk_of_the_transposing_kernel_moves_the_same_bytes(walk, monkeypatch):
+    # the library picks one walk per shape; every walk it can pick (and the variants the A/B sweep forces) must give the
+    # same bytes: whole and partial tiles, batches, a tile count that is no multiple of 8, pitches that are and are not
+    # multiples of 4 KiB
+    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_WALK", walk)
+    g = torch.Generator().manual_seed(sum(walk.encode()))
+    cases = [(torch.int16, (1, 256, 384, 384)), (torch.int16, (3, 200, 333, 340)), (torch.int32, (1, 192, 64, 64)),
+             (torch.int32, (2, 130, 257, 300)), (torch.uint8, (1, 512, 768, 768)), (torch.uint8, (2, 300, 515, 600)),
+             (torch.int64, (1, 96, 160, 160)), (torch.int32, (1, 1024, 2048, 2048)), (torch.int16, (1, 2048, 1024, 2048))]
+    for dtype, (b, r, c, pitch) in cases:
+        info = torch.iinfo(dtype)
+        host = torch.randint(info.min, info.max, (b, r, pitch), dtype=dtype, generator=g)
+        dev = host.to(DEV)
+        view, hview = dev[:, :, :c].transpose(1, 2), host[:, :, :c].transpose(1, 2)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.cpu(), hview.contiguous().flatten()), (walk, dtype, b, r, c, pitch)
+        back = torch.zeros_like(dev)
+        staging.unpack(back, s, out)
+        sync()
+        ref = torch.zeros_like(host)
+        ref[:, :, :c] = host[:, :, :c]
+        assert torch.equal(back.cpu(), ref), (walk, dtype, b, r, c, pitch)

@@ -54,3 +54,33 @@ def test_pack_on_one_stream_reduce_on_another():
     for s in (s1, s2):
         check(L.mhip_stream_synchronize(s))
         check(L.mhip_stream_destroy(s))
+
+
+def test_bucket_unpacks_on_a_side_stream_keep_their_pointer_tables():
+    # FlatBucket uploads a table of output pointers per set of outputs; launches on a stream that torch's allocator
+    # does not track read it asynchronously.  Several unpacks into different output sets are queued on a side stream
+    # behind a long-running kernel, more tensors are allocated and freed meanwhile, and every result must still land
+    # in its own outputs.
+    from monarch_amd import fp8
+    sizes = [4096, 1, 70000, 333, 2048, 9]
+    total = sum(sizes)
+    side = torch.cuda.Stream()
+    src = [torch.zeros(n, dtype=torch.float32, device=DEV) for n in sizes]
+    bucket = fp8.FlatBucket(src)
+    flats = [torch.full((total,), float(k + 1), device=DEV) for k in range(6)]
+    torch.cuda.synchronize()
+    out_sets = []
+    with torch.cuda.stream(side):
+        big = torch.empty(1 << 28, dtype=torch.float32, device=DEV)
+        big.normal_()                                       # keeps the side stream busy while the calls below queue up
+    for k, flat in enumerate(flats):
+        outs = [torch.empty(n, dtype=torch.float32, device=DEV) for n in sizes]
+        bucket.unpack(flat, outs, stream=side)
+        out_sets.append(outs)
+        junk = [torch.full((len(sizes),), -1, dtype=torch.int64, device=DEV) for _ in range(8)]   # table-sized allocations
+        del junk
+    side.synchronize()
+    torch.cuda.synchronize()
+    for k, outs in enumerate(out_sets):
+        for o in outs:
+            assert torch.all(o == float(k + 1)), k
