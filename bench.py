@@ -755,10 +755,24 @@ WORKLOADS = {
 }
 
 
-def sweep_transpose_walks(dtypes, reps=5, launches=30):
-    """A/B of the transposing kernel's tile walks (--sweep transpose_walks): every variant is switched in turn inside
-    one process through MONARCH_HIP_TRANSPOSE_WALK, medians of `reps` alternations of `launches` launches, three
-    rotating buffer sets.  Prints one Markdown table per element size: fraction of HBM peak per variant."""
+SWEEPS = {
+    # name -> (environment variable the library reads at every call, {column: value or None for the library's choice})
+    "transpose_walks": ("MONARCH_HIP_TRANSPOSE_WALK",
+                        {"library": None, "blocked 4": "0,1,4,0", "blocked 4 rot": "0,1,4,1", "blocked 8": "0,1,8,0",
+                         "blocked 8 rot": "0,1,8,1", "blocked 16": "0,1,16,0", "packed fastest": "1,0", "memory fastest": "2,0",
+                         "diagonal, XCD ranges": "3,1", "diagonal": "3,0"}),
+    "transpose_policies": ("MONARCH_HIP_TRANSPOSE_POLICY",
+                           {"library": None, "cached loads, write-through stores": "0", "streaming loads and stores": "1",
+                            "streaming loads only": "2", "streaming stores only": "3"}),
+}
+
+
+def sweep_transpose(which, dtypes, reps=5, launches=30):
+    """A/B of the transposing kernel's tile walks (--sweep transpose_walks) or cache policies (--sweep
+    transpose_policies): every variant is switched in turn inside one process through an environment variable the
+    library reads at every call, medians of `reps` alternations of `launches` launches, three rotating buffer sets.
+    Prints one Markdown table per element size: fraction of HBM peak per variant."""
+    envvar, variants = SWEEPS[which]
     torch, lib, _ = _load()
     from monarch_amd import Slice
     torch.cuda.set_device(0)
@@ -767,9 +781,9 @@ def sweep_transpose_walks(dtypes, reps=5, launches=30):
 
     def setenv(v):
         if v is None:
-            libc.unsetenv(b"MONARCH_HIP_TRANSPOSE_WALK")
+            libc.unsetenv(envvar.encode())
         else:
-            libc.setenv(b"MONARCH_HIP_TRANSPOSE_WALK", v.encode(), 1)
+            libc.setenv(envvar.encode(), v.encode(), 1)
 
     types = {"u8": (torch.uint8, 1), "bf16": (torch.bfloat16, 2), "f32": (torch.float32, 4), "f64": (torch.float64, 8)}
     # (batch, rows, cols, pitch): of a [batch, rows, pitch] tensor the part [:, :, :cols] is packed transposed
@@ -777,9 +791,6 @@ def sweep_transpose_walks(dtypes, reps=5, launches=30):
               (1, 8192, 16384, 16384), (1, 8192, 4096, 4096), (1, 4096, 8192, 8192), (8, 2048, 8192, 8192),
               (1, 8064, 8064, 8064), (1, 8200, 8200, 8200), (1, 8192, 8192, 8320), (1, 8192, 8192, 8256),
               (1, 6144, 6144, 6144), (1, 12288, 12288, 12288), (1, 5000, 7000, 7000)]
-    variants = {"library": None, "blocked 4": "0,1,4,0", "blocked 4 rot": "0,1,4,1", "blocked 8": "0,1,8,0",
-                "blocked 8 rot": "0,1,8,1", "blocked 16": "0,1,16,0", "packed fastest": "1,0", "memory fastest": "2,0",
-                "diagonal, XCD ranges": "3,1", "diagonal": "3,0"}
     for name in dtypes:
         dt, es = types[name]
         print(f"\n### {name} ({es}-byte elements)\n")
@@ -918,13 +929,13 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", choices=["transpose_walks"], help="print an A/B table instead of the bench line")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS), help="print an A/B table instead of the bench line")
     ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
-    if args.sweep == "transpose_walks":
-        sweep_transpose_walks(args.dtypes.split(","))
+    if args.sweep:
+        sweep_transpose(args.sweep, args.dtypes.split(","))
         return
     headline = args.workload or "c2"
     if args.all:

@@ -139,9 +139,19 @@ __device__ __forceinline__ void store8_unaligned(void* p, uint32_t a, uint32_t b
 // takes 71.6 us with these against 74.1 us with nt stores and 75.8 us with plain stores.
 // It is the wrong choice where stores are a large or ragged share (fp8 dequant-accumulate
 // into tensors: 1.68 ms vs 1.23 ms with nt), so only the reduce kernels use it.
+//
+// The store is inline assembly, so the compiler does not know that it is a store of more than 64 bits.  On gfx940 and
+// later a vector-ALU write to the data registers of such a store needs TWO wait states after it; the compiler inserts
+// them for its own stores only.  Without them the instruction scheduled right after the asm can overwrite the first
+// data register before the store has read it (seen as a stray loop counter or LDS address in the first dword of a
+// stored vector; one wait state cured the 4-byte transposing kernel and not the 1-byte one, whose next instruction
+// is the address computation of the following LDS read).  s_nop 1 is two wait states, two issue cycles per store.
+__device__ __forceinline__ void store16_writethrough_raw(void* p, const u32x4& w) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(w) : "memory");
+}
 __device__ __forceinline__ void store16_writethrough(void* p, const uint4& v) {
     const u32x4 w = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(w) : "memory");
+    store16_writethrough_raw(p, w);
 }
 __device__ __forceinline__ uint32_t load4_unaligned(const void* p) {
     return __builtin_nontemporal_load(static_cast<const u32_unaligned*>(p));

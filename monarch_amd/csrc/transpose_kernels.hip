@@ -33,7 +33,7 @@ struct TransArgs {
     uint32_t rotate;    // rotate the c-groups of each eighth of the walk against the previous one (see the host side)
     uint32_t qgroups;   // ceil(qtiles / group)
     uint64_t rows_per_eighth;  // ceil(nbatch * qgroups / 8)
-    uint32_t aligned_stores;  // every 16-byte store of this launch is 16-byte aligned
+    uint32_t aligned_stores;  // kStore*: how tile rows are written (write-through / streaming need 16-byte aligned rows)
     uint32_t group;    // tiles are walked in group x group blocks so that concurrently running workgroups
     uint32_t cgroups;  // touch neighbouring segments on BOTH sides (DRAM row locality); cgroups = ceil(ctiles/group)
     int n_inner;       // dimensions after c (decode q -> memory offset), outermost first
@@ -51,13 +51,17 @@ struct TransArgs {
 // between neighbouring workgroups matter (measured: bf16 4.4 TB/s cached vs 2.4 TB/s with nt).
 template <typename T> __device__ __forceinline__ T ldg(const T* p) { return *p; }
 template <typename T> __device__ __forceinline__ void stg(T* p, T v) { *p = v; }
-// A tile row stored to HBM.  Rows that start on 16-byte boundaries go out write-through: switched on and off in
-// turn on one GPU over eleven shapes and both directions, +0.014 of peak on average for fp32 (-0.003 to +0.029) and
-// +0.006 for bf16.  Rows that do not are written through the cache, which combines the partial lines that
-// neighbouring tiles share.
-__device__ __forceinline__ void tstore(void* p, const u32x4& v, bool write_through) {
-    if (write_through) asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+// A tile row stored to HBM: through the cache, write-through or streaming (see choose_cache_policy).
+enum : uint32_t { kStoreCached = 0, kStoreWriteThrough = 1, kStoreStreaming = 2 };
+__device__ __forceinline__ void tstore(void* p, const u32x4& v, uint32_t policy) {
+    if (policy == kStoreWriteThrough) store16_writethrough_raw(p, v);
+    else if (policy == kStoreStreaming) __builtin_nontemporal_store(v, static_cast<u32x4_unaligned*>(p));
     else *static_cast<u32x4_unaligned*>(p) = v;
+}
+// A tile row loaded from HBM; STREAM marks the lines as not worth keeping (the nt bit).
+template <bool STREAM> __device__ __forceinline__ u32x4 tload(const void* p) {
+    if constexpr (STREAM) return __builtin_nontemporal_load(static_cast<const u32x4_unaligned*>(p));
+    else return *static_cast<const u32x4_unaligned*>(p);
 }
 
 template <typename T, int TILE, bool PACK>
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(kThreads) void slice_transpose_kernel(TransArgs a) 
 // range of the blocked walk: tiles whose 256-byte rows share a cache line when rows are not
 // 256-byte aligned are then combined in one L2 instead of being written as partial lines from
 // eight of them.
-template <typename T, int THREADS, bool PACK, int ROWB = 256>
+template <typename T, int THREADS, bool PACK, int ROWB = 256, bool STREAM = false>
 __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs a) {
     constexpr int E = 16 / sizeof(T);
     constexpr int TQ = ROWB / sizeof(T), TC = TQ;
@@ -288,7 +292,7 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 #pragma unroll
             for (int p = 0; p < PASSES; ++p) {
                 const int q = r16 + ROWS * p;
-                d[p].v = *reinterpret_cast<const u32x4_unaligned*>(mem_tile + s_off[q] + v16 * E);
+                d[p].v = tload<STREAM>(mem_tile + s_off[q] + v16 * E);
             }
 #pragma unroll
             for (int p = 0; p < PASSES; ++p) {
@@ -332,8 +336,8 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 #pragma unroll
                 for (int p = 0; p < PASSES / 2; ++p) {
                     const int c = 2 * (r16 + ROWS * p);
-                    d[2 * p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)c * a.Q + v16 * E);
-                    d[2 * p + 1].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E);
+                    d[2 * p].v = tload<STREAM>(packed_tile + (uint64_t)c * a.Q + v16 * E);
+                    d[2 * p + 1].v = tload<STREAM>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E);
                 }
 #pragma unroll
                 for (int p = 0; p < PASSES / 2; ++p) {
@@ -351,7 +355,7 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
                     const int cc = cc0 + CSTEP * p;
-                    d[p].v = *reinterpret_cast<const u32x4_unaligned*>(packed_tile + (uint64_t)cc * a.Q + qv * E);
+                    d[p].v = tload<STREAM>(packed_tile + (uint64_t)cc * a.Q + qv * E);
                 }
 #pragma unroll
                 for (int p = 0; p < PASSES; ++p) {
@@ -415,6 +419,31 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
             const int q = i / TC, c = i % TC;
             if (q0 + q < a.Q && c0 + c < a.Sc) mem_tile[s_off[q] + c] = tile[at(q, c)];
         }
+    }
+}
+
+// Cache policy of a launch, from an A/B over fifteen shapes, both directions and four element sizes (fractions of the
+// HBM peak, averages over the table; "cached" = plain loads, write-through stores on aligned rows):
+//   1/2-byte elements: cached loads + streaming (nt) stores 0.664 / 0.672 against 0.607 / 0.613 cached, never more than
+//     0.02 lower and up to 0.2 higher (u8 8192^2 0.58 -> 0.77 / 0.81, bf16 6144^2 0.59 -> 0.80); streaming the loads as
+//     well helps some shapes by 0.02 and costs others 0.08, so they stay cached;
+//   4/8-byte elements: streaming loads + streaming stores 0.679 / 0.672 against 0.640 / 0.650 (fp32 8192^2 0.73 ->
+//     0.78), never more than 0.04 lower.
+// Streaming stores of rows that are not 16-byte aligned write partial lines (u8 5000 x 7000: 0.57 -> 0.42), so rows like
+// that keep going through the cache, which combines what neighbouring tiles share.
+// MONARCH_HIP_TRANSPOSE_POLICY overrides the choice (tuning aid, read at every call): 0 cached loads + write-through /
+// cached stores, 1 streaming loads + streaming stores, 2 streaming loads only, 3 streaming stores only.
+static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint32_t unit, bool stores_aligned, bool both_sides_aligned) {
+    if (unit <= 2) {
+        if (stores_aligned) a->aligned_stores = kStoreStreaming;
+    } else if (both_sides_aligned) {
+        *stream_loads = true;
+        a->aligned_stores = kStoreStreaming;
+    }
+    if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_POLICY")) {
+        const int p = std::atoi(e);
+        *stream_loads = p == 1 || p == 2;
+        a->aligned_stores = (p == 1 || p == 3) ? kStoreStreaming : stores_aligned ? kStoreWriteThrough : kStoreCached;
     }
 }
 
@@ -510,17 +539,17 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     // never lower than 8 on the shapes of the walk table.
     a.group = big ? 8 : (unit == 4 || unit == 8) ? 16 : unit == 2 ? 8 : 4;
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
+    bool stream_loads = false;
     if (vec) {
-        // 16-byte stores land on 16-byte boundaries when the rows of the side that is written do
+        // 16-byte accesses land on 16-byte boundaries when the rows of that side do
         const uint64_t e16 = 16 / unit;  // elements per vector
-        if (PACK) {
-            a.aligned_stores = ((uintptr_t)packed & 15u) == 0 && Q % e16 == 0;
-        } else {
-            bool ok = ((uintptr_t)base & 15u) == 0 && c.offset % e16 == 0 && Sc % e16 == 0;
-            for (int k = 0; ok && k < c.ndim; ++k)
-                if (k != cd && c.dims[k].stride % e16 != 0) ok = false;
-            a.aligned_stores = ok;
-        }
+        const bool packed_aligned = ((uintptr_t)packed & 15u) == 0 && Q % e16 == 0;
+        bool memory_aligned = ((uintptr_t)base & 15u) == 0 && c.offset % e16 == 0 && Sc % e16 == 0;
+        for (int k = 0; memory_aligned && k < c.ndim; ++k)
+            if (k != cd && c.dims[k].stride % e16 != 0) memory_aligned = false;
+        const bool stores_aligned = PACK ? packed_aligned : memory_aligned;
+        a.aligned_stores = stores_aligned ? kStoreWriteThrough : kStoreCached;
+        choose_cache_policy(&a, &stream_loads, unit, stores_aligned, packed_aligned && memory_aligned);
     }
     {
         // Rows that are a multiple of 8 KiB apart share at most two of the 64 positions at which HBM interleaves
@@ -551,6 +580,18 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         *rc = launch_in_pieces(nblocks, lanes, 8, [&](uint64_t wg0, uint32_t count) {
             a.wg0 = wg0;
             const dim3 grid(count);
+            if (stream_loads) {
+                switch (unit) {
+                    case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a); break;
+                    case 2: MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a); break;
+                    case 4:
+                        if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512, true>), grid, dim3(1024), 0, stream, a);
+                        else MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a);
+                        break;
+                    default: MHIP_LAUNCH((slice_transpose_vec_kernel<uint64_t, 256, PACK, 256, true>), grid, dim3(256), 0, stream, a); break;
+                }
+                return;
+            }
             switch (unit) {
                 case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
                 case 2: MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;

@@ -623,3 +623,29 @@ def test_every_tile_walk_of_the_transposing_kernel_moves_the_same_bytes(walk, mo
         ref = torch.zeros_like(host)
         ref[:, :, :c] = host[:, :, :c]
         assert torch.equal(back.cpu(), ref), (walk, dtype, b, r, c, pitch)
+
+
+@pytest.mark.parametrize("policy", ["0", "1", "2", "3"])
+def test_every_cache_policy_of_the_transposing_kernel_moves_the_same_bytes(policy, monkeypatch):
+    # cached / write-through / streaming loads and stores, forced on aligned and unaligned rows alike (the library only
+    # streams aligned rows; correctness must not depend on that)
+    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_POLICY", policy)
+    g = torch.Generator().manual_seed(40 + int(policy))
+    cases = [(torch.int32, (1, 523, 772, 777)), (torch.int16, (2, 300, 515, 600)), (torch.uint8, (1, 512, 768, 768)),
+             (torch.int64, (1, 96, 160, 160)), (torch.int32, (1, 1024, 2048, 2048)), (torch.int16, (1, 515, 260, 261))]
+    for dtype, (b, r, c, pitch) in cases:
+        info = torch.iinfo(dtype)
+        host = torch.randint(info.min, info.max, (b, r, pitch), dtype=dtype, generator=g)
+        dev = host.to(DEV)
+        view, hview = dev[:, :, :c].transpose(1, 2), host[:, :, :c].transpose(1, 2)
+        s = Slice.of_tensor(view)
+        for rep in range(3):
+            out = staging.pack(view, s)
+            sync()
+            assert torch.equal(out.cpu(), hview.contiguous().flatten()), (policy, dtype, b, r, c, pitch, rep)
+        back = torch.zeros_like(dev)
+        staging.unpack(back, s, out)
+        sync()
+        ref = torch.zeros_like(host)
+        ref[:, :, :c] = host[:, :, :c]
+        assert torch.equal(back.cpu(), ref), (policy, dtype, b, r, c, pitch)
