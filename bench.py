@@ -767,6 +767,37 @@ SWEEPS = {
 }
 
 
+_SWEEP_COMMON = """\
+Command (repository root, one GPU; under a minute):
+
+    python bench.py --sweep {which} > profiles/{file}
+
+Every cell is the fraction of the 8 TB/s HBM peak that `mhip_slice_pack` / `mhip_slice_unpack` reach on a transposing
+view (`x[:, :, :cols].transpose(1, 2)` of a `[batch, rows, pitch]` tensor; algorithmic bytes = 2 x elements x element
+size) with one variant forced through `{{envvar}}`; `library` is what the host code picks by itself.  All variants of a
+row are switched in turn inside one process on one GPU: medians of {{reps}} alternations of {{launches}} launches, 3 rotating
+buffer sets.  Matrices of 4096 x 4096 and smaller partly live in the 256 MB Infinity Cache across the three buffer sets.
+"""
+SWEEP_HEADERS = {
+    "transpose_walks": "# Transposing pack / unpack: A/B of the tile walks (MI355X)\n\n"
+    + _SWEEP_COMMON.format(which="transpose_walks", file="transpose_walk_ab.md") + """\
+`blocked g`: XCD-contiguous ranges of g x g tile blocks (`rot`: each XCD's share starts an eighth of the c-groups
+further on); `packed fastest` / `memory fastest`: plain row-major walks; `diagonal`: consecutive workgroups step one
+tile along both axes.  The selection rule (`choose_walk` in `monarch_amd/csrc/transpose_kernels.hip`): 1/2/4-byte
+elements whose row pitches are multiples of 4 KiB on both sides take the diagonal walk, everything else the blocked
+walk (block 4 for 1-byte, 8 for 2-byte, 16 for 4/8-byte elements; 8 with the 512-byte-row tile of fp32).  Every walk
+runs with the cache policy the library picks for the element size.""",
+    "transpose_policies": "# Transposing pack / unpack: A/B of the cache policies of its loads and stores (MI355X)\n\n"
+    + _SWEEP_COMMON.format(which="transpose_policies", file="transpose_cache_policy_ab.md") + """\
+`cached loads, write-through stores`: plain 128-bit loads, `global_store_dwordx4 ... sc1`; `streaming`: the `nt`
+policy bit on loads and/or stores.  The selection rule (`choose_cache_policy` in
+`monarch_amd/csrc/transpose_kernels.hip`): stores of whole aligned 16-byte vectors stream; loads stream too when both
+sides are aligned and the packed bytes reach 120 MiB (source and destination together no longer fit the 256 MiB
+Infinity Cache); everything else keeps cached loads and write-through or cached stores.  Every policy runs with the tile walk the
+library picks for the shape.""",
+}
+
+
 def sweep_transpose(which, dtypes, reps=5, launches=30):
     """A/B of the transposing kernel's tile walks (--sweep transpose_walks) or cache policies (--sweep
     transpose_policies): every variant is switched in turn inside one process through an environment variable the
@@ -790,7 +821,8 @@ def sweep_transpose(which, dtypes, reps=5, launches=30):
     shapes = [(1, 8192, 8192, 8192), (1, 4096, 4096, 4096), (4, 4096, 4096, 4096), (1, 16384, 8192, 8192),
               (1, 8192, 16384, 16384), (1, 8192, 4096, 4096), (1, 4096, 8192, 8192), (8, 2048, 8192, 8192),
               (1, 8064, 8064, 8064), (1, 8200, 8200, 8200), (1, 8192, 8192, 8320), (1, 8192, 8192, 8256),
-              (1, 6144, 6144, 6144), (1, 12288, 12288, 12288), (1, 5000, 7000, 7000)]
+              (1, 6144, 6144, 6144), (1, 12288, 12288, 12288), (1, 5000, 7000, 7000), (1, 3072, 4096, 4096)]
+    print(SWEEP_HEADERS[which].format(envvar=envvar, reps=reps, launches=launches))
     for name in dtypes:
         dt, es = types[name]
         print(f"\n### {name} ({es}-byte elements)\n")

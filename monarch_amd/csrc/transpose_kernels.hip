@@ -422,24 +422,23 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
     }
 }
 
-// Cache policy of a launch, from an A/B over fifteen shapes, both directions and four element sizes (fractions of the
-// HBM peak, averages over the table; "cached" = plain loads, write-through stores on aligned rows):
-//   1/2-byte elements: cached loads + streaming (nt) stores 0.664 / 0.672 against 0.607 / 0.613 cached, never more than
-//     0.02 lower and up to 0.2 higher (u8 8192^2 0.58 -> 0.77 / 0.81, bf16 6144^2 0.59 -> 0.80); streaming the loads as
-//     well helps some shapes by 0.02 and costs others 0.08, so they stay cached;
-//   4/8-byte elements: streaming loads + streaming stores 0.679 / 0.672 against 0.640 / 0.650 (fp32 8192^2 0.73 ->
-//     0.78), never more than 0.04 lower.
+// Cache policy of a launch, from an A/B over sixteen shapes, both directions and four element sizes (fractions of the
+// HBM peak; "cached" = plain loads, write-through stores on aligned rows; the table is
+// profiles/transpose_cache_policy_ab.md):
+//   * stores of whole aligned 16-byte vectors stream (nt) at every element size: 1/2-byte elements 0.66 / 0.67 on
+//     average against 0.61 / 0.61 cached, up to 0.2 higher (u8 8192^2 0.58 -> 0.77 / 0.81, bf16 6144^2 0.59 -> 0.80);
+//   * loads stream as well once source and destination together no longer fit the 256 MiB Infinity Cache (packed
+//     bytes >= 120 MiB): +0.01 to +0.03 there for every element size (bf16 8192^2 0.66 -> 0.68, fp32 8192^2 0.75 ->
+//     0.78), while below that size streaming loads cost up to 0.17 (bf16 6144^2 0.80 -> 0.63, fp32 4096^2 0.81 ->
+//     0.69, u8 8192^2 0.77 -> 0.66).
 // Streaming stores of rows that are not 16-byte aligned write partial lines (u8 5000 x 7000: 0.57 -> 0.42), so rows like
-// that keep going through the cache, which combines what neighbouring tiles share.
+// that keep going through the cache, which combines what neighbouring tiles share; streaming loads need both sides
+// aligned for the same reason.
 // MONARCH_HIP_TRANSPOSE_POLICY overrides the choice (tuning aid, read at every call): 0 cached loads + write-through /
 // cached stores, 1 streaming loads + streaming stores, 2 streaming loads only, 3 streaming stores only.
-static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint32_t unit, bool stores_aligned, bool both_sides_aligned) {
-    if (unit <= 2) {
-        if (stores_aligned) a->aligned_stores = kStoreStreaming;
-    } else if (both_sides_aligned) {
-        *stream_loads = true;
-        a->aligned_stores = kStoreStreaming;
-    }
+static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint64_t packed_bytes, bool stores_aligned, bool both_sides_aligned) {
+    if (stores_aligned) a->aligned_stores = kStoreStreaming;
+    if (both_sides_aligned && packed_bytes >= (120ull << 20)) *stream_loads = true;
     if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_POLICY")) {
         const int p = std::atoi(e);
         *stream_loads = p == 1 || p == 2;
@@ -447,7 +446,7 @@ static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint32_t unit,
     }
 }
 
-// Which walk a launch takes.  Measured on MI355X over fifteen shapes, both directions and four element sizes, every
+// Which walk a launch takes.  Measured on MI355X over sixteen shapes, both directions and four element sizes, every
 // variant switched in turn inside one process (the table is profiles/transpose_walk_ab.md):
 //   * when every row pitch of both sides is a multiple of 4 KiB (power-of-two matrices and the like), the rows of a
 //     tile all fall on the same few positions of HBM's address interleave, and so do the tiles of a block of the
@@ -549,7 +548,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
             if (k != cd && c.dims[k].stride % e16 != 0) memory_aligned = false;
         const bool stores_aligned = PACK ? packed_aligned : memory_aligned;
         a.aligned_stores = stores_aligned ? kStoreWriteThrough : kStoreCached;
-        choose_cache_policy(&a, &stream_loads, unit, stores_aligned, packed_aligned && memory_aligned);
+        choose_cache_policy(&a, &stream_loads, nbatch * Sc * Q * unit, stores_aligned, packed_aligned && memory_aligned);
     }
     {
         // Rows that are a multiple of 8 KiB apart share at most two of the 64 positions at which HBM interleaves
