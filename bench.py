@@ -615,7 +615,7 @@ def wl_c5(torch, stage="quantize"):
     if stage == "flat_pack":
         nbytes, kern = 4 * total, "flat_copy_kernel<pack>"
         launch = prepared("mhip_flat_pack", flat.data_ptr(), bucket.d_ptrs.data_ptr(), bucket.d_offsets.data_ptr(),
-                          len(sizes), total, 2, STREAM())
+                          len(sizes), total, 2, index, STREAM())
     elif stage == "quantize":
         nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_kernel"
         launch = prepared("mhip_fp8_quantize", q.data_ptr(), s.data_ptr(), flat.data_ptr(), total, 1024, STREAM())
@@ -660,7 +660,7 @@ def wl_c5(torch, stage="quantize"):
         ptrs = bucket.pointer_table(outs)
 
         launch = prepared("mhip_flat_unpack", ptrs.data_ptr(), acc.data_ptr(), bucket.d_offsets.data_ptr(), len(sizes),
-                          total, 4, STREAM())
+                          total, 4, index, STREAM())
 
     def cpu():
         import numpy as np
@@ -749,6 +749,8 @@ WORKLOADS = {
     "c5_quantize_bucket_search": lambda t: wl_c5(t, "quantize_bucket_search"),
     "c5_dequant_bucket_search": lambda t: wl_c5(t, "dequant_bucket_search"),
     "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
+    "c5_flat_pack_search": lambda t: wl_c5(t, "flat_pack_search"),
+    "c5_flat_unpack_search": lambda t: wl_c5(t, "flat_unpack_search"),
     "c5_dequant_many8": lambda t: wl_c5(t, "dequant_many8"),
     "c5_dequant_many8_overwrite": lambda t: wl_c5(t, "dequant_many8_overwrite"),
     "c5_dequant_bucket_many8": lambda t: wl_c5(t, "dequant_bucket_many8"),

@@ -120,8 +120,8 @@ extern "C" {
     pub fn mhip_slice_unpack(dst_base: *mut c_void, src: *const c_void, s: *const mhip_slice_t, elem_size: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_slice_pack_many(dsts: *const *mut c_void, src_base: *const c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_slice_unpack_many(dst_base: *mut c_void, srcs: *const *const c_void, views: *const mhip_slice_t, nviews: u32, elem_size: u32, stream: mhip_stream_t) -> c_int;
-    pub fn mhip_flat_pack(flat: *mut c_void, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
-    pub fn mhip_flat_unpack(d_tensors: *const *mut c_void, flat: *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_flat_pack(flat: *mut c_void, d_tensors: *const *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_flat_unpack(d_tensors: *const *mut c_void, flat: *const c_void, d_offsets: *const u64, ntensors: u32, total: u64, elem_size: u32, d_index: *const u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_reduce(out: *mut c_void, input: *const *const c_void, n: u32, numel: u64, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
     pub fn mhip_reduce_scatter(outs: *const *mut c_void, out_views: *const mhip_slice_t, n_out: u32, input: *const *const c_void, in_view: *const mhip_slice_t, in_numel: u64, n_in: u32, dtype: c_int, op: c_int, stream: mhip_stream_t) -> c_int;
     pub fn mhip_stack(out: *mut c_void, input: *const *const c_void, n: u32, numel: u64, elem_size: u32, stream: mhip_stream_t) -> c_int;

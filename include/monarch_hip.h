@@ -184,11 +184,16 @@ int mhip_slice_unpack_many(void* dst_base, const void* const* srcs, const mhip_s
  * python/tests/simulator/test_simulator.py:190-203, for ragged tensors):
  * flat[offsets[t] + j] = tensors[t][j].  d_tensors (ntensors pointers) and d_offsets
  * (ntensors+1 element offsets, offsets[0] == 0) live in DEVICE memory; total ==
- * offsets[ntensors] is passed by value so that the call needs no device read-back. */
+ * offsets[ntensors] is passed by value so that the call needs no device read-back.
+ * d_index: the bucket's block index written by mhip_bucket_index_build (below), or NULL.
+ * With it a wavefront finds its tensor with one load instead of a table search and the copy
+ * runs as single-wavefront workgroups; the bytes moved are the same either way. */
 int mhip_flat_pack(void* flat, const void* const* d_tensors, const uint64_t* d_offsets,
-                   uint32_t ntensors, uint64_t total, uint32_t elem_size, mhip_stream_t stream);
+                   uint32_t ntensors, uint64_t total, uint32_t elem_size, const uint32_t* d_index,
+                   mhip_stream_t stream);
 int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d_offsets,
-                     uint32_t ntensors, uint64_t total, uint32_t elem_size, mhip_stream_t stream);
+                     uint32_t ntensors, uint64_t total, uint32_t elem_size, const uint32_t* d_index,
+                     mhip_stream_t stream);
 
 /* ====================================================================== */
 /* Reduce: the chunks one GPU owns                                         */

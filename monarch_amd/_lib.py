@@ -124,8 +124,8 @@ SIGNATURES = {
     "mhip_slice_unpack": (C.c_int, [_vp, _vp, _slicep, C.c_uint32, _vp]),
     "mhip_slice_pack_many": (C.c_int, [_vpp, _vp, _slicep, C.c_uint32, C.c_uint32, _vp]),
     "mhip_slice_unpack_many": (C.c_int, [_vp, _vpp, _slicep, C.c_uint32, C.c_uint32, _vp]),
-    "mhip_flat_pack": (C.c_int, [_vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
-    "mhip_flat_unpack": (C.c_int, [_vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp]),
+    "mhip_flat_pack": (C.c_int, [_vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
+    "mhip_flat_unpack": (C.c_int, [_vp, _vp, _vp, C.c_uint32, C.c_uint64, C.c_uint32, _vp, _vp]),
     "mhip_reduce": (C.c_int, [_vp, _vpp, C.c_uint32, C.c_uint64, C.c_int, C.c_int, _vp]),
     "mhip_reduce_scatter": (C.c_int, [_vpp, _slicep, C.c_uint32, _vpp, _slicep, C.c_uint64, C.c_uint32,
                                       C.c_int, C.c_int, _vp]),

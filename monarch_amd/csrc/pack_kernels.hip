@@ -9,8 +9,7 @@
 //                             straddling a row boundary moves as two overlapping vectors
 //   slice_gather_kernel       runs shorter than (a few) chunks: the chunk's units are
 //                             gathered / scattered one by one
-//   contiguous_copy_kernel    one run: plain copy (contiguous_copy_shift_kernel when an end or an
-//                             address is not 16-byte aligned)
+//   contiguous_copy_kernel    one run of any alignment: rows on the destination's 1 KiB boundaries
 // (views whose memory-contiguous dimension is not the innermost one go to the LDS-tiled
 // transposing kernels instead).  The host picks the form per launch from the canonical slice.
 #include "mhip_device.h"
@@ -352,91 +351,66 @@ __global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) 
     }
 }
 
-// Plain contiguous copy of 16-byte units, both sides 16-byte aligned (a contiguous view, the
-// "transfer" of a staging buffer): one chunk per lane, non-temporal load, write-through
-// store.  For a 50/50 read/write stream this shape beats the 8-deep tile above by ~5%
-// (16.6 vs 17.4 us for 48 MiB), and single-wavefront workgroups beat larger ones (48 MiB:
-// 64 lanes 15.9-16.4 us, 128 lanes 16.7-17.1, 256 lanes 16.6-16.9, 1024 lanes 16.5).
-constexpr int kCopyThreads = 64;
-
-__global__ __launch_bounds__(kCopyThreads) void contiguous_copy_kernel(char* __restrict__ dst, const char* __restrict__ src,
-                                                                       uint64_t nchunks) {
-    const uint64_t c = (uint64_t)blockIdx.x * kCopyThreads + threadIdx.x;
-    if (c < nchunks) store16_writethrough(dst + c * 16, load16_aligned(src + c * 16));
-}
-
-// Contiguous copy between byte ranges of any alignment.  The chunk grid is aligned on the destination
-// (aligned 128-bit write-through stores); the source is read as the enclosing aligned vectors, which
-// a wavefront shifts into place (shift_rows_into_place), so neither side sees an unaligned 128-bit
-// access.  A wavefront owns ROWS consecutive 1 KiB rows.  [head, head + 16 * nvec) of the range is the
-// part whose aligned source vectors all lie inside the source range; the bytes before and after it
-// (fewer than 32 each) are copied one by one by the first workgroup.
-struct ShiftCopyArgs {
+// Contiguous copy between byte ranges of any alignment (a contiguous view, the "transfer" of a staging buffer):
+// single-wavefront workgroups, one 16-byte vector per lane, non-temporal load, write-through store.  For a 50/50
+// read/write stream this shape beats the 8-deep tile above by ~5% (16.6 vs 17.4 us for 48 MiB), and single-wavefront
+// workgroups beat larger ones (48 MiB: 64 lanes 15.9-16.4 us, 128 lanes 16.7-17.1, 256 lanes 16.6-16.9, 1024 lanes
+// 16.5; at 3 GiB 0.85 of peak against 0.75 with 256 lanes x 2 vectors).
+//
+// What a wavefront writes must be whole cache lines: a 1 KiB row that starts 16 bytes past a line boundary shares its
+// first and last line with its neighbours, which run on other XCDs (workgroup i runs on XCD i mod 8) and write the
+// line back as two partial lines (3 GiB with both ends 4 bytes past a 16-byte boundary: 0.60-0.65 of peak against
+// 0.85).  So the rows are laid on the destination's 1 KiB boundaries - the first row starts with `pad` idle lanes -
+// after a head of fewer than 16 bytes, which the first workgroup moves one by one together with the tail.
+// The source is read with unaligned 128-bit loads where it is not aligned like the destination; its rows then share
+// lines on the read side only, and each XCD takes a contiguous eighth of the rows (per_xcd != 0) so that the shared
+// lines meet in one L2 (3 GiB, source 2 bytes off: 0.65 -> 0.70; reading the enclosing aligned vectors and shifting
+// them into place instead measured the same with this shape, 0.71 / 0.70, and lower without the XCD shares).
+struct ContigArgs {
     char* dst;
     const char* src;
     uint64_t nbytes;
-    uint64_t head;   // bytes before the vector part
-    uint64_t nvec;   // 16-byte destination vectors in the vector part
-    uint64_t wg0;    // workgroups of this copy launched before this grid
+    uint64_t head;     // bytes before the first 16-byte boundary of dst
+    uint64_t nvec;     // whole 16-byte destination vectors after the head
+    uint64_t per_xcd;  // rows in each XCD's contiguous share; 0: row i is workgroup i
+    uint64_t wg0;      // workgroups of this copy launched before this grid
+    uint32_t pad;      // idle lanes at the start of row 0
 };
+constexpr int kCopyThreads = 64;
 
-template <int ROWS>
-__global__ __launch_bounds__(kPackThreads) void contiguous_copy_shift_kernel(ShiftCopyArgs a) {
-    const int lane = threadIdx.x & 63;
-    const uint64_t wave = (a.wg0 + blockIdx.x) * (kPackThreads / 64) + (threadIdx.x >> 6);
-    char* __restrict__ dst = a.dst + a.head;            // 16-byte aligned
-    const char* src = a.src + a.head;
-    const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
-    const char* __restrict__ base = src - shift;        // 16-byte aligned
-    // source vectors 0 .. nvec are readable when the source is shifted (one more than is stored), 0 .. nvec - 1 otherwise
-    const uint64_t last = shift ? a.nvec : a.nvec - 1;
-    const uint64_t row0 = wave * (ROWS * 64);
-    if (row0 < a.nvec) {
-        uint4 v[ROWS];
-#pragma unroll
-        for (int k = 0; k < ROWS; ++k) {
-            const uint64_t c = row0 + k * 64 + lane;
-            v[k] = load16_aligned(base + (c < last ? c : last) * 16);  // clamped: never predicated
-        }
-        if (shift != 0) {  // wave-uniform
-            const uint64_t ct = row0 + ROWS * 64;
-            const uint4 tail = load16_aligned(base + (ct < last ? ct : last) * 16);
-            shift_rows_into_place<ROWS>(v, tail, shift);
-        }
-#pragma unroll
-        for (int k = 0; k < ROWS; ++k) {
-            const uint64_t c = row0 + k * 64 + lane;
-            if (c < a.nvec) store16_writethrough(dst + c * 16, v[k]);
-        }
+__global__ __launch_bounds__(kCopyThreads) void contiguous_copy_kernel(ContigArgs a) {
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t row = a.per_xcd != 0 ? (wg & 7) * a.per_xcd + (wg >> 3) : wg;
+    const uint64_t c = row * kCopyThreads + threadIdx.x;  // position in the padded vector grid
+    if (c >= a.pad && c - a.pad < a.nvec) {
+        const uint64_t at = a.head + (c - a.pad) * 16;
+        store16_writethrough(a.dst + at, load16_unaligned(a.src + at));
     }
-    if (a.wg0 + blockIdx.x == 0) {
-        for (uint64_t i = threadIdx.x; i < a.head; i += kPackThreads) a.dst[i] = a.src[i];
-        for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kPackThreads) a.dst[i] = a.src[i];
+    if (wg == 0) {
+        for (uint64_t i = threadIdx.x; i < a.head; i += kCopyThreads) a.dst[i] = a.src[i];
+        for (uint64_t i = a.head + a.nvec * 16 + threadIdx.x; i < a.nbytes; i += kCopyThreads) a.dst[i] = a.src[i];
     }
 }
 
-constexpr int kShiftCopyRows = 2;
-
-// Plans and launches the copy above.  Returns false when the range is too short to have a vector part.
-static bool launch_shift_copy(char* dst, const char* src, uint64_t nbytes, hipStream_t stream, int* rc) {
-    if (nbytes < 96) return false;
-    uint64_t head = (16 - ((uintptr_t)dst & 15u)) & 15u;
-    const uint32_t shift = (uint32_t)(((uintptr_t)src + head) & 15u);
-    if (head < shift) head += 16;                       // the first aligned source vector must not start before src
-    uint64_t nvec = (nbytes - head) / 16;
-    uint64_t tail = nbytes - head - nvec * 16;
-    if (shift != 0 && tail < 16 - shift) {              // nor may the last one end after src + nbytes
-        --nvec;
-        tail += 16;
+static int launch_contiguous_copy(char* dst, const char* src, uint64_t nbytes, hipStream_t stream) {
+    ContigArgs a{};
+    a.dst = dst;
+    a.src = src;
+    a.nbytes = nbytes;
+    a.head = (16 - ((uintptr_t)dst & 15u)) & 15u;
+    if (a.head > nbytes) a.head = nbytes;
+    a.nvec = (nbytes - a.head) / 16;
+    a.pad = (uint32_t)(((uintptr_t)(dst + a.head) & 1023u) / 16);
+    uint64_t rows = (a.nvec + a.pad + kCopyThreads - 1) / kCopyThreads;
+    if (rows == 0) rows = 1;  // the byte loops of the first workgroup
+    if ((((uintptr_t)src - (uintptr_t)dst) & 127u) != 0) {
+        a.per_xcd = (rows + 7) / 8;
+        rows = a.per_xcd * 8;
     }
-    if (nvec == 0) return false;
-    ShiftCopyArgs a{dst, src, nbytes, head, nvec, 0};
-    const uint64_t per_wg = (uint64_t)(kPackThreads / 64) * kShiftCopyRows * 64;
-    *rc = launch_in_pieces((nvec + per_wg - 1) / per_wg, kPackThreads, 1, [&](uint64_t first, uint32_t count) {
-        a.wg0 = first;
-        MHIP_LAUNCH(contiguous_copy_shift_kernel<kShiftCopyRows>, dim3(count), dim3(kPackThreads), 0, stream, a);
+    return launch_in_pieces(rows, kCopyThreads, 8, [&](uint64_t wg0, uint32_t count) {
+        a.wg0 = wg0;
+        MHIP_LAUNCH(contiguous_copy_kernel, dim3(count), dim3(kCopyThreads), 0, stream, a);
     });
-    return true;
 }
 
 // ---------------- flat bucket <-> ragged tensors ----------------
@@ -451,6 +425,8 @@ struct FlatArgs {
     uint32_t shift;           // units
     uint32_t units_per_elem;
     uint64_t wg0;             // workgroups of this copy launched before this grid
+    const uint32_t* index;    // block index of the bucket (tensor of element b * 1024), or null
+    uint64_t per_xcd;         // indexed form: tiles in each XCD's contiguous share of the flat buffer
 };
 
 // Chunks per lane: 4 when gathering tensors into the flat buffer (0.74 of peak; 8 -> 0.71, 2 -> 0.69),
@@ -459,13 +435,47 @@ struct FlatArgs {
 constexpr int kFlatThreads = kThreads;
 template <bool PACK> struct FlatUnroll { static constexpr int value = PACK ? 4 : 2; };
 
-template <int U, bool PACK>
-__global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
+// With a block index (FlatArgs::index, the one mhip_bucket_index_build writes) a wavefront finds the tensor of its
+// first unit with one load instead of a table search, which makes single-wavefront workgroups of THREADS = 64 lanes
+// with one 1 KiB row each affordable: the shape in which plain copies stream best on this part (a bucket of three
+// 1 GiB tensors: 0.73-0.79 of peak with the search form, 0.85 indexed; 2 rows per wavefront 0.80, 4 rows 0.77).
+// A tile is a 1 KiB row of the flat buffer, so on the tensor side a row starts wherever the tensor's offset puts it
+// and shares its first and last cache line with the neighbouring rows.  Under the plain mapping (workgroup i runs
+// on XCD i mod 8) neighbours sit on different XCDs, every shared line is fetched into two L2s and - scattering - is
+// written back as two partial lines: 1500 ragged fp32 tensors in separate allocations unpack at 0.72 and pack at
+// 0.77, against 0.83 when every tensor is a whole number of 512 B.  The indexed form therefore gives each XCD a
+// contiguous eighth of the rows (tile = (wg mod 8) * per_xcd + wg / 8), so that neighbours meet in one L2:
+// 0.80 / 0.78 on the ragged bucket, 0.83 / 0.82 on the aligned one (plain mapping: 0.83 / 0.83).  Blocks of 2 to
+// 256 rows per XCD instead of one share each measured lower than both (0.72-0.78).
+template <int U, bool PACK, int THREADS, int UNROLL, bool INDEXED>
+__global__ __launch_bounds__(THREADS) void flat_copy_kernel(FlatArgs a) {
     constexpr int VU = 16 / U;
-    constexpr int kUnroll = FlatUnroll<PACK>::value;
+    constexpr int kFlatThreads = THREADS;
+    constexpr int kUnroll = UNROLL;
+    static_assert(!INDEXED || THREADS == 64, "the indexed form is one wavefront per workgroup");
     __shared__ uint32_t s_range[2];
-    const uint64_t block_c0 = (a.wg0 + blockIdx.x) * (kFlatThreads * kUnroll);
-    if (threadIdx.x < 64) {
+    uint32_t r_lo = 0, r_hi = 0;  // tensors of the first and the last unit of this workgroup's tile
+    uint64_t tile_id = a.wg0 + blockIdx.x;
+    if constexpr (INDEXED) tile_id = (tile_id & 7) * a.per_xcd + (tile_id >> 3);
+    const uint64_t block_c0 = tile_id * (kFlatThreads * kUnroll);
+    if (block_c0 >= a.nchunks) return;  // padding of the last XCD shares (workgroup-uniform)
+    if constexpr (INDEXED) {
+        uint64_t c_last = block_c0 + kFlatThreads * kUnroll - 1;
+        if (c_last >= a.nchunks) c_last = a.nchunks - 1;
+        const uint64_t tb_first = block_c0 * VU, tb_last = c_last * VU + VU - 1;
+        uint64_t u_first = tb_first >= a.shift ? tb_first - a.shift : 0;
+        uint64_t u_last = tb_last >= a.shift ? tb_last - a.shift : 0;
+        if (u_first >= a.total) u_first = a.total - 1;
+        if (u_last >= a.total) u_last = a.total - 1;
+        // index[b] holds the tensor of element b * 1024, which is at or before the tensor of this tile's first unit
+        uint32_t lo = a.index[(u_first / a.units_per_elem) >> 10];
+        while (lo + 1 < a.ntensors && a.offsets[lo + 1] * a.units_per_elem <= u_first) ++lo;
+        uint32_t hi = lo;
+        if (lo + 1 < a.ntensors && a.offsets[lo + 1] * a.units_per_elem <= u_last)
+            hi = wave_find_tensor(a.offsets, a.units_per_elem, lo, a.ntensors, u_last);
+        r_lo = lo;
+        r_hi = hi;
+    } else if (threadIdx.x < 64) {
         // wavefront 0 finds the tensors holding the first and the last unit this block touches
         uint64_t c_last = block_c0 + kFlatThreads * kUnroll - 1;
         if (c_last >= a.nchunks) c_last = a.nchunks - 1;
@@ -481,8 +491,12 @@ __global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
             s_range[1] = hi;
         }
     }
-    __syncthreads();
-    const uint32_t t_lo = s_range[0], t_hi = s_range[1] + 1;
+    if constexpr (!INDEXED) {
+        __syncthreads();
+        r_lo = s_range[0];
+        r_hi = s_range[1];
+    }
+    const uint32_t t_lo = r_lo, t_hi = r_hi + 1;
     const uint32_t upe = a.units_per_elem;
 
     {
@@ -490,12 +504,13 @@ __global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
         // bucket's bytes are in tensors much larger than a tile) and inside the flat buffer.
         const uint64_t tile_first = block_c0 * VU;
         const uint64_t tile_end = tile_first + (uint64_t)(kFlatThreads * kUnroll) * VU;
-        if (s_range[0] == s_range[1] && tile_first >= a.shift && tile_end - a.shift <= a.total) {
+        if (r_lo == r_hi && tile_first >= a.shift && tile_end - a.shift <= a.total) {
             if constexpr (PACK) {
                 // Gathering: the tensor side is the one that is read.  Each wavefront takes kUnroll consecutive
                 // 1 KiB rows, and when the tensor extends far enough around them it reads the enclosing
                 // aligned vectors and shifts them into place instead of issuing unaligned 128-bit loads
-                // (0.74 -> 0.77 of peak on a bucket of ragged bf16 tensors).
+                // (0.74 -> 0.77 of peak on a bucket of ragged bf16 tensors).  With one row per wavefront the
+                // extra vector per row costs more than it saves (0.78 against 0.82 with unaligned loads).
                 const int lane = threadIdx.x & 63;
                 const uint64_t row0 = (block_c0 + (uint64_t)(threadIdx.x >> 6) * (kUnroll * 64)) * VU - a.shift;  // units
                 const uint64_t t_begin = a.offsets[t_lo] * upe, t_end = a.offsets[t_lo + 1] * upe;
@@ -503,7 +518,7 @@ __global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(FlatArgs a) {
                 const char* t = a.tensors[t_lo] + (row0 - t_begin) * U;
                 const uint32_t shift = (uint32_t)((uintptr_t)t & 15u);
                 uint4 d[kUnroll];
-                if (shift != 0 && (row0 - t_begin) * U >= shift && (t_end - row0) * U >= (uint64_t)kUnroll * 1024 + 16 - shift) {
+                if (kUnroll > 1 && shift != 0 && (row0 - t_begin) * U >= shift && (t_end - row0) * U >= (uint64_t)kUnroll * 1024 + 16 - shift) {
                     const char* base = t - shift;
 #pragma unroll
                     for (int i = 0; i < kUnroll; ++i) d[i] = load16_aligned(base + i * 1024 + lane * 16);
@@ -690,28 +705,12 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             ++k;
             continue;
         }
-        if (first.ndim == 0 && unit == 16) {
-            char* strided = base + first.offset * 16;
-            char* dst = PACK ? packed[k] : strided;
-            const char* src = PACK ? strided : packed[k];
-            const uint64_t wgs = (first.total + kCopyThreads - 1) / kCopyThreads;
-            if (int rc = launch_in_pieces(wgs, kCopyThreads, 1, [&](uint64_t wg0, uint32_t count) {
-                    const uint64_t c0 = wg0 * kCopyThreads;  // chunks already launched
-                    MHIP_LAUNCH(contiguous_copy_kernel, dim3(count), dim3(kCopyThreads), 0, stream, dst + c0 * 16,
-                                       src + c0 * 16, first.total - c0);
-                }))
+        if (first.ndim == 0) {  // one run, of any alignment
+            char* strided = base + first.offset * unit;
+            if (int rc = launch_contiguous_copy(PACK ? packed[k] : strided, PACK ? strided : packed[k], first.total * unit, stream))
                 return rc;
             ++k;
             continue;
-        }
-        if (first.ndim == 0 && unit < 16) {  // one run whose ends or addresses are not 16-byte aligned
-            char* strided = base + first.offset * unit;
-            int crc = MHIP_SUCCESS;
-            if (launch_shift_copy(PACK ? packed[k] : strided, PACK ? strided : packed[k], first.total * unit, stream, &crc)) {
-                if (crc) return crc;
-                ++k;
-                continue;
-            }
         }
         {
             int trc = MHIP_SUCCESS;
@@ -794,7 +793,7 @@ static int slice_copy_entry(char* base, char* const* packed, const mhip_slice_t*
 
 template <bool PACK>
 static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d_offsets, uint32_t ntensors,
-                           uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+                           uint64_t total, uint32_t elem_size, const uint32_t* d_index, mhip_stream_t stream) {
     if (elem_size == 0) return MHIP_ERR_INVALID_ARGUMENT;
     if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
     if (!flat || !d_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
@@ -812,19 +811,35 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
     a.shift = (uint32_t)(((uintptr_t)flat & 15u) / unit);
     const uint32_t vu = 16 / unit;
     a.nchunks = (a.total + a.shift + vu - 1) / vu;
-    const uint64_t per_block = (uint64_t)kFlatThreads * FlatUnroll<PACK>::value;
-    const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
+    if (d_index != nullptr) {
+        a.index = d_index;
+        a.per_xcd = ((a.nchunks + 63) / 64 + 7) / 8;  // one 64-chunk row per workgroup, eight equal shares
+        return launch_in_pieces(a.per_xcd * 8, 64, 8, [&](uint64_t wg0, uint32_t count) {
+            a.wg0 = wg0;
+            const dim3 grid(count), block(64);
+            switch (unit) {
+                case 1: MHIP_LAUNCH((flat_copy_kernel<1, PACK, 64, 1, true>), grid, block, 0, hs, a); break;
+                case 2: MHIP_LAUNCH((flat_copy_kernel<2, PACK, 64, 1, true>), grid, block, 0, hs, a); break;
+                case 4: MHIP_LAUNCH((flat_copy_kernel<4, PACK, 64, 1, true>), grid, block, 0, hs, a); break;
+                case 8: MHIP_LAUNCH((flat_copy_kernel<8, PACK, 64, 1, true>), grid, block, 0, hs, a); break;
+                default: MHIP_LAUNCH((flat_copy_kernel<16, PACK, 64, 1, true>), grid, block, 0, hs, a); break;
+            }
+        });
+    }
+    constexpr int kUnroll = FlatUnroll<PACK>::value;
+    const uint64_t per_block = (uint64_t)kFlatThreads * kUnroll;
+    const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
     return launch_in_pieces(blocks, kFlatThreads, 1, [&](uint64_t wg0, uint32_t count) {
         a.wg0 = wg0;
         const dim3 grid(count), block(kFlatThreads);
         switch (unit) {
-            case 1: MHIP_LAUNCH((flat_copy_kernel<1, PACK>), grid, block, 0, hs, a); break;
-            case 2: MHIP_LAUNCH((flat_copy_kernel<2, PACK>), grid, block, 0, hs, a); break;
-            case 4: MHIP_LAUNCH((flat_copy_kernel<4, PACK>), grid, block, 0, hs, a); break;
-            case 8: MHIP_LAUNCH((flat_copy_kernel<8, PACK>), grid, block, 0, hs, a); break;
-            default: MHIP_LAUNCH((flat_copy_kernel<16, PACK>), grid, block, 0, hs, a); break;
+            case 1: MHIP_LAUNCH((flat_copy_kernel<1, PACK, kFlatThreads, kUnroll, false>), grid, block, 0, hs, a); break;
+            case 2: MHIP_LAUNCH((flat_copy_kernel<2, PACK, kFlatThreads, kUnroll, false>), grid, block, 0, hs, a); break;
+            case 4: MHIP_LAUNCH((flat_copy_kernel<4, PACK, kFlatThreads, kUnroll, false>), grid, block, 0, hs, a); break;
+            case 8: MHIP_LAUNCH((flat_copy_kernel<8, PACK, kFlatThreads, kUnroll, false>), grid, block, 0, hs, a); break;
+            default: MHIP_LAUNCH((flat_copy_kernel<16, PACK, kFlatThreads, kUnroll, false>), grid, block, 0, hs, a); break;
         }
     });
 }
@@ -864,18 +879,18 @@ int mhip_slice_unpack_many(void* dst_base, const void* const* srcs, const mhip_s
 }
 
 int mhip_flat_pack(void* flat, const void* const* d_tensors, const uint64_t* d_offsets, uint32_t ntensors,
-                   uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+                   uint64_t total, uint32_t elem_size, const uint32_t* d_index, mhip_stream_t stream) {
     return flat_copy_entry<true>(static_cast<char*>(flat),
                                  reinterpret_cast<char* const*>(const_cast<void* const*>(
                                      reinterpret_cast<const void* const*>(d_tensors))),
-                                 d_offsets, ntensors, total, elem_size, stream);
+                                 d_offsets, ntensors, total, elem_size, d_index, stream);
 }
 
 int mhip_flat_unpack(void* const* d_tensors, const void* flat, const uint64_t* d_offsets, uint32_t ntensors,
-                     uint64_t total, uint32_t elem_size, mhip_stream_t stream) {
+                     uint64_t total, uint32_t elem_size, const uint32_t* d_index, mhip_stream_t stream) {
     return flat_copy_entry<false>(const_cast<char*>(static_cast<const char*>(flat)),
                                   reinterpret_cast<char* const*>(d_tensors), d_offsets, ntensors, total,
-                                  elem_size, stream);
+                                  elem_size, d_index, stream);
 }
 
 }  // extern "C"

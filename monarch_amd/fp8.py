@@ -105,8 +105,8 @@ class FlatBucket:
             return None if self._index is None else self._index.data_ptr()
         return self.block_index(stream).data_ptr() if indexed else None
 
-    def pack(self, flat: torch.Tensor = None, d_ptrs: torch.Tensor = None, stream=None) -> torch.Tensor:
-        """flat[offsets[t] + j] = tensors[t][j]"""
+    def pack(self, flat: torch.Tensor = None, d_ptrs: torch.Tensor = None, stream=None, indexed: bool = None) -> torch.Tensor:
+        """flat[offsets[t] + j] = tensors[t][j]; ``indexed`` as in ``_index_ptr``."""
         if flat is None:
             flat = torch.empty(self.total, dtype=self.dtype, device=self.device)
         else:
@@ -115,7 +115,8 @@ class FlatBucket:
         if ptrs.dtype != torch.int64 or ptrs.numel() != len(self.sizes) or ptrs.device != self.device:
             raise ValueError("the pointer table must hold one int64 device pointer per tensor of the bucket")
         check(lib().mhip_flat_pack(flat.data_ptr(), ptrs.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
-                                   self.total, self.tensors[0].element_size(), _torch.stream_handle(stream)))
+                                   self.total, self.tensors[0].element_size(), self._index_ptr(indexed, stream),
+                                   _torch.stream_handle(stream)))
         return flat
 
     def _check_flat(self, flat: torch.Tensor, dtype: torch.dtype) -> None:
@@ -125,8 +126,9 @@ class FlatBucket:
         if flat.dtype != dtype or flat.numel() != self.total:
             raise ValueError(f"flat buffer must hold {self.total} elements of {dtype}, got {flat.numel()} of {flat.dtype}")
 
-    def unpack(self, flat: torch.Tensor, outs: Sequence[torch.Tensor], stream=None) -> None:
-        """outs[t][j] = flat[offsets[t] + j]; ``flat`` may have any dtype of the outs' element size."""
+    def unpack(self, flat: torch.Tensor, outs: Sequence[torch.Tensor], stream=None, indexed: bool = None) -> None:
+        """outs[t][j] = flat[offsets[t] + j]; ``flat`` may have any dtype of the outs' element size;
+        ``indexed`` as in ``_index_ptr``."""
         _torch.require_contiguous(flat)
         if flat.numel() != self.total or flat.device != self.device:
             raise ValueError(f"flat buffer must hold {self.total} elements on {self.device}")
@@ -138,7 +140,8 @@ class FlatBucket:
                 raise ValueError(f"output is on {t.device}, the bucket on {self.device}")
         ptrs = self.pointer_table(outs)
         check(lib().mhip_flat_unpack(ptrs.data_ptr(), flat.data_ptr(), self.d_offsets.data_ptr(), len(self.sizes),
-                                     self.total, flat.element_size(), _torch.stream_handle(stream)))
+                                     self.total, flat.element_size(), self._index_ptr(indexed, stream),
+                                     _torch.stream_handle(stream)))
 
 
 def quantize_bucket(bucket: FlatBucket, q: torch.Tensor = None, scales: torch.Tensor = None, stream=None,

@@ -252,19 +252,63 @@ def test_flat_pack_alignment_and_empty_tensors():
             v.copy_(t)
             dev.append(v)
         bucket = fp8.FlatBucket(dev)
-        for shift in (0, 1, 3):  # flat buffer alignment
+        for shift, indexed in ((0, False), (1, False), (3, False), (0, True), (1, True), (3, True)):  # flat buffer alignment
             fstore = torch.zeros(bucket.total + 8, dtype=dtype, device=DEV)
             flat = fstore[shift: shift + bucket.total]
-            bucket.pack(flat)
+            bucket.pack(flat, indexed=indexed)
             sync()
             want = oracle.flat_pack([bits(t) for t in tensors], bucket.offsets)
             assert np.array_equal(bits(flat), want)
             assert fstore[:shift].abs().sum() == 0 and fstore[shift + bucket.total:].abs().sum() == 0
             outs = [torch.zeros(n + 2, dtype=dtype, device=DEV)[1: 1 + n] for n in sizes]
-            bucket.unpack(flat, outs)
+            bucket.unpack(flat, outs, indexed=indexed)
             sync()
             for o, t in zip(outs, tensors):
                 assert torch.equal(o.cpu(), t)
+
+
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.bfloat16, torch.float32, torch.float64, torch.complex128])
+def test_flat_copies_with_block_index_match_table_search(dtype):
+    """The indexed form (one wavefront per 1 KiB row of the flat buffer, tensor found through the block index, each XCD
+    on a contiguous share of the rows) and the table-search form move the same bytes: rows inside one tensor, rows that
+    straddle many small or empty tensors, a bucket shorter than a row, guard elements around every destination."""
+    rng = np.random.default_rng(77)
+    es = torch.empty(0, dtype=dtype).element_size()
+    row = 1024 // es  # elements per 1 KiB row
+    for trial, sizes in enumerate((
+            [3],
+            [row - 1, 1, row, row + 1, 0, 0, 5 * row + 3],
+            rng.integers(0, 12, size=300).tolist() + [7 * row + 1] + rng.integers(0, 3 * row, size=90).tolist(),
+            np.round(np.exp(rng.uniform(np.log(2**4), np.log(2**17), size=120))).astype(np.int64).tolist() + [0, 1])):
+        host = [torch.from_numpy(rng.integers(0, 256, size=n * es, dtype=np.uint8)) for n in sizes]
+        store = [torch.zeros(n * es + 64, dtype=torch.uint8, device=DEV) for n in sizes]
+        dev = []
+        for i, (h, st) in enumerate(zip(host, store)):
+            v = st[(i % 4) * es: (i % 4) * es + h.numel()]  # staggered, only element-aligned
+            v.copy_(h)
+            dev.append(v.view(dtype))
+        bucket = fp8.FlatBucket(dev)
+        want = np.concatenate([h.numpy() for h in host])
+        for shift in (0, 1):
+            flats = []
+            for indexed in (False, True):
+                fstore = torch.full(((bucket.total + 8) * es,), 0xA5, dtype=torch.uint8, device=DEV)
+                flat = fstore[shift * es: (shift + bucket.total) * es].view(dtype)
+                bucket.pack(flat, indexed=indexed)
+                sync()
+                got = fstore.cpu().numpy()
+                assert np.array_equal(got[shift * es: (shift + bucket.total) * es], want), (trial, shift, indexed)
+                assert (got[:shift * es] == 0xA5).all() and (got[(shift + bucket.total) * es:] == 0xA5).all()
+                flats.append(flat)
+                ostore = [torch.full((n * es + 64,), 0x5A, dtype=torch.uint8, device=DEV) for n in sizes]
+                outs = [st[(1 + i % 3) * es: (1 + i % 3) * es + n * es].view(dtype) for i, (st, n) in enumerate(zip(ostore, sizes))]
+                bucket.unpack(flat, outs, indexed=indexed)
+                sync()
+                for i, (st, h, n) in enumerate(zip(ostore, host, sizes)):
+                    o = st.cpu().numpy()
+                    lo = (1 + i % 3) * es
+                    assert np.array_equal(o[lo: lo + n * es], h.numpy()), (trial, shift, indexed, i)
+                    assert (o[:lo] == 0x5A).all() and (o[lo + n * es:] == 0x5A).all(), (trial, shift, indexed, i)
 
 
 def test_config5_full_size_properties():
