@@ -89,29 +89,33 @@ def test_fuzz_slices_with_longer_rows(elem_size):
 
 
 def test_contiguous_copy_at_every_alignment():
-    # one run of bytes, every combination of source and destination alignment, lengths around the
-    # point where the copy gets a vector part (aligned stores, shifted aligned loads) plus ragged ends
+    # one run of bytes, every combination of source and destination alignment within a 16-byte vector, and
+    # destinations anywhere inside a 1 KiB row (the copy lays its rows on the destination's 1 KiB boundaries and
+    # gives each XCD an eighth of them when the source is aligned differently); lengths around a vector, a row
+    # and eight rows, plus ragged ends
     import ctypes as C
     from monarch_amd._lib import check, lib
     g = torch.Generator().manual_seed(9)
     host = torch.randint(0, 256, (80_000,), dtype=torch.uint8, generator=g)
     src_store = host.to(DEV)
     stream = torch.cuda.current_stream().cuda_stream
-    for n in (1, 15, 95, 96, 97, 111, 128, 1000, 4097, 70_001):
+    cases = [(n, so, do) for n in (1, 15, 95, 96, 97, 111, 128, 1000, 4097, 70_001) for so in (0, 1, 2, 5, 8, 15)
+             for do in (0, 1, 3, 8, 14)]
+    cases += [(n, so, do) for n in (1, 17, 1023, 1024, 1025, 8191, 8192, 8193, 9000, 66_000) for so in (0, 3, 128, 1000)
+              for do in (112, 496, 1000, 1007)]
+    for n, so, do in cases:
         s = Slice.new_row_major([n])
-        for so in (0, 1, 2, 5, 8, 15):
-            for do in (0, 1, 3, 8, 14):
-                dst_store = torch.full((n + 64,), 0xEE, dtype=torch.uint8, device=DEV)
-                check(lib().mhip_slice_pack(dst_store.data_ptr() + 16 + do, src_store.data_ptr() + so, C.byref(s.c), 1, stream))
-                back = torch.full((n + 64,), 0x11, dtype=torch.uint8, device=DEV)
-                check(lib().mhip_slice_unpack(back.data_ptr() + 16 + so, dst_store.data_ptr() + 16 + do, C.byref(s.c), 1, stream))
-                sync()
-                got = dst_store.cpu()
-                assert torch.equal(got[16 + do: 16 + do + n], host[so: so + n]), (n, so, do)
-                assert bool((got[:16 + do] == 0xEE).all()) and bool((got[16 + do + n:] == 0xEE).all()), (n, so, do)
-                gb = back.cpu()
-                assert torch.equal(gb[16 + so: 16 + so + n], host[so: so + n]), (n, so, do)
-                assert bool((gb[:16 + so] == 0x11).all()) and bool((gb[16 + so + n:] == 0x11).all()), (n, so, do)
+        dst_store = torch.full((n + 1100,), 0xEE, dtype=torch.uint8, device=DEV)
+        check(lib().mhip_slice_pack(dst_store.data_ptr() + 16 + do, src_store.data_ptr() + so, C.byref(s.c), 1, stream))
+        back = torch.full((n + 1100,), 0x11, dtype=torch.uint8, device=DEV)
+        check(lib().mhip_slice_unpack(back.data_ptr() + 16 + so, dst_store.data_ptr() + 16 + do, C.byref(s.c), 1, stream))
+        sync()
+        got = dst_store.cpu()
+        assert torch.equal(got[16 + do: 16 + do + n], host[so: so + n]), (n, so, do)
+        assert bool((got[:16 + do] == 0xEE).all()) and bool((got[16 + do + n:] == 0xEE).all()), (n, so, do)
+        gb = back.cpu()
+        assert torch.equal(gb[16 + so: 16 + so + n], host[so: so + n]), (n, so, do)
+        assert bool((gb[:16 + so] == 0x11).all()) and bool((gb[16 + so + n:] == 0x11).all()), (n, so, do)
 
 
 def test_odd_byte_alignment():
