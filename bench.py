@@ -386,9 +386,10 @@ def wl_c3(torch, unpack=False, sets=3):
     return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 
 
-def wl_c3_reshard(torch, sets=3):
+def wl_c3_reshard(torch, sets=3, one_by_one=False):
     """Configuration 3 end to end (SendTensor / to_mesh of a column-sharded weight): the 8 column blocks are packed
-    into 8 staging buffers in one launch, and each buffer is transferred into its receiver's contiguous tensor.
+    into 8 staging buffers in one launch, and the buffers are transferred into their receivers' contiguous tensors
+    in a second one (``one_by_one``: one launch per buffer, as the reference posts its work requests).
     Bytes per step: pack reads and writes 117 MB, the transfers read and write them again."""
     from monarch_amd import Slice, staging
     from monarch_amd._lib import ptr_array
@@ -410,8 +411,13 @@ def wl_c3_reshard(torch, sets=3):
     for x, area, recv in bufs:
         seq = [prepared("mhip_slice_pack_many", ptr_array([area.slot(j).data_ptr() for j in range(k)]), x.data_ptr(), arr, k, 2,
                         STREAM())]
-        seq += [prepared("mhip_buffer_transfer", recv[j].data_ptr(), area.slot(j).data_ptr(), rows * w * 2, 0, STREAM(), None)
-                for j in range(k)]
+        if one_by_one:
+            seq += [prepared("mhip_buffer_transfer", recv[j].data_ptr(), area.slot(j).data_ptr(), rows * w * 2, 0, STREAM(), None)
+                    for j in range(k)]
+        else:
+            seq.append(prepared("mhip_buffer_transfer_many", ptr_array([t.data_ptr() for t in recv]),
+                                ptr_array([area.slot(j).data_ptr() for j in range(k)]), (C.c_size_t * k)(*[rows * w * 2] * k), k, 0,
+                                STREAM(), None))
         seqs.append(seq)
 
     def launch(i):
@@ -430,7 +436,9 @@ def wl_c3_reshard(torch, sets=3):
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "1 of the 8 column blocks through the oracle's send_tensor (Slice::get walk + byte copy), scaled x8"}
 
-    return "c3_reshard_end_to_end", nbytes, launch, cpu, "slice_copy_kernel<16> + 8 x contiguous_copy_kernel", "u8"
+    if one_by_one:
+        return "c3_reshard_end_to_end_one_transfer_per_buffer", nbytes, launch, cpu, "slice_copy_kernel<16> + 8 x contiguous_copy_kernel", "u8"
+    return "c3_reshard_end_to_end", nbytes, launch, cpu, "slice_copy_kernel<16> + copy_many_kernel", "u8"
 
 
 def wl_stack(torch, scatter=False, sets=2):
@@ -471,7 +479,7 @@ def wl_stack(torch, scatter=False, sets=2):
         return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                 "sample": "full workload, 1 pass of the oracle's byte loops"}
 
-    return ("stack_scatter_bf16_8" if scatter else "stack_bf16_8"), nbytes, launch, cpu, "stack_copy_kernel", "u8"
+    return ("stack_scatter_bf16_8" if scatter else "stack_bf16_8"), nbytes, launch, cpu, "copy_many_kernel", "u8"
 
 
 def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
@@ -733,6 +741,7 @@ WORKLOADS = {
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
     "c3_reshard_e2e": wl_c3_reshard,
+    "c3_reshard_e2e_one_by_one": lambda t: wl_c3_reshard(t, one_by_one=True),
     "stack8": lambda t: wl_stack(t, False),
     "stack_scatter8": lambda t: wl_stack(t, True),
     "c4": wl_c4,

@@ -129,6 +129,7 @@ extern "C" {
     pub fn mhip_buffer_read_into(local: *const mhip_rdma_buffer_t, remote: *const mhip_rdma_buffer_t, stream: mhip_stream_t) -> c_int;
     pub fn mhip_buffer_write_from(local: *const mhip_rdma_buffer_t, remote: *const mhip_rdma_buffer_t, stream: mhip_stream_t) -> c_int;
     pub fn mhip_buffer_transfer(dst: *mut c_void, src: *const c_void, bytes: usize, max_segment_bytes: usize, stream: mhip_stream_t, segments: *mut u32) -> c_int;
+    pub fn mhip_buffer_transfer_many(dsts: *const *mut c_void, srcs: *const *const c_void, bytes: *const usize, n: u32, max_segment_bytes: usize, stream: mhip_stream_t, segments: *mut u32) -> c_int;
     pub fn mhip_send_tensor_route(from_ranks: *const mhip_slice_t, to_ranks: *const mhip_slice_t, rank: u64, from_rank: *mut u64, to_rank: *mut u64) -> c_int;
     pub fn mhip_to_mesh_from_ranks(slicing_names: *const *const c_char, slicing: *const mhip_slice_t, mesh_names: *const *const c_char, mesh_sizes: *const u64, mesh_ndim: u32, out_sizes: *mut u64, out_strides: *mut u64, out_ndim: *mut u32, broadcast_dims: *mut u32, n_broadcast: *mut u32, culprit: *mut u32) -> c_int;
     pub fn mhip_send_tensor(result: *mut c_void, result_bytes: usize, src_base: *const c_void, src_view: *const mhip_slice_t, elem_size: u32, staging: *mut c_void, stream: mhip_stream_t) -> c_int;

@@ -265,6 +265,13 @@ int mhip_buffer_write_from(const mhip_rdma_buffer_t* local, const mhip_rdma_buff
  * NULL, receives the number of requests posted. */
 int mhip_buffer_transfer(void* dst, const void* src, size_t bytes, size_t max_segment_bytes,
                          mhip_stream_t stream, uint32_t* segments);
+/* n such transfers, bytes[g] bytes from srcs[g] to dsts[g], with the requests of all of them in one launch
+ * (64 requests per launch): a message that moves several staging buffers, such as the column blocks
+ * of a reshard, pays for one launch instead of n.  The reference posts its work requests one by one
+ * (rdma_components.rs:842-858, :986-1002), so this has no single counterpart there; the bytes moved are
+ * those of n mhip_buffer_transfer calls.  Buffers must not overlap each other. */
+int mhip_buffer_transfer_many(void* const* dsts, const void* const* srcs, const size_t* bytes, uint32_t n,
+                              size_t max_segment_bytes, mhip_stream_t stream, uint32_t* segments);
 
 #define MHIP_NO_RANK UINT64_MAX
 /* WorkerActor::send_tensor's routing (monarch_tensor_worker/src/lib.rs:722-731): the i-th rank of

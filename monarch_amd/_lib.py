@@ -134,6 +134,7 @@ SIGNATURES = {
     "mhip_buffer_read_into": (C.c_int, [_bufp, _bufp, _vp]),
     "mhip_buffer_write_from": (C.c_int, [_bufp, _bufp, _vp]),
     "mhip_buffer_transfer": (C.c_int, [_vp, _vp, C.c_size_t, C.c_size_t, _vp, _u32p]),
+    "mhip_buffer_transfer_many": (C.c_int, [_vp, _vp, _vp, C.c_uint32, C.c_size_t, _vp, _vp]),
     "mhip_send_tensor_route": (C.c_int, [_slicep, _slicep, C.c_uint64, _u64p, _u64p]),
     "mhip_to_mesh_from_ranks": (C.c_int, [_cpp, _slicep, _cpp, _u64p, C.c_uint32, _u64p, _u64p, _u32p, _u32p, _u32p, _u32p]),
     "mhip_send_tensor": (C.c_int, [_vp, C.c_size_t, _vp, _slicep, C.c_uint32, _vp, _vp]),

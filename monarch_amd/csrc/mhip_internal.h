@@ -41,4 +41,9 @@ bool canonicalize(const mhip_slice_t& s, uint32_t elem_size, uint64_t align_mask
 // Same dimension list for two canonical slices (offsets may differ).
 bool same_shape(const CanonSlice& a, const CanonSlice& b);
 
+// n <= kCopyManyMax contiguous copies of nbytes[g] bytes from src[g] to dst[g] in one launch on `stream` (a
+// hipStream_t); src[g] may equal dst[g], other overlaps are not allowed.  Copies of no bytes are skipped.
+constexpr int kCopyManyMax = 64;
+int copy_many(void* const* dst, const void* const* src, const uint64_t* nbytes, uint32_t n, void* stream);
+
 }  // namespace mhip

@@ -37,6 +37,7 @@ struct PackArgs {
     uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
     uint32_t nviews;             // views handled by this launch
     uint64_t wg0;                // workgroups of this copy launched before this grid
+    uint64_t per_xcd, nwg;       // EXPERIMENT
     DimsArg dims;
 };
 
@@ -71,7 +72,11 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if (a.per_xcd != 0) {
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -188,7 +193,11 @@ template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArgs a) {
     constexpr int VU = 16 / U;
     constexpr int UN = kRaggedUnroll;
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if (a.per_xcd != 0) {
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -264,7 +273,11 @@ __global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) 
     using T = typename UnitType<U>::type;
     constexpr int VU = 16 / U;
     constexpr int UN = kGatherUnroll;
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if (a.per_xcd != 0) {
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -765,7 +778,15 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         const uint64_t per_block = (uint64_t)kPackThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
         const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
         a.nviews = nbatch;
-        if (int rc = launch_in_pieces(blocks * nbatch, kPackThreads, 1, [&](uint64_t wg0, uint32_t count) {
+        uint64_t nwg = blocks * nbatch;
+        if (const char* e = std::getenv("MONARCH_HIP_PACK_MAP")) {
+            if (std::atoi(e) == 1) {
+                a.nwg = nwg;
+                a.per_xcd = (nwg + 7) / 8;
+                nwg = a.per_xcd * 8;
+            }
+        }
+        if (int rc = launch_in_pieces(nwg, kPackThreads, 8, [&](uint64_t wg0, uint32_t count) {
                 a.wg0 = wg0;
                 launch_slice_copy<PACK>(unit, !fits32, large, form, dim3(count), stream, a);
             }))

@@ -31,6 +31,40 @@ static int transfer(void* dst, const void* src, uint64_t bytes, uint64_t max_seg
     return MHIP_SUCCESS;
 }
 
+// The same walk for n buffers at once: every request of every buffer becomes one entry of a many-copy launch
+// (kCopyManyMax entries per launch).
+static int transfer_many(void* const* dsts, const void* const* srcs, const size_t* bytes, uint32_t n, uint64_t max_segment,
+                         mhip_stream_t stream, uint32_t* segments) {
+    if (segments) *segments = 0;
+    if (n == 0) return MHIP_SUCCESS;
+    if (!dsts || !srcs || !bytes) return MHIP_ERR_INVALID_ARGUMENT;
+    if (max_segment == 0 || max_segment > kMaxSegmentBytes) max_segment = kMaxSegmentBytes;
+    for (uint32_t g = 0; g < n; ++g)
+        if (bytes[g] != 0 && (!dsts[g] || !srcs[g])) return MHIP_ERR_UNDEFINED_TENSOR;
+    void* d[kCopyManyMax];
+    const void* s[kCopyManyMax];
+    uint64_t len[kCopyManyMax];
+    uint32_t pending = 0, posted = 0;
+    for (uint32_t g = 0; g < n; ++g) {
+        for (uint64_t done = 0; done < bytes[g];) {
+            const uint64_t l = bytes[g] - done < max_segment ? bytes[g] - done : max_segment;
+            d[pending] = static_cast<char*>(dsts[g]) + done;
+            s[pending] = static_cast<const char*>(srcs[g]) + done;
+            len[pending] = l;
+            done += l;
+            ++posted;
+            if (++pending == (uint32_t)kCopyManyMax) {
+                if (int rc = copy_many(d, s, len, pending, stream)) return rc;
+                pending = 0;
+            }
+        }
+    }
+    if (pending != 0)
+        if (int rc = copy_many(d, s, len, pending, stream)) return rc;
+    if (segments) *segments = posted;
+    return MHIP_SUCCESS;
+}
+
 static inline bool bad_slice(const mhip_slice_t* s) {
     return s == nullptr || s->ndim > MHIP_MAX_DIMS || (s->ndim > 0 && (!s->sizes || !s->strides));
 }
@@ -44,6 +78,11 @@ extern "C" {
 int mhip_buffer_transfer(void* dst, const void* src, size_t bytes, size_t max_segment_bytes, mhip_stream_t stream,
                          uint32_t* segments) {
     return transfer(dst, src, bytes, max_segment_bytes, stream, segments);
+}
+
+int mhip_buffer_transfer_many(void* const* dsts, const void* const* srcs, const size_t* bytes, uint32_t n,
+                              size_t max_segment_bytes, mhip_stream_t stream, uint32_t* segments) {
+    return transfer_many(dsts, srcs, bytes, n, max_segment_bytes, stream, segments);
 }
 
 int mhip_buffer_read_into(const mhip_rdma_buffer_t* local, const mhip_rdma_buffer_t* remote, mhip_stream_t stream) {

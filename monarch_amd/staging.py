@@ -114,6 +114,19 @@ def transfer(dst_ptr: int, src_ptr: int, nbytes: int, max_segment_bytes: int = 0
     return posted.value
 
 
+def transfer_many(dst_ptrs, src_ptrs, nbytes, max_segment_bytes: int = 0, stream=None) -> int:
+    """The same for several buffers at once, the requests of all of them in one launch (64 per launch); returns
+    the number of requests posted."""
+    n = len(nbytes)
+    if len(dst_ptrs) != n or len(src_ptrs) != n:
+        raise ValueError("transfer_many needs one destination, one source and one length per buffer")
+    posted = C.c_uint32()
+    check(lib().mhip_buffer_transfer_many((C.c_void_p * n)(*dst_ptrs), (C.c_void_p * n)(*src_ptrs),
+                                          (C.c_size_t * n)(*nbytes), n, max_segment_bytes,
+                                          _torch.stream_handle(stream), C.byref(posted)))
+    return posted.value
+
+
 class RDMABuffer:
     """A registered contiguous byte range ``{addr, size}`` (rdma_components.rs:94-102).
 

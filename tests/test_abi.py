@@ -123,7 +123,7 @@ _RUST_TYPE = {
     "size_t": "usize", "size_t*": "*mut usize", "uint32_t": "u32", "uint64_t": "u64", "uint64_t*": "*mut u64",
     "uint8_t*": "*mut u8", "void*": "*mut c_void", "void* const*": "*const *mut c_void", "void**": "*mut *mut c_void",
     "const char*": "*const c_char", "const char* const*": "*const *const c_char", "uint32_t*": "*mut u32",
-    "const mhip_rdma_buffer_t*": "*const mhip_rdma_buffer_t",
+    "const mhip_rdma_buffer_t*": "*const mhip_rdma_buffer_t", "const size_t*": "*const usize",
 }
 
 

@@ -399,6 +399,34 @@ def test_rdma_buffer_transfer_in_segments():
     assert torch.all(a == 7)
 
 
+def test_transfer_of_many_buffers_in_one_launch():
+    # the requests of several buffers in one launch: ragged lengths, every alignment of source and destination,
+    # empty buffers, more requests than one launch holds (64), guard bytes around every destination
+    import ctypes as C
+    from monarch_amd._lib import lib
+    g = torch.Generator().manual_seed(12)
+    host = torch.randint(0, 256, (400_000,), dtype=torch.uint8, generator=g)
+    src = host.to(DEV)
+    for limit, lens in ((0, [1, 0, 15, 16, 17, 1023, 1024, 1025, 70_001, 33]), (4096, [100_000, 5, 0, 40_000, 4096, 4097]),
+                        (1000, [60_000, 30_000, 7]), (0, list(range(90, 190)))):
+        n = len(lens)
+        so = [(7 * j) % 19 + 1000 * j for j in range(n)]
+        do = [(5 * j) % 1031 for j in range(n)]
+        dsts = [torch.full((l + 1100,), 0xEE, dtype=torch.uint8, device=DEV) for l in lens]
+        posted = staging.transfer_many([d.data_ptr() + o for d, o in zip(dsts, do)], [src.data_ptr() + o for o in so], lens, limit)
+        sync()
+        assert posted == sum((1 if limit == 0 else -(-l // limit)) if l else 0 for l in lens)
+        for j, (d, l) in enumerate(zip(dsts, lens)):
+            got = d.cpu()
+            assert torch.equal(got[do[j]: do[j] + l], host[so[j]: so[j] + l]), (limit, j)
+            assert bool((got[:do[j]] == 0xEE).all()) and bool((got[do[j] + l:] == 0xEE).all()), (limit, j)
+    assert lib().mhip_buffer_transfer_many(None, None, None, 0, 0, None, None) == 0
+    one = (C.c_void_p * 1)(src.data_ptr())
+    null = (C.c_void_p * 1)(None)
+    assert lib().mhip_buffer_transfer_many(null, one, (C.c_size_t * 1)(8), 1, 0, None, None) == 10108  # UndefinedTensor
+    assert lib().mhip_buffer_transfer_many(null, one, (C.c_size_t * 1)(0), 1, 0, None, None) == 0
+
+
 def test_staging_buffers_are_validated_before_launch():
     x = torch.zeros(8, 8, device=DEV)
     s = Slice(offset=0, sizes=[8, 4], strides=[8, 1])
@@ -438,6 +466,12 @@ def test_config3_reshard_end_to_end():
         assert np.array_equal(bits(recv[j]).reshape(-1), want), j
     for j in range(k):
         assert torch.equal(recv[j], x[:, j * w:(j + 1) * w])
+    # the same transfers as one launch
+    recv2 = [torch.empty(rows, w, dtype=torch.bfloat16, device=DEV) for _ in range(k)]
+    assert staging.transfer_many([r.data_ptr() for r in recv2], [b.data_ptr() for b in bufs], [rows * w * 2] * k) == k
+    sync()
+    for j in range(k):
+        assert torch.equal(recv2[j], recv[j])
     back = torch.zeros_like(x)
     staging.unpack_many(back, views, [r.view(-1) for r in recv])
     sync()
