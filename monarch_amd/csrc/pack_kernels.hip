@@ -37,7 +37,7 @@ struct PackArgs {
     uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
     uint32_t nviews;             // views handled by this launch
     uint64_t wg0;                // workgroups of this copy launched before this grid
-    uint64_t per_xcd, nwg;       // EXPERIMENT
+    uint32_t pieces;             // slice_unpack_rows_kernel: 1 KiB pieces per row
     DimsArg dims;
 };
 
@@ -72,11 +72,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
-    uint64_t wg = a.wg0 + blockIdx.x;
-    if (a.per_xcd != 0) {
-        wg = (wg & 7) * a.per_xcd + (wg >> 3);
-        if (wg >= a.nwg) return;
-    }
+    const uint64_t wg = a.wg0 + blockIdx.x;
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -193,11 +189,7 @@ template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArgs a) {
     constexpr int VU = 16 / U;
     constexpr int UN = kRaggedUnroll;
-    uint64_t wg = a.wg0 + blockIdx.x;
-    if (a.per_xcd != 0) {
-        wg = (wg & 7) * a.per_xcd + (wg >> 3);
-        if (wg >= a.nwg) return;
-    }
+    const uint64_t wg = a.wg0 + blockIdx.x;
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -258,6 +250,37 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
     }
 }
 
+// Unpacking rows that are not whole 16-byte chunks, laid out for the side that is WRITTEN.  The two-vector form
+// above cuts the work on the packed side's 16-byte grid, so on the strided side every 1 KiB a wavefront writes starts
+// and ends inside a cache line that the neighbouring wavefronts (on other XCDs) write as well, and such a line goes to
+// HBM as two partial writes.  Here a workgroup takes one 1 KiB-aligned piece of one row of the strided side: whole
+// aligned vectors inside the row (unaligned loads from the packed image, whose lines are only read), the row's
+// first and last 16 bytes as unaligned vectors where its ends cut a vector, and nothing outside the row.  A row of R bytes needs at most
+// (R + 2046) / 1024 pieces whatever its address; pieces that miss the row exit at once.
+template <int U, bool WIDE, int NDIM>
+__global__ __launch_bounds__(kPackThreads) void slice_unpack_rows_kernel(PackArgs a) {
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile = wg / a.nviews;
+    const uint32_t v = (uint32_t)(wg % a.nviews);
+    const uint64_t r = tile / a.pieces;                         // row of the view, in iteration order
+    const uint32_t piece = (uint32_t)(tile - r * a.pieces);
+    uint64_t col;
+    const uint64_t loc = decode<WIDE, NDIM>(a.dims, r * a.dims.run, &col);  // first unit of the row; col == 0
+    char* __restrict__ row = a.base + (a.offset[v] + loc) * U;
+    const char* __restrict__ prow = a.packed[v] + r * a.dims.run * U;       // the row in the packed image
+    const int64_t run_bytes = (int64_t)(a.dims.run * U);
+    const int64_t lead = (int64_t)((uintptr_t)row & 1023u);                 // the row starts `lead` bytes into piece 0
+    const int64_t at = (int64_t)piece * 1024 + (int64_t)threadIdx.x * 16 - lead;  // this lane's vector, relative to the row
+    if (at >= 0 && at + 16 <= run_bytes) {
+        store16_aligned(row + at, load16_unaligned(prow + at));
+    } else if (at + 16 > 0 && at < run_bytes) {
+        // a vector that the row's start or end cuts: the row's first or last 16 bytes instead, as one unaligned
+        // vector that stays inside the row; where it overlaps the neighbouring lane's vector both write the same bytes
+        const int64_t o = at < 0 ? 0 : run_bytes - 16;
+        store16_unaligned(row + o, load16_unaligned(prow + o));
+    }
+}
+
 // Views whose contiguous runs are shorter than a chunk (element-strided selections such as
 // x[:, ::2], rows of a few bytes): a lane still owns whole 16-byte chunks of the packed side,
 // which it moves with one aligned 128-bit access, and gathers (pack) or scatters (unpack) the
@@ -273,11 +296,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) 
     using T = typename UnitType<U>::type;
     constexpr int VU = 16 / U;
     constexpr int UN = kGatherUnroll;
-    uint64_t wg = a.wg0 + blockIdx.x;
-    if (a.per_xcd != 0) {
-        wg = (wg & 7) * a.per_xcd + (wg >> 3);
-        if (wg >= a.nwg) return;
-    }
+    const uint64_t wg = a.wg0 + blockIdx.x;
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -621,7 +640,7 @@ __global__ __launch_bounds__(THREADS) void flat_copy_kernel(FlatArgs a) {
 
 // ---------------- host side ----------------
 
-enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns };
+enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns, kUnpackRows };
 
 template <int U, bool PACK, int UNROLL>
 static void launch_whole_chunks_u(bool wide, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
@@ -657,6 +676,20 @@ static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, 
                 case 1: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
                 case 2: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
                 default: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
+            }
+            return;
+        }
+        if (form == kUnpackRows) {
+            if constexpr (!PACK) {
+                if (wide) {
+                    MHIP_LAUNCH((slice_unpack_rows_kernel<U, true, -1>), grid, block, 0, stream, a);
+                    return;
+                }
+                switch (ndim) {
+                    case 1: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, 1>), grid, block, 0, stream, a); break;
+                    case 2: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, 2>), grid, block, 0, stream, a); break;
+                    default: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, -1>), grid, block, 0, stream, a); break;
+                }
             }
             return;
         }
@@ -774,19 +807,22 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             if (first.run < gather_below && first.total >= 2 * vu) form = kShortRuns;
             else if (first.run >= vu) form = kRaggedRows;
         }
+        uint64_t row_pieces = 0;
+        // Unpacking ragged rows of 2 KiB and more in pieces aligned on the written side: bf16 rows of 1790 0.52 -> 0.59 of
+        // peak, of 1790 starting at column 3 0.49 -> 0.55, fp32 rows of 1791 0.59 -> 0.61.  Not for 1-byte units at odd
+        // pitches (0.62 -> 0.51: there the loads would be the byte-misaligned side, which costs more than such stores) nor
+        // for rows around 1 KiB, where half the pieces are nearly empty (fp32 rows of 255: 0.41 -> 0.36).
+        if (!PACK && form == kRaggedRows && unit >= 2 && first.run * unit >= 2048) {
+            form = kUnpackRows;
+            row_pieces = (first.run * unit + 2046) / 1024;
+            a.pieces = (uint32_t)row_pieces;
+        }
         const bool large = a.nchunks >= kLargeCopyChunks;
         const uint64_t per_block = (uint64_t)kPackThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
-        const uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
+        uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
+        if (form == kUnpackRows) blocks = (first.total / first.run) * row_pieces;  // one workgroup per piece of every row
         a.nviews = nbatch;
-        uint64_t nwg = blocks * nbatch;
-        if (const char* e = std::getenv("MONARCH_HIP_PACK_MAP")) {
-            if (std::atoi(e) == 1) {
-                a.nwg = nwg;
-                a.per_xcd = (nwg + 7) / 8;
-                nwg = a.per_xcd * 8;
-            }
-        }
-        if (int rc = launch_in_pieces(nwg, kPackThreads, 8, [&](uint64_t wg0, uint32_t count) {
+        if (int rc = launch_in_pieces(blocks * nbatch, kPackThreads, 1, [&](uint64_t wg0, uint32_t count) {
                 a.wg0 = wg0;
                 launch_slice_copy<PACK>(unit, !fits32, large, form, dim3(count), stream, a);
             }))

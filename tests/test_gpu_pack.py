@@ -138,6 +138,43 @@ def test_rows_that_are_not_whole_chunks(elem_size):
             _roundtrip(s, elem_size, seed=i, misalign=(i % 3) * elem_size, dst_misalign=dst_misalign)
 
 
+@pytest.mark.parametrize("elem_size", [2, 4, 8, 6])
+def test_unpack_of_long_ragged_rows_in_pieces_of_the_written_side(elem_size):
+    # rows of 2 KiB and more that are not whole 16-byte chunks are unpacked in 1 KiB-aligned pieces of the strided
+    # side: rows that start anywhere inside a piece, rows of exactly 2 KiB, three and four dimensions, shifted staging
+    cases = [Slice(offset=3, sizes=[5, 40, 1027], strides=[46200, 1100, 1]), Slice(offset=0, sizes=[64, 1025], strides=[1031, 1]),
+             Slice(offset=509, sizes=[31, 2049], strides=[2051, 1]), Slice(offset=1, sizes=[2, 3, 5, 1301], strides=[33600, 8400, 1400, 1]),
+             Slice(offset=7, sizes=[3, 9001], strides=[9002, 1])]
+    for i, s in enumerate(cases):
+        for dst_misalign in (0, elem_size, 7 * elem_size):
+            _roundtrip(s, elem_size, seed=20 + i, misalign=(i % 4) * elem_size, dst_misalign=dst_misalign)
+    # several views of one tensor in one launch
+    g = torch.Generator().manual_seed(21)
+    nbytes = elem_size
+    x = torch.randint(0, 256, (40, 5000 * nbytes), dtype=torch.uint8, generator=g)
+    dev = x.to(DEV)
+    views = [Slice(offset=k * 1203 + 1, sizes=[40, 1201], strides=[5000, 1]) for k in range(4)]
+    outs = [torch.empty(40 * 1201 * nbytes + 3, dtype=torch.uint8, device=DEV)[3:] for _ in views]
+    import ctypes as C
+    from monarch_amd._lib import check, lib, ptr_array
+    from monarch_amd.ndslice import slice_array
+    arr = slice_array(views)
+    stream = torch.cuda.current_stream().cuda_stream
+    check(lib().mhip_slice_pack_many(ptr_array([o.data_ptr() for o in outs]), dev.data_ptr(), arr, len(views), nbytes, stream))
+    back = torch.full_like(dev, 0x3C)
+    check(lib().mhip_slice_unpack_many(back.data_ptr(), ptr_array([o.data_ptr() for o in outs]), arr, len(views), nbytes, stream))
+    sync()
+    want = torch.full_like(x, 0x3C)
+    for v in views:
+        want[:, (v.offset) * nbytes: (v.offset + 1201) * nbytes] = x[:, v.offset * nbytes: (v.offset + 1201) * nbytes]
+    assert torch.equal(back.cpu(), want)
+
+
+def test_wide_index_unpack_of_long_ragged_rows():
+    # more than 2^31 two-byte units in rows of 32767 at a pitch of 32769: 64-bit decode in the piecewise unpack
+    _check_large_view(torch.int16, [65600, 32767], [32769, 1], offset=1)
+
+
 @pytest.mark.parametrize("elem_size", [1, 2, 4, 8, 6])
 def test_runs_shorter_than_a_chunk(elem_size):
     # element-strided selections and rows of a few bytes: packed chunks are gathered / scattered unit by
