@@ -222,6 +222,32 @@ int main(void) {
                 fprintf(stderr, "stack mismatch in member %d\n", g);
                 return 1;
             }
+        /* the eight members back out of the stack in one launch: 8 transfers of ragged length */
+        {
+            void* back[G];
+            const void* from[G];
+            size_t len[G];
+            for (int g = 0; g < G; ++g) {
+                CHECK(mhip_malloc(&back[g], M * sizeof(uint16_t)));
+                CHECK(mhip_memset(back[g], 0, M * sizeof(uint16_t), stream));
+                from[g] = (const char*)dstack + (size_t)g * M * sizeof(uint16_t);
+                len[g] = M * sizeof(uint16_t) - 3 * (size_t)g;
+            }
+            uint32_t posted = 0;
+            CHECK(mhip_buffer_transfer_many(back, from, len, G, 0, stream, &posted));
+            for (int g = 0; g < G; ++g) {
+                CHECK(mhip_memcpy_dtoh(out, back[g], M * sizeof(uint16_t), stream));
+                CHECK(mhip_stream_synchronize(stream));
+                const unsigned char* o = (const unsigned char*)out;
+                int tail_ok = 1;  /* the 3 g bytes after a buffer's length keep their zeros */
+                for (size_t i = len[g]; i < M * sizeof(uint16_t); ++i) tail_ok = tail_ok && o[i] == 0;
+                if (posted != G || memcmp(o, h[g], len[g]) != 0 || !tail_ok) {
+                    fprintf(stderr, "transfer of many buffers failed at buffer %d (%u requests)\n", g, posted);
+                    return 1;
+                }
+                CHECK(mhip_free(back[g]));
+            }
+        }
         /* columns [64, 192) of the [1024, 256] f32 matrix at the start of x, sent as a [1024, 128] tensor */
         const uint64_t csizes[2] = {1024, 128}, cstrides[2] = {256, 1};
         const mhip_slice_t col = {64, 2, csizes, cstrides};
