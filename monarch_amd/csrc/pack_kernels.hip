@@ -38,6 +38,8 @@ struct PackArgs {
     uint32_t nviews;             // views handled by this launch
     uint64_t wg0;                // workgroups of this copy launched before this grid
     uint32_t pieces;             // slice_unpack_rows_kernel: 1 KiB pieces per row
+    uint64_t per_xcd;            // packs of rows that are not whole cache lines: workgroups in each XCD's contiguous
+    uint64_t nwg;                //   share of the nwg workgroups (0: workgroup i takes tile i)
     DimsArg dims;
 };
 
@@ -72,7 +74,13 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     // The view index is the fastest-varying part of the workgroup id, so that workgroups
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if constexpr (PACK) {
+        if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
+            wg = (wg & 7) * a.per_xcd + (wg >> 3);
+            if (wg >= a.nwg) return;
+        }
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
@@ -739,6 +747,16 @@ static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint3
     return MHIP_SUCCESS;
 }
 
+// A pack of one view reads rows of the strided side in 1 KiB pieces cut on the packed side's grid.  When the rows are
+// not whole cache lines (a column block that starts 16 bytes into a line, a pitch that is not a multiple of 128 bytes),
+// nearly every piece starts and ends inside a line that the neighbouring pieces read as well - on other XCDs under the
+// plain mapping (workgroup i runs on XCD i mod 8), so the line crosses HBM twice.  Giving each XCD a contiguous eighth
+// of the pieces lets the neighbours meet in one L2: bf16 [16384, 14336] columns 8:1800 0.68 -> 0.72 of peak, columns
+// 0:1784 0.69 -> 0.73, pitch 14335 0.68 -> 0.73, fp32 rows of 1024 at pitch 8191 0.70 -> 0.75.  Rows of whole lines
+// measure the same either way or better (64 of 256 fp32 columns 0.57 -> 0.63; bf16 columns 0:1792 0.746 both ways), so
+// every single-view pack of whole chunks takes the shares.  The gathering form does not (bf16 rows of 1790: 0.69 -> 0.59,
+// though fp32 rows of 255 gain 0.03), nor the two-vector form (fp32 rows of 1791: 0.71 -> 0.70), nor unpacks, where
+// shares help some shapes (+0.04) and cost others (-0.07).
 template <bool PACK>
 static int copy_views(char* base, char* const* packed, const mhip_slice_t* views, uint32_t nviews,
                       uint32_t elem_size, hipStream_t stream) {
@@ -822,7 +840,13 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
         if (form == kUnpackRows) blocks = (first.total / first.run) * row_pieces;  // one workgroup per piece of every row
         a.nviews = nbatch;
-        if (int rc = launch_in_pieces(blocks * nbatch, kPackThreads, 1, [&](uint64_t wg0, uint32_t count) {
+        uint64_t nwg = blocks * nbatch;
+        if (PACK && nbatch == 1 && form == kWholeChunks) {  // see the note above copy_views
+            a.nwg = nwg;
+            a.per_xcd = (nwg + 7) / 8;
+            nwg = a.per_xcd * 8;
+        }
+        if (int rc = launch_in_pieces(nwg, kPackThreads, 8, [&](uint64_t wg0, uint32_t count) {
                 a.wg0 = wg0;
                 launch_slice_copy<PACK>(unit, !fits32, large, form, dim3(count), stream, a);
             }))
