@@ -754,7 +754,8 @@ static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint3
 // of the pieces lets the neighbours meet in one L2: bf16 [16384, 14336] columns 8:1800 0.68 -> 0.72 of peak, columns
 // 0:1784 0.69 -> 0.73, pitch 14335 0.68 -> 0.73, fp32 rows of 1024 at pitch 8191 0.70 -> 0.75.  Rows of whole lines
 // measure the same either way or better (64 of 256 fp32 columns 0.57 -> 0.63; bf16 columns 0:1792 0.746 both ways), so
-// every single-view pack of whole chunks takes the shares.  The gathering form does not (bf16 rows of 1790: 0.69 -> 0.59,
+// every single-view pack of whole chunks takes the shares (the eight column blocks of one tensor in one launch, where
+// the view index already pins each view to one XCD, lose with them: 0.78 -> 0.68).  The gathering form does not (bf16 rows of 1790: 0.69 -> 0.59,
 // though fp32 rows of 255 gain 0.03), nor the two-vector form (fp32 rows of 1791: 0.71 -> 0.70), nor unpacks, where
 // shares help some shapes (+0.04) and cost others (-0.07).
 template <bool PACK>
