@@ -883,6 +883,8 @@ SUMMARY = {
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
     "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
+    # configuration 1 (1 MiB views): launch-bound, reported as time per call
+    "c1_pack": None, "c1_unpack": None, "c1_reduce": None, "c1_pipeline": None, "c1_pipeline_fused": None,
 }
 
 
@@ -932,7 +934,7 @@ def run(workload: str, steps: int, warmup: int, cpu_baseline: bool, summary: boo
         # sets), fewer launches; the CPU legs here are the short ones (the headline's own leg runs above)
         import gc
         k_steps, k_warm = max(5, min(steps, 60)), max(2, min(warmup, 10))
-        cpu_legs = ("c2p_pack", "c3_pack", "c3_reshard_e2e", "c4", "c5_quantize", "c5_dequant", "stack8")
+        cpu_legs = ("c2p_pack", "c3_pack", "c3_reshard_e2e", "c4", "c5_quantize", "c5_dequant", "stack8", "c1_pack", "c1_reduce")
 
         def entry(w, mm, with_cpu):
             ach = mm["nbytes"] / (mm["kernel_ms"] * 1e-3) / 1e9
