@@ -294,7 +294,8 @@ def wl_c2(torch, in_place=False, sets=3, separate=False):
                 "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                               "sample": "one pass of torch.stack(xs).float().sum(0)/8 -> bf16"}}
 
-    name = "c2_bf16_bucket_reduce_avg8" + ("_inplace" if in_place else "") + ("_separate_allocations" if separate else "")
+    name = ("c2_bf16_bucket_reduce_avg8" + ("_inplace" if in_place else "") + ("_separate_allocations" if separate else "")
+            + (f"_{sets}_buffer_sets" if sets != 3 else ""))
     return name, nbytes, launch, cpu, "reduce_kernel<bf16,8,avg>", "bf16"
 
 
@@ -576,7 +577,7 @@ def wl_c4(torch, sets=2, slots=False):
                 "torch_cpu": {"value": nbytes / dt_torch / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
                               "sample": "one pass of x.sum(1) and 8 .contiguous() column slices on the full tensor"}}
 
-    name = "c4_mesh_dim_reduce_scatter_f32" + ("_staging_slots" if slots else "")
+    name = "c4_mesh_dim_reduce_scatter_f32" + ("_staging_slots" if slots else "") + (f"_{sets}_buffer_sets" if sets != 2 else "")
     return name, nbytes, launch, cpu, "reduce_scatter_kernel<f32,vec>", "f32"
 
 
@@ -719,6 +720,8 @@ LAYOUT = {  # where a workload's inputs live, when that is the library's choice
     "c2": "8 slots of one staging area, pitch mhip_staging_slot_pitch(48 MiB) = 48 MiB + 8 KiB",
     "c2_inplace": "8 slots of one staging area, pitch 48 MiB + 8 KiB; output = slot 0",
     "c2_separate": "8 separate torch allocations",
+    "c2_cold": "as c2, rotating over 8 buffer sets (3.6 GB)",
+    "c4_cold": "as c4, rotating over 5 buffer sets (3 GB)",
     "c2_inplace_separate": "8 separate torch allocations; output = input 0",
     "c4": "one dense [2,8,2048,4096] tensor (slab pitch 32 MiB)",
     "c4_slots": "16 slots of one staging area, pitch 32 MiB + 8 KiB",
@@ -735,6 +738,10 @@ WORKLOADS = {
     "c2": lambda t: wl_c2(t, False),
     "c2_inplace": lambda t: wl_c2(t, True),
     "c2_separate": lambda t: wl_c2(t, False, separate=True),
+    # the same launches rotated over 3.6 GB (c2) and 3 GB (c4) instead of 1.4 / 1.2 GB: nothing of a buffer set is
+    # left in the 256 MB Infinity Cache or the L2s when its turn comes again
+    "c2_cold": lambda t: wl_c2(t, False, sets=8),
+    "c4_cold": lambda t: wl_c4(t, sets=5),
     "c2_inplace_separate": lambda t: wl_c2(t, True, separate=True),
     "c2p_pack": lambda t: wl_c2p(t, False),
     "c2p_unpack": lambda t: wl_c2p(t, True),
@@ -877,8 +884,8 @@ def sweep_transpose(which, dtypes, reps=5, launches=30):
 # The default run reports these beside the headline workload, measured in the same process:
 # workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
 SUMMARY = {
-    "c2": 0.75, "c2_inplace": 0.75, "c2_separate": 0.75, "c2p_pack": 0.75, "c2p_unpack": 0.75,
-    "c3_pack": 0.60, "c3_unpack": 0.60, "c3_reshard_e2e": 0.60, "c4": 0.60, "c4_slots": 0.60,
+    "c2": 0.75, "c2_inplace": 0.75, "c2_separate": 0.75, "c2_cold": 0.75, "c2p_pack": 0.75, "c2p_unpack": 0.75,
+    "c3_pack": 0.60, "c3_unpack": 0.60, "c3_reshard_e2e": 0.60, "c4": 0.60, "c4_slots": 0.60, "c4_cold": 0.60,
     "c5_flat_pack": 0.60, "c5_quantize": 0.60, "c5_dequant": 0.60, "c5_flat_unpack": 0.60,
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
