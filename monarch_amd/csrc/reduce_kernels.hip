@@ -568,7 +568,6 @@ int mhip_reduce(void* out, const void* const* in, uint32_t n, uint64_t numel, in
     a.n = n;
     avg_factors(n, op, &a.scale, &a.divisor);
     a.xcd_contiguous = inputs_alias(in, n);
-    if (const char* e = std::getenv("MONARCH_HIP_EXPERIMENT")) a.xcd_contiguous = std::atoi(e);
     a.op = (uint32_t)op;
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
