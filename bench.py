@@ -442,9 +442,11 @@ def wl_c3_reshard(torch, sets=3, one_by_one=False):
     return "c3_reshard_end_to_end", nbytes, launch, cpu, "slice_copy_kernel<16> + copy_many_kernel", "u8"
 
 
-def wl_stack(torch, scatter=False, sets=2):
+def wl_stack(torch, scatter=False, sets=None):
     """Reduction::Stack of the C2 bucket's 8 chunks in one launch: all_gather_into_tensor (out[g] = in[g]) or, with
-    scatter, all_to_all_single as member 3 sees it (out chunk g = chunk 3 of member g)."""
+    scatter, all_to_all_single as member 3 sees it (out chunk g = chunk 3 of member g).  The all_to_all touches
+    96 MiB per launch, so it rotates over 12 buffer sets (1.1 GB touched); the all_gather moves 1.6 GB per set."""
+    sets = sets or (12 if scatter else 2)
     from monarch_amd import staging
     from monarch_amd._lib import ptr_array
     n, numel = 8, 25_165_824
