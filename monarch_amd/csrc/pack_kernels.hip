@@ -38,8 +38,9 @@ struct PackArgs {
     uint32_t nviews;             // views handled by this launch
     uint64_t wg0;                // workgroups of this copy launched before this grid
     uint32_t pieces;             // slice_unpack_rows_kernel: 1 KiB pieces per row
-    uint64_t per_xcd;            // packs of rows that are not whole cache lines: workgroups in each XCD's contiguous
+    uint64_t per_xcd;            // copies whose pieces share cache lines: workgroups in each XCD's contiguous
     uint64_t nwg;                //   share of the nwg workgroups (0: workgroup i takes tile i)
+    uint32_t stream_stores;      // slice_copy_kernel unpacking 16-byte units: non-temporal instead of write-through stores
     DimsArg dims;
 };
 
@@ -75,11 +76,9 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
     // running side by side work on the same rows of neighbouring views (for column blocks
     // of one tensor: neighbouring segments of the same rows).
     uint64_t wg = a.wg0 + blockIdx.x;
-    if constexpr (PACK) {
-        if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
-            wg = (wg & 7) * a.per_xcd + (wg >> 3);
-            if (wg >= a.nwg) return;
-        }
+    if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
     }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
@@ -148,9 +147,10 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
         for (int i = 0; i < kUnroll; ++i) {
             if constexpr (PACK)
                 store16_writethrough(packed + first[i] * U, data[i]);
-            else if constexpr (U == 16)
-                store16_writethrough(strided + loc[i] * U, data[i]);
-            else
+            else if constexpr (U == 16) {
+                if (a.stream_stores) store16_aligned(strided + loc[i] * U, data[i]);  // wave-uniform
+                else store16_writethrough(strided + loc[i] * U, data[i]);
+            } else
                 store16_unaligned(strided + loc[i] * U, data[i]);
         }
         return;
@@ -187,30 +187,42 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
 // fall off the predicate-free path above.  A straddling chunk is moved as two whole
 // 16-byte vectors instead, each inside one row on both sides: "A" ends where the row ends,
 // "B" starts where the next row starts.  They overlap the neighbouring chunks, which write
-// the same bytes there.  Every lane issues both loads for each of its chunks without
-// predicates (lanes with nothing to do read unit 0, one address for the whole wavefront),
-// so they stay in flight together; only the stores are predicated.  Needs rows of at least one
-// chunk; the ragged first and last chunk of a view still go unit by unit.
+// the same bytes there.  Every lane issues its loads without per-lane predicates, so they stay
+// in flight together; only the stores are predicated.  Lanes with nothing to load read the 16-byte
+// aligned vector that holds the first byte of the side that is read: one address for the whole
+// wavefront, and an ALIGNED one - a wavefront whose lanes all read the same vector at an address
+// that is not 4-byte aligned (a bf16 view that starts at an odd column) takes far longer over it
+// than over 64 consecutive ones.  The "B" loads are skipped by wavefronts without a straddling
+// chunk (decided for the whole wavefront): bf16 rows of 7166 starting at column 1 0.57 -> 0.72 of
+// peak, rows of 3580 0.54 -> 0.68, rows of 1790 0.50 -> 0.60; views on 4-byte boundaries unchanged.
+// Needs rows of at least one chunk; the ragged first and last chunk of a view still go unit by unit.
 constexpr int kRaggedUnroll = 1;  // measured: 1 chunk per lane 0.75, 2 0.73, 4 0.72, 8 0.72 of peak (fp32 rows of 1791)
 
 template <int U, bool PACK, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArgs a) {
     constexpr int VU = 16 / U;
     constexpr int UN = kRaggedUnroll;
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
+    // what idle lanes load: the aligned vector around unit 0 of the side that is read (a "negative" unit index)
+    const uint64_t idle = 0 - (uint64_t)(((uintptr_t)(PACK ? strided : packed) & 15u) / U);
     uint64_t pa[UN], sa[UN], pb[UN], sb[UN];  // packed / strided unit index of vector A and vector B
     bool do_a[UN], do_b[UN], edge[UN];
+    bool any_b = false;
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
         const uint64_t c = c0 + (uint64_t)i * kPackThreads;
         const uint64_t tb = c * VU;
         const uint64_t first = tb - a.shift;
-        pa[i] = sa[i] = pb[i] = sb[i] = 0;
+        pa[i] = sa[i] = pb[i] = sb[i] = idle;
         do_a[i] = do_b[i] = edge[i] = false;
         if (c < a.nchunks) {
             if (tb >= a.shift && first + VU <= a.total) {
@@ -226,18 +238,20 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
                     sa[i] = loc + rem - VU;
                     pb[i] = first + rem;
                     sb[i] = decode<WIDE, NDIM>(a.dims, first + rem, &col);
-                    do_b[i] = true;
+                    do_b[i] = any_b = true;
                 }
             } else {
                 edge[i] = true;
             }
         }
     }
-    uint4 da[UN], db[UN];
+    uint4 da[UN], db[UN] = {};
 #pragma unroll
     for (int i = 0; i < UN; ++i) da[i] = PACK ? load16_unaligned(strided + sa[i] * U) : load16_unaligned(packed + pa[i] * U);
+    if (__builtin_amdgcn_ballot_w64(any_b) != 0) {  // one branch for the whole wavefront
 #pragma unroll
-    for (int i = 0; i < UN; ++i) db[i] = PACK ? load16_unaligned(strided + sb[i] * U) : load16_unaligned(packed + pb[i] * U);
+        for (int i = 0; i < UN; ++i) db[i] = PACK ? load16_unaligned(strided + sb[i] * U) : load16_unaligned(packed + pb[i] * U);
+    }
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
         if (do_a[i]) {
@@ -267,7 +281,11 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
 // (R + 2046) / 1024 pieces whatever its address; pieces that miss the row exit at once.
 template <int U, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_unpack_rows_kernel(PackArgs a) {
-    const uint64_t wg = a.wg0 + blockIdx.x;
+    uint64_t wg = a.wg0 + blockIdx.x;
+    if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
+        wg = (wg & 7) * a.per_xcd + (wg >> 3);
+        if (wg >= a.nwg) return;
+    }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     const uint64_t r = tile / a.pieces;                         // row of the view, in iteration order
@@ -756,8 +774,21 @@ static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint3
 // measure the same either way or better (64 of 256 fp32 columns 0.57 -> 0.63; bf16 columns 0:1792 0.746 both ways), so
 // every single-view pack of whole chunks takes the shares (the eight column blocks of one tensor in one launch, where
 // the view index already pins each view to one XCD, lose with them: 0.78 -> 0.68).  The gathering form does not (bf16 rows of 1790: 0.69 -> 0.59,
-// though fp32 rows of 255 gain 0.03), nor the two-vector form (fp32 rows of 1791: 0.71 -> 0.70), nor unpacks, where
-// shares help some shapes (+0.04) and cost others (-0.07).
+// though fp32 rows of 255 gain 0.03).  The two-vector form and the row-piece unpack take them for rows of 6 KiB and
+// more (bf16 [16384, 14336], columns c:c+7166, packing 0.75 -> 0.78, unpacking 0.72 -> 0.755; rows of 7160 bytes +0.02 /
+// +0.03 to +0.10; rows of 3580 bytes -0.02 either way, so shorter rows keep the plain mapping).
+//
+// Unpacks of whole chunks write the strided side in 1 KiB pieces cut on the packed side's grid.  With units under 16
+// bytes (a view that starts 2-8 bytes past a 16-byte boundary, a pitch that is not a multiple of 16) every piece
+// starts and ends inside a line its neighbours write as well, and the shares let those partial lines meet in one L2
+// before they go to HBM: bf16 columns 1:7169 0.66 -> 0.73, 1:3585 0.60 -> 0.68, 1:1793 0.53 -> 0.59.  16-byte units
+// store write-through while the copy is small enough to stay in the Infinity Cache (58 MB views: 0.87-0.89 in a
+// rotation of 350 MB, 0.54-0.68 with non-temporal stores); from 96 MiB on they stream with non-temporal stores
+// (one column block of 235 MB: 0.70 -> 0.81; 117 MB: 0.70 -> 0.755), and take the shares when rows do not start and
+// end on cache lines (columns 8:7176 0.59 -> 0.73; rows of 14320 bytes 0.545 -> 0.74).  Several views in one launch
+// keep write-through stores at any size (the eight column blocks of a 117 MB tensor: 0.794 against 0.777).
+constexpr uint64_t kSharesFromRowBytes = 6144;
+constexpr uint64_t kStreamUnpackFromBytes = 96ull << 20;
 template <bool PACK>
 static int copy_views(char* base, char* const* packed, const mhip_slice_t* views, uint32_t nviews,
                       uint32_t elem_size, hipStream_t stream) {
@@ -842,7 +873,27 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         if (form == kUnpackRows) blocks = (first.total / first.run) * row_pieces;  // one workgroup per piece of every row
         a.nviews = nbatch;
         uint64_t nwg = blocks * nbatch;
-        if (PACK && nbatch == 1 && form == kWholeChunks) {  // see the note above copy_views
+        // which single-view copies take XCD-contiguous shares, and how an unpack of 16-byte units stores: see the
+        // note above copy_views
+        bool shares = false;
+        if (nbatch == 1) {
+            const uint64_t run_bytes = first.run * unit;
+            if (PACK) {
+                shares = form == kWholeChunks || (form == kRaggedRows && run_bytes >= kSharesFromRowBytes);
+            } else if (form == kUnpackRows) {
+                shares = run_bytes >= kSharesFromRowBytes;
+            } else if (form == kWholeChunks) {
+                if (unit < 16) {
+                    shares = true;
+                } else if (first.total * unit >= kStreamUnpackFromBytes) {
+                    a.stream_stores = 1;
+                    uint64_t mask = (uint64_t)(uintptr_t)(base + first.offset * unit) | run_bytes;
+                    for (int d = 0; d < first.ndim; ++d) mask |= first.dims[d].stride * unit;
+                    shares = (mask & 127u) != 0;  // the 1 KiB pieces a wavefront writes are not whole cache lines
+                }
+            }
+        }
+        if (shares) {
             a.nwg = nwg;
             a.per_xcd = (nwg + 7) / 8;
             nwg = a.per_xcd * 8;

@@ -329,7 +329,7 @@ def test_wide_index_path_over_2g_units():
     assert torch.equal(dst[1: n + 1], src[1: n + 1])
 
 
-def _check_large_view(dtype, sizes, strides, offset=0):
+def _check_large_view(dtype, sizes, strides, offset=0, min_bytes=2**31):
     """pack against torch's own strided gather on the GPU (the CPU walk would take minutes at this size),
     then unpack into zeros: the view comes back and nothing else is written."""
     s = Slice(offset=offset, sizes=sizes, strides=strides)
@@ -345,7 +345,7 @@ def _check_large_view(dtype, sizes, strides, offset=0):
     want = torch.as_strided(src, sizes, strides, offset).contiguous().reshape(-1)
     got = staging.pack(src, s)
     sync()
-    assert got.numel() * es >= 2**31
+    assert got.numel() * es >= min_bytes
     assert torch.equal(got.view(torch.uint8), want.view(torch.uint8))
     del want
     back = torch.zeros_like(src)
@@ -370,6 +370,14 @@ def test_wide_index_short_runs():
 def test_wide_index_whole_chunks():
     # more than 2^31 two-byte units in rows of 4096 bf16 at an odd pitch: 64-bit decode in the whole-chunk form
     _check_large_view(torch.bfloat16, [524_296, 4096], [4097, 1])
+
+
+@pytest.mark.parametrize("c0,cols", [(0, 7168), (8, 7168), (0, 7160), (1, 7168), (3, 7163)])
+def test_single_view_unpacks_of_96_mib_and_more(c0, cols):
+    # from 96 MiB on, an unpack of one view streams its stores and, where its rows do not start and end on cache
+    # lines, gives each XCD a contiguous share of the pieces: whole-line rows, rows 16 bytes into a line, rows of
+    # 14320 bytes, rows at a 2-byte offset (whole chunks) and ragged rows
+    _check_large_view(torch.bfloat16, [8192, cols], [14336, 1], offset=c0, min_bytes=96 << 20)
 
 
 def test_tensor_buffer_round_trip():
