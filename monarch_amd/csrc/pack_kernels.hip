@@ -7,6 +7,7 @@
 //   slice_copy_kernel         rows are whole chunks: one 128-bit access per chunk and side
 //   slice_copy_ragged_kernel  rows of at least a chunk that are not whole chunks: a chunk
 //                             straddling a row boundary moves as two overlapping vectors
+//   slice_unpack_lines_kernel unpacks of such rows from 256 bytes on: whole cache lines of the written side
 //   slice_gather_kernel       runs shorter than (a few) chunks: the chunk's units are
 //                             gathered / scattered one by one
 //   contiguous_copy_kernel    one run of any alignment: rows on the destination's 1 KiB boundaries
@@ -37,7 +38,9 @@ struct PackArgs {
     uint32_t shift;              // units missing from chunk 0 so that chunk c starts 16-byte aligned
     uint32_t nviews;             // views handled by this launch
     uint64_t wg0;                // workgroups of this copy launched before this grid
-    uint32_t pieces;             // slice_unpack_rows_kernel: 1 KiB pieces per row
+    uint32_t pieces;             // slice_unpack_lines_kernel: cache lines a row can overlap
+    FastDiv32 pieces_div;        //   division by it, valid in 32-bit mode
+    uint64_t nrows;              //   rows per view
     uint64_t per_xcd;            // copies whose pieces share cache lines: workgroups in each XCD's contiguous
     uint64_t nwg;                //   share of the nwg workgroups (0: workgroup i takes tile i)
     uint32_t stream_stores;      // slice_copy_kernel unpacking 16-byte units: non-temporal instead of write-through stores
@@ -272,15 +275,21 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
     }
 }
 
-// Unpacking rows that are not whole 16-byte chunks, laid out for the side that is WRITTEN.  The two-vector form
-// above cuts the work on the packed side's 16-byte grid, so on the strided side every 1 KiB a wavefront writes starts
-// and ends inside a cache line that the neighbouring wavefronts (on other XCDs) write as well, and such a line goes to
-// HBM as two partial writes.  Here a workgroup takes one 1 KiB-aligned piece of one row of the strided side: whole
-// aligned vectors inside the row (unaligned loads from the packed image, whose lines are only read), the row's
-// first and last 16 bytes as unaligned vectors where its ends cut a vector, and nothing outside the row.  A row of R bytes needs at most
-// (R + 2046) / 1024 pieces whatever its address; pieces that miss the row exit at once.
+// Unpacking rows that are not whole 16-byte chunks, laid out on the CACHE LINES of the side that is written.  The
+// two-vector form above cuts the work on the packed side's 16-byte grid, so on the strided side every 1 KiB a
+// wavefront writes starts and ends inside a cache line that the neighbouring wavefronts (on other XCDs) write as well,
+// and such a line goes to HBM as two partial writes.  Here a row of R bytes overlaps at most `pieces` lines, and eight
+// consecutive lanes take the eight 16-byte vectors of one line of one row: a wavefront writes eight whole lines, and no
+// line is written by two wavefronts, whatever the rows' length and alignment.  Vectors inside the row are aligned on
+// the written side (unaligned loads from the packed image, whose lines are only read); a vector that the row's start
+// or end cuts is replaced by the row's first or last 16 bytes, an unaligned vector that overlaps its neighbour with the
+// same bytes; lanes past the row's last line idle (they load the row's last vector and store nothing), so no load is
+// predicated.  Against the two-vector form, [16384 rows at a 28 KiB pitch]: bf16 rows of 894 0.36 -> 0.43 of peak, of
+// 1790 0.58 -> 0.62, of 3580 0.66 -> 0.70; u8 rows of 3581 0.51 -> 0.60, of 14333 0.645 -> 0.75; fp32 rows of 447
+// 0.36 -> 0.42, of 1791 0.67 -> 0.71.  (A form with one 1 KiB-aligned piece of one row per wavefront, which this one
+// replaces, gave 0.59 / 0.66 on bf16 rows of 1790 / 3580 and lost on rows around 1 KiB, whose pieces are half empty.)
 template <int U, bool WIDE, int NDIM>
-__global__ __launch_bounds__(kPackThreads) void slice_unpack_rows_kernel(PackArgs a) {
+__global__ __launch_bounds__(kPackThreads) void slice_unpack_lines_kernel(PackArgs a) {
     uint64_t wg = a.wg0 + blockIdx.x;
     if (a.per_xcd != 0) {  // each XCD on a contiguous share: see the note above copy_views
         wg = (wg & 7) * a.per_xcd + (wg >> 3);
@@ -288,23 +297,32 @@ __global__ __launch_bounds__(kPackThreads) void slice_unpack_rows_kernel(PackArg
     }
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
-    const uint64_t r = tile / a.pieces;                         // row of the view, in iteration order
-    const uint32_t piece = (uint32_t)(tile - r * a.pieces);
+    const uint64_t task = tile * (kPackThreads / 8) + (threadIdx.x >> 3);  // one line of one row
+    uint64_t r;                                                             // row of the view, in iteration order
+    uint32_t line;
+    if constexpr (WIDE) {
+        r = task / a.pieces;
+        line = (uint32_t)(task - r * a.pieces);
+    } else {
+        uint32_t q, m;
+        a.pieces_div.divmod((uint32_t)task, q, m);
+        r = q;
+        line = m;
+    }
+    const bool live = r < a.nrows;
+    if (!live) r = 0;
     uint64_t col;
     const uint64_t loc = decode<WIDE, NDIM>(a.dims, r * a.dims.run, &col);  // first unit of the row; col == 0
     char* __restrict__ row = a.base + (a.offset[v] + loc) * U;
     const char* __restrict__ prow = a.packed[v] + r * a.dims.run * U;       // the row in the packed image
-    const int64_t run_bytes = (int64_t)(a.dims.run * U);
-    const int64_t lead = (int64_t)((uintptr_t)row & 1023u);                 // the row starts `lead` bytes into piece 0
-    const int64_t at = (int64_t)piece * 1024 + (int64_t)threadIdx.x * 16 - lead;  // this lane's vector, relative to the row
-    if (at >= 0 && at + 16 <= run_bytes) {
-        store16_aligned(row + at, load16_unaligned(prow + at));
-    } else if (at + 16 > 0 && at < run_bytes) {
-        // a vector that the row's start or end cuts: the row's first or last 16 bytes instead, as one unaligned
-        // vector that stays inside the row; where it overlaps the neighbouring lane's vector both write the same bytes
-        const int64_t o = at < 0 ? 0 : run_bytes - 16;
-        store16_unaligned(row + o, load16_unaligned(prow + o));
-    }
+    const int64_t run_bytes = (int64_t)(a.dims.run * U);                    // at least 16
+    const int64_t lead = (int64_t)((uintptr_t)row & 127u);                  // the row starts `lead` bytes into its first line
+    const int64_t at = (int64_t)line * 128 + (int64_t)(threadIdx.x & 7u) * 16 - lead;  // this lane's vector, relative to the row
+    const bool active = live && at + 16 > 0 && at < run_bytes;
+    int64_t o = at < 0 ? 0 : at;
+    if (o > run_bytes - 16) o = run_bytes - 16;
+    const uint4 d = load16_unaligned(prow + o);
+    if (active) store16_unaligned(row + o, d);
 }
 
 // Views whose contiguous runs are shorter than a chunk (element-strided selections such as
@@ -666,7 +684,7 @@ __global__ __launch_bounds__(THREADS) void flat_copy_kernel(FlatArgs a) {
 
 // ---------------- host side ----------------
 
-enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns, kUnpackRows };
+enum CopyForm { kWholeChunks, kRaggedRows, kShortRuns, kUnpackLines };
 
 template <int U, bool PACK, int UNROLL>
 static void launch_whole_chunks_u(bool wide, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
@@ -705,16 +723,16 @@ static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, 
             }
             return;
         }
-        if (form == kUnpackRows) {
+        if (form == kUnpackLines) {
             if constexpr (!PACK) {
                 if (wide) {
-                    MHIP_LAUNCH((slice_unpack_rows_kernel<U, true, -1>), grid, block, 0, stream, a);
+                    MHIP_LAUNCH((slice_unpack_lines_kernel<U, true, -1>), grid, block, 0, stream, a);
                     return;
                 }
                 switch (ndim) {
-                    case 1: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, 1>), grid, block, 0, stream, a); break;
-                    case 2: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, 2>), grid, block, 0, stream, a); break;
-                    default: MHIP_LAUNCH((slice_unpack_rows_kernel<U, false, -1>), grid, block, 0, stream, a); break;
+                    case 1: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 1>), grid, block, 0, stream, a); break;
+                    case 2: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 2>), grid, block, 0, stream, a); break;
+                    default: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, -1>), grid, block, 0, stream, a); break;
                 }
             }
             return;
@@ -774,7 +792,7 @@ static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint3
 // measure the same either way or better (64 of 256 fp32 columns 0.57 -> 0.63; bf16 columns 0:1792 0.746 both ways), so
 // every single-view pack of whole chunks takes the shares (the eight column blocks of one tensor in one launch, where
 // the view index already pins each view to one XCD, lose with them: 0.78 -> 0.68).  The gathering form does not (bf16 rows of 1790: 0.69 -> 0.59,
-// though fp32 rows of 255 gain 0.03).  The two-vector form and the row-piece unpack take them for rows of 6 KiB and
+// though fp32 rows of 255 gain 0.03).  The two-vector form and the line-by-line unpack take them for rows of 6 KiB and
 // more (bf16 [16384, 14336], columns c:c+7166, packing 0.75 -> 0.78, unpacking 0.72 -> 0.755; rows of 7160 bytes +0.02 /
 // +0.03 to +0.10; rows of 3580 bytes -0.02 either way, so shorter rows keep the plain mapping).
 //
@@ -857,20 +875,31 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             if (first.run < gather_below && first.total >= 2 * vu) form = kShortRuns;
             else if (first.run >= vu) form = kRaggedRows;
         }
-        uint64_t row_pieces = 0;
-        // Unpacking ragged rows of 2 KiB and more in pieces aligned on the written side: bf16 rows of 1790 0.52 -> 0.59 of
-        // peak, of 1790 starting at column 3 0.49 -> 0.55, fp32 rows of 1791 0.59 -> 0.61.  Not for 1-byte units at odd
-        // pitches (0.62 -> 0.51: there the loads would be the byte-misaligned side, which costs more than such stores) nor
-        // for rows around 1 KiB, where half the pieces are nearly empty (fp32 rows of 255: 0.41 -> 0.36).
-        if (!PACK && form == kRaggedRows && unit >= 2 && first.run * unit >= 2048) {
-            form = kUnpackRows;
-            row_pieces = (first.run * unit + 2046) / 1024;
-            a.pieces = (uint32_t)row_pieces;
+        // Unpacking ragged rows of 256 bytes and more line by line of the written side (see slice_unpack_lines_kernel).
+        // Shorter rows keep the two-vector form: their two or three lines would leave half the lanes idle.
+        uint64_t line_blocks = 0;
+        bool wide = !fits32;
+        if (!PACK && form == kRaggedRows && first.run * unit >= 256) {
+            const uint64_t run_bytes = first.run * unit;
+            uint64_t pitch_mask = 0;
+            for (int d = 0; d < first.ndim; ++d) pitch_mask |= first.dims[d].stride * unit;
+            // lines a row overlaps: every row starts at the same place in its line when all pitches are whole lines
+            uint64_t lines = (run_bytes + 128 - unit + 127) / 128;
+            if ((pitch_mask & 127u) == 0) lines = (((uintptr_t)(base + first.offset * unit) & 127u) + run_bytes + 127) / 128;
+            const uint64_t nrows = first.total / first.run;
+            if (lines < kFastDivLimit && nrows <= UINT64_MAX / 8 / lines) {
+                form = kUnpackLines;
+                a.pieces = (uint32_t)lines;
+                a.pieces_div = FastDiv32((uint32_t)lines);
+                a.nrows = nrows;
+                if (nrows * lines + kPackThreads >= kFastDivLimit) wide = true;
+                line_blocks = (nrows * lines + kPackThreads / 8 - 1) / (kPackThreads / 8);
+            }
         }
         const bool large = a.nchunks >= kLargeCopyChunks;
         const uint64_t per_block = (uint64_t)kPackThreads * (form == kRaggedRows ? kRaggedUnroll : form == kShortRuns ? kGatherUnroll : large ? kUnrollLarge : kUnrollSmall);
         uint64_t blocks = (a.nchunks + per_block - 1) / per_block;
-        if (form == kUnpackRows) blocks = (first.total / first.run) * row_pieces;  // one workgroup per piece of every row
+        if (form == kUnpackLines) blocks = line_blocks;  // eight lanes per line of every row
         a.nviews = nbatch;
         uint64_t nwg = blocks * nbatch;
         // which single-view copies take XCD-contiguous shares, and how an unpack of 16-byte units stores: see the
@@ -880,7 +909,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             const uint64_t run_bytes = first.run * unit;
             if (PACK) {
                 shares = form == kWholeChunks || (form == kRaggedRows && run_bytes >= kSharesFromRowBytes);
-            } else if (form == kUnpackRows) {
+            } else if (form == kUnpackLines) {
                 shares = run_bytes >= kSharesFromRowBytes;
             } else if (form == kWholeChunks) {
                 if (unit < 16) {
@@ -900,7 +929,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         }
         if (int rc = launch_in_pieces(nwg, kPackThreads, 8, [&](uint64_t wg0, uint32_t count) {
                 a.wg0 = wg0;
-                launch_slice_copy<PACK>(unit, !fits32, large, form, dim3(count), stream, a);
+                launch_slice_copy<PACK>(unit, wide, large, form, dim3(count), stream, a);
             }))
             return rc;
         k += nbatch;

@@ -139,12 +139,15 @@ def test_rows_that_are_not_whole_chunks(elem_size):
 
 
 @pytest.mark.parametrize("elem_size", [2, 4, 8, 6])
-def test_unpack_of_long_ragged_rows_in_pieces_of_the_written_side(elem_size):
-    # rows of 2 KiB and more that are not whole 16-byte chunks are unpacked in 1 KiB-aligned pieces of the strided
-    # side: rows that start anywhere inside a piece, rows of exactly 2 KiB, three and four dimensions, shifted staging
+def test_unpack_of_ragged_rows_by_cache_lines_of_the_written_side(elem_size):
+    # rows of 256 bytes and more that are not whole 16-byte chunks are unpacked line by line of the strided side:
+    # rows that start anywhere inside a line, rows of exactly 2 KiB, three and four dimensions, shifted staging,
+    # rows just above and below 256 bytes, rows that end one element into a line
     cases = [Slice(offset=3, sizes=[5, 40, 1027], strides=[46200, 1100, 1]), Slice(offset=0, sizes=[64, 1025], strides=[1031, 1]),
              Slice(offset=509, sizes=[31, 2049], strides=[2051, 1]), Slice(offset=1, sizes=[2, 3, 5, 1301], strides=[33600, 8400, 1400, 1]),
-             Slice(offset=7, sizes=[3, 9001], strides=[9002, 1])]
+             Slice(offset=7, sizes=[3, 9001], strides=[9002, 1]),
+             Slice(offset=0, sizes=[700, 129], strides=[192, 1]), Slice(offset=5, sizes=[900, 127], strides=[131, 1]),
+             Slice(offset=0, sizes=[333, 65], strides=[64 * 3, 1]), Slice(offset=63, sizes=[50, 7, 257], strides=[7 * 320, 320, 1])]
     for i, s in enumerate(cases):
         for dst_misalign in (0, elem_size, 7 * elem_size):
             _roundtrip(s, elem_size, seed=20 + i, misalign=(i % 4) * elem_size, dst_misalign=dst_misalign)
