@@ -94,12 +94,16 @@ __device__ __forceinline__ uint64_t decode(const DimsArg& d, uint64_t t, uint64_
     return off;
 }
 
+// `type` is the unit as a value; `mem` is what a pointer into tensor memory points to.  The strided side of a copy is
+// only guaranteed byte-aligned up to the element size of the CALLER's tensor, which may be less than the unit (a view
+// of 4-byte-granular shape that starts at an odd bf16 column), so units in memory carry no alignment assumption;
+// gfx950 under the HSA runtime services such accesses in hardware.
 template <int U> struct UnitType;
-template <> struct UnitType<1> { using type = uint8_t; };
-template <> struct UnitType<2> { using type = uint16_t; };
-template <> struct UnitType<4> { using type = uint32_t; };
-template <> struct UnitType<8> { using type = uint64_t; };
-template <> struct UnitType<16> { using type = uint4; };
+template <> struct UnitType<1> { using type = uint8_t; using mem = uint8_t; };
+template <> struct UnitType<2> { using type = uint16_t; typedef uint16_t __attribute__((aligned(1))) mem; };
+template <> struct UnitType<4> { using type = uint32_t; typedef uint32_t __attribute__((aligned(1))) mem; };
+template <> struct UnitType<8> { using type = uint64_t; typedef uint64_t __attribute__((aligned(1))) mem; };
+template <> struct UnitType<16> { using type = uint4; using mem = uint4; };
 
 // 16-byte access at an address that is only known to be unit-aligned.  gfx950 under
 // the HSA runtime services unaligned global dwordx4 accesses in hardware, and the

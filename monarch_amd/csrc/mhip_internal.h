@@ -35,8 +35,11 @@ struct CanonSlice {
 // chosen as the largest power of two <= max_unit that divides the element size, every
 // byte stride, the byte offset, and the alignments passed in `align_mask` (OR of the
 // addresses involved).  Returns false for an empty slice.
+// With `skew` the view's own byte offset does not limit the unit (for kernels whose accesses to the strided side
+// tolerate any address): out->offset is rounded down to whole units and *skew receives the bytes left over, which the
+// caller adds to the base pointer.
 bool canonicalize(const mhip_slice_t& s, uint32_t elem_size, uint64_t align_mask, uint32_t max_unit,
-                  CanonSlice* out, uint32_t* unit);
+                  CanonSlice* out, uint32_t* unit, uint64_t* skew = nullptr);
 
 // Same dimension list for two canonical slices (offsets may differ).
 bool same_shape(const CanonSlice& a, const CanonSlice& b);

@@ -50,10 +50,11 @@ struct PackArgs {
 template <int U, bool PACK>
 __device__ __forceinline__ void move_unit(char* strided, char* packed) {
     using T = typename UnitType<U>::type;
+    using M = typename UnitType<U>::mem;  // the strided side may be less aligned than the unit
     if constexpr (PACK)
-        *reinterpret_cast<T*>(packed) = *reinterpret_cast<const T*>(strided);
+        *reinterpret_cast<T*>(packed) = *reinterpret_cast<const M*>(strided);
     else
-        *reinterpret_cast<T*>(strided) = *reinterpret_cast<const T*>(packed);
+        *reinterpret_cast<M*>(strided) = *reinterpret_cast<const T*>(packed);
 }
 
 // One chunk moved unit by unit, with every unit tested against the view's extent: the ragged first
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_kernel(PackArgs a) {
             if constexpr (PACK)
                 store16_writethrough(packed + first[i] * U, data[i]);
             else if constexpr (U == 16) {
-                if (a.stream_stores) store16_aligned(strided + loc[i] * U, data[i]);  // wave-uniform
+                if (a.stream_stores) store16_unaligned(strided + loc[i] * U, data[i]);  // wave-uniform
                 else store16_writethrough(strided + loc[i] * U, data[i]);
             } else
                 store16_unaligned(strided + loc[i] * U, data[i]);
@@ -215,8 +216,8 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
     char* __restrict__ packed = a.packed[v];
     char* __restrict__ strided = a.base + a.offset[v] * U;
     const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
-    // what idle lanes load: the aligned vector around unit 0 of the side that is read (a "negative" unit index)
-    const uint64_t idle = 0 - (uint64_t)(((uintptr_t)(PACK ? strided : packed) & 15u) / U);
+    // what idle lanes load: the aligned vector that holds the first byte of the side that is read
+    const char* const idle = reinterpret_cast<const char*>((uintptr_t)(PACK ? strided : packed) & ~(uintptr_t)15);
     uint64_t pa[UN], sa[UN], pb[UN], sb[UN];  // packed / strided unit index of vector A and vector B
     bool do_a[UN], do_b[UN], edge[UN];
     bool any_b = false;
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
         const uint64_t c = c0 + (uint64_t)i * kPackThreads;
         const uint64_t tb = c * VU;
         const uint64_t first = tb - a.shift;
-        pa[i] = sa[i] = pb[i] = sb[i] = idle;
+        pa[i] = sa[i] = pb[i] = sb[i] = 0;
         do_a[i] = do_b[i] = edge[i] = false;
         if (c < a.nchunks) {
             if (tb >= a.shift && first + VU <= a.total) {
@@ -250,10 +251,16 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
     }
     uint4 da[UN], db[UN] = {};
 #pragma unroll
-    for (int i = 0; i < UN; ++i) da[i] = PACK ? load16_unaligned(strided + sa[i] * U) : load16_unaligned(packed + pa[i] * U);
+    for (int i = 0; i < UN; ++i) {
+        const char* from = PACK ? strided + sa[i] * U : packed + pa[i] * U;
+        da[i] = load16_unaligned(do_a[i] ? from : idle);
+    }
     if (__builtin_amdgcn_ballot_w64(any_b) != 0) {  // one branch for the whole wavefront
 #pragma unroll
-        for (int i = 0; i < UN; ++i) db[i] = PACK ? load16_unaligned(strided + sb[i] * U) : load16_unaligned(packed + pb[i] * U);
+        for (int i = 0; i < UN; ++i) {
+            const char* from = PACK ? strided + sb[i] * U : packed + pb[i] * U;
+            db[i] = load16_unaligned(do_b[i] ? from : idle);
+        }
     }
 #pragma unroll
     for (int i = 0; i < UN; ++i) {
@@ -344,7 +351,8 @@ __global__ __launch_bounds__(kPackThreads) void slice_gather_kernel(PackArgs a) 
     const uint64_t tile = wg / a.nviews;
     const uint32_t v = (uint32_t)(wg % a.nviews);
     char* __restrict__ packed = a.packed[v];
-    T* __restrict__ strided = reinterpret_cast<T*>(a.base) + a.offset[v];
+    using M = typename UnitType<U>::mem;  // the strided side may be less aligned than the unit
+    M* __restrict__ strided = reinterpret_cast<M*>(a.base) + a.offset[v];
     const uint64_t c0 = tile * (kPackThreads * UN) + threadIdx.x;
     const int nd = NDIM >= 0 ? NDIM : a.dims.ndim;
     const uint64_t run = a.dims.run;
@@ -834,6 +842,24 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
                 continue;
             }
         }
+        // The direct forms reach the strided side with accesses that tolerate any address (see UnitType), so the
+        // address at which a view starts need not limit the unit: a bf16 view of even row length and pitch that
+        // starts at an odd column is moved in 4-byte units from a base that is 2 bytes off.  On bf16 [16384, 14336]:
+        // columns 1:895 pack 0.46 -> 0.66 of peak (the 4-byte gathering form instead of the 2-byte two-vector form),
+        // 1:1791 0.61 -> 0.67, columns 1:897 unpack 0.41 -> 0.60, 1:1793 0.59 -> 0.70; never slower.
+        uint64_t skew = 0;  // bytes from `base` to the address the unit offsets count from
+        if (unit < 16) {
+            CanonSlice relaxed;
+            uint32_t unit_r = 0;
+            uint64_t skew_r = 0;
+            canonicalize(views[k], elem_size, (uint64_t)(uintptr_t)packed[k], 16, &relaxed, &unit_r, &skew_r);
+            if (unit_r > unit) {
+                first = relaxed;
+                unit = unit_r;
+                skew = skew_r;
+            }
+        }
+        const bool any_base = skew != 0 || ((uintptr_t)base & (unit - 1)) != 0;  // the unit was chosen without the strided address
         PackArgs a{};
         bool fits32 = false;
         if (!make_dims_arg(first, &a.dims, &fits32)) {
@@ -842,7 +868,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             continue;
         }
         const uint32_t shift_bytes = (uint32_t)((uintptr_t)packed[k] & 15u);
-        a.base = base;
+        a.base = base + skew;
         a.total = first.total;
         a.shift = shift_bytes / unit;
         const uint32_t vu = 16 / unit;
@@ -854,9 +880,10 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
         while (k + nbatch < nviews && nbatch < (uint32_t)kMaxViews) {
             CanonSlice next;
             uint32_t unit2 = 0;
-            const uint64_t mask = (uint64_t)(uintptr_t)base | (uint64_t)(uintptr_t)packed[k + nbatch];
-            if (!canonicalize(views[k + nbatch], elem_size, mask, 16, &next, &unit2)) break;
-            if (unit2 != unit || !same_shape(first, next)) break;
+            uint64_t skew2 = 0;
+            const uint64_t mask = (any_base ? 0 : (uint64_t)(uintptr_t)base) | (uint64_t)(uintptr_t)packed[k + nbatch];
+            if (!canonicalize(views[k + nbatch], elem_size, mask, 16, &next, &unit2, any_base ? &skew2 : nullptr)) break;
+            if (unit2 != unit || skew2 != skew || !same_shape(first, next)) break;
             if (((uintptr_t)packed[k + nbatch] & 15u) != shift_bytes) break;
             a.packed[nbatch] = packed[k + nbatch];
             a.offset[nbatch] = next.offset;
@@ -885,7 +912,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             for (int d = 0; d < first.ndim; ++d) pitch_mask |= first.dims[d].stride * unit;
             // lines a row overlaps: every row starts at the same place in its line when all pitches are whole lines
             uint64_t lines = (run_bytes + 128 - unit + 127) / 128;
-            if ((pitch_mask & 127u) == 0) lines = (((uintptr_t)(base + first.offset * unit) & 127u) + run_bytes + 127) / 128;
+            if ((pitch_mask & 127u) == 0) lines = (((uintptr_t)(a.base + first.offset * unit) & 127u) + run_bytes + 127) / 128;
             const uint64_t nrows = first.total / first.run;
             if (lines < kFastDivLimit && nrows <= UINT64_MAX / 8 / lines) {
                 form = kUnpackLines;
@@ -916,7 +943,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
                     shares = true;
                 } else if (first.total * unit >= kStreamUnpackFromBytes) {
                     a.stream_stores = 1;
-                    uint64_t mask = (uint64_t)(uintptr_t)(base + first.offset * unit) | run_bytes;
+                    uint64_t mask = (uint64_t)(uintptr_t)(a.base + first.offset * unit) | run_bytes;
                     for (int d = 0; d < first.ndim; ++d) mask |= first.dims[d].stride * unit;
                     shares = (mask & 127u) != 0;  // the 1 KiB pieces a wavefront writes are not whole cache lines
                 }

@@ -13,7 +13,7 @@ static inline uint32_t pow2_factor(uint64_t v, uint32_t cap) {
 }
 
 bool canonicalize(const mhip_slice_t& s, uint32_t elem_size, uint64_t align_mask, uint32_t max_unit,
-                  CanonSlice* out, uint32_t* unit) {
+                  CanonSlice* out, uint32_t* unit, uint64_t* skew) {
     uint64_t len = 1;
     for (uint32_t k = 0; k < s.ndim; ++k) len *= s.sizes[k];
     if (len == 0 || elem_size == 0) return false;
@@ -43,11 +43,12 @@ bool canonicalize(const mhip_slice_t& s, uint32_t elem_size, uint64_t align_mask
         merged.pop_back();
     }
 
-    uint64_t mask = align_mask | run_bytes | (s.offset * elem_size);
+    uint64_t mask = align_mask | run_bytes | (skew ? 0 : s.offset * elem_size);
     for (const CanonDim& d : merged) mask |= d.stride;
     const uint32_t u = pow2_factor(mask, max_unit);
 
     out->offset = s.offset * elem_size / u;
+    if (skew) *skew = s.offset * elem_size % u;
     out->total = len * elem_size / u;
     out->run = run_bytes / u;
     out->ndim = (int)merged.size();

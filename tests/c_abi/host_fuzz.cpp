@@ -42,14 +42,14 @@ static uint64_t byte_by_definition(const mhip_slice_t& s, uint32_t elem_size, ui
 }
 
 // the same through the canonical form: row-major decode of the dimensions outside the run
-static uint64_t byte_by_canonical_form(const CanonSlice& c, uint32_t unit, uint64_t byte) {
+static uint64_t byte_by_canonical_form(const CanonSlice& c, uint32_t unit, uint64_t byte, uint64_t skew = 0) {
     const uint64_t t = byte / unit;
     uint64_t row = t / c.run, off = c.offset + t % c.run;
     for (int k = c.ndim - 1; k >= 0; --k) {
         off += (row % c.dims[k].size) * c.dims[k].stride;
         row /= c.dims[k].size;
     }
-    return off * unit + byte % unit;
+    return off * unit + byte % unit + skew;
 }
 
 int main() {
@@ -178,6 +178,15 @@ int main() {
             const uint64_t stride = nbytes > 4096 ? 1 + below(7) : 1;  // sample long ones
             for (uint64_t byte = below(stride); byte < nbytes; byte += stride)
                 CHECK(byte_by_canonical_form(c, unit, byte) == byte_by_definition(s, es, byte));
+            // the form whose unit the view's own offset does not limit: at least as coarse, same bytes
+            CanonSlice r;
+            uint32_t unit_r = 0;
+            uint64_t skew = ~0ull;
+            CHECK(canonicalize(s, es, mask, max_unit, &r, &unit_r, &skew));
+            CHECK(unit_r >= unit && unit_r <= max_unit && (unit_r & (unit_r - 1)) == 0 && (mask & (unit_r - 1)) == 0);
+            CHECK(skew < unit_r && r.total * unit_r == len * es && r.ndim == c.ndim);
+            for (uint64_t byte = below(stride); byte < nbytes; byte += stride)
+                CHECK(byte_by_canonical_form(r, unit_r, byte, skew) == byte_by_definition(s, es, byte));
         }
 
         // a mesh over the same slice: the members of each dimension contain the rank itself

@@ -138,6 +138,45 @@ def test_rows_that_are_not_whole_chunks(elem_size):
             _roundtrip(s, elem_size, seed=i, misalign=(i % 3) * elem_size, dst_misalign=dst_misalign)
 
 
+@pytest.mark.parametrize("elem_size", [1, 2, 4])
+def test_views_that_start_off_the_unit_of_their_shape(elem_size):
+    # row length and pitch allow a wider unit than the address the view starts at (a bf16 view of even shape at an odd
+    # column, a base pointer that is only element-aligned): the copy runs in the wider unit from a skewed base
+    e = elem_size
+    cases = [Slice(offset=1, sizes=[300, 8 // e * 447], strides=[8 // e * 1024, 1]),     # rows of 3576 bytes: 8-byte units
+             Slice(offset=3, sizes=[100, 16 // e * 224], strides=[16 // e * 512, 1]),    # whole 16-byte chunks, 16-byte units
+             Slice(offset=1, sizes=[64, 16 // e * 500], strides=[16 // e * 512, 1]),     # rows of 8000 bytes
+             Slice(offset=5, sizes=[9, 40, 4 // e * 33], strides=[40 * 4 // e * 64, 4 // e * 64, 1]),  # rows of 132 bytes: gathered
+             Slice(offset=7, sizes=[2000, 4 // e * 3], strides=[4 // e * 5, 1]),          # runs of 12 bytes
+             Slice(offset=2, sizes=[70, 16 // e * 70], strides=[16 // e * 71, 1])]
+    for i, s in enumerate(cases):
+        for misalign in (0, e, 3 * e):
+            for dst_misalign in (0, 16):
+                _roundtrip(s, e, seed=40 + i, misalign=misalign, dst_misalign=dst_misalign)
+    # several views in one launch: equal skews batch, different ones do not
+    g = torch.Generator().manual_seed(41)
+    x = torch.randint(0, 256, (64, 8192 * e), dtype=torch.uint8, generator=g)
+    dev = x.to(DEV)
+    n = 16 // e * 100
+    offsets = [1, 1 + n, 1 + 2 * n, 2 + 3 * n, 5 + 4 * n]
+    views = [Slice(offset=o, sizes=[64, n], strides=[8192, 1]) for o in offsets]
+    outs = [torch.empty(64 * n * e, dtype=torch.uint8, device=DEV) for _ in views]
+    import ctypes as C
+    from monarch_amd._lib import check, lib, ptr_array
+    from monarch_amd.ndslice import slice_array
+    arr = slice_array(views)
+    stream = torch.cuda.current_stream().cuda_stream
+    check(lib().mhip_slice_pack_many(ptr_array([o.data_ptr() for o in outs]), dev.data_ptr(), arr, len(views), e, stream))
+    back = torch.full_like(dev, 0x3C)
+    check(lib().mhip_slice_unpack_many(back.data_ptr(), ptr_array([o.data_ptr() for o in outs]), arr, len(views), e, stream))
+    sync()
+    want = torch.full_like(x, 0x3C)
+    for o, out in zip(offsets, outs):
+        assert torch.equal(out.cpu().view(64, n * e), x[:, o * e: (o + n) * e]), o
+        want[:, o * e: (o + n) * e] = x[:, o * e: (o + n) * e]
+    assert torch.equal(back.cpu(), want)
+
+
 @pytest.mark.parametrize("elem_size", [2, 4, 8, 6])
 def test_unpack_of_ragged_rows_by_cache_lines_of_the_written_side(elem_size):
     # rows of 256 bytes and more that are not whole 16-byte chunks are unpacked line by line of the strided side:
