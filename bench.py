@@ -883,6 +883,73 @@ def sweep_transpose(which, dtypes, reps=5, launches=30):
             torch.cuda.empty_cache()
 
 
+STRIDED_VIEWS_HEADER = """\
+# Strided pack / unpack of one column range: row length x alignment (MI355X)
+
+Command (repository root, one GPU; under a minute):
+
+    python bench.py --sweep strided_views > profiles/strided_views_map.md
+
+Every cell is the fraction of the 8 TB/s HBM peak that `mhip_slice_pack` / `mhip_slice_unpack` reach on the view
+`x[:, c0:c0 + cols]` of a `[16384, pitch]` matrix whose rows are 28 KiB apart (algorithmic bytes = 2 x elements x
+element size); median of 3 runs of {launches} launches, 3 rotating buffer sets.  Rows of a multiple of 16 bytes take the
+whole-chunk form (line by line when a view of 96 MiB and more does not start and end its rows on cache lines), other
+rows the two-vector form when packed (the gathering form under 4 KiB where shape and pitch are 4-byte granular) and the
+line-by-line form when unpacked; a view that starts off the unit of its shape (c0 = 1) is moved in that unit from a
+skewed base.  Views of 59 MB and less (rows of 1792 bytes and less) partly live in the 256 MB Infinity Cache across the
+three buffer sets; the larger ones do not.
+"""
+
+
+def sweep_strided_views(dtypes, launches=20):
+    """Fraction of HBM peak of single-view strided packs and unpacks over row lengths and starting columns
+    (--sweep strided_views): whole-chunk rows, ragged rows, views that start off the unit of their shape."""
+    torch, lib, _ = _load()
+    from monarch_amd import Slice
+    torch.cuda.set_device(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    types = {"u8": (torch.uint8, 1), "bf16": (torch.bfloat16, 2), "f32": (torch.float32, 4), "f64": (torch.float64, 8)}
+    rows, pitch_bytes = 16384, 28672
+    print(STRIDED_VIEWS_HEADER.format(launches=launches))
+    for name in dtypes:
+        dt, es = types[name]
+        pitch = pitch_bytes // es
+        bufs = []
+        for _ in range(3):
+            x = torch.empty(rows, pitch, dtype=dt, device="cuda:0")
+            x.view(torch.uint8).random_(0, 255)
+            bufs.append((x, torch.empty(rows * pitch // 2, dtype=dt, device="cuda:0")))
+        print(f"\n### {name} ({es}-byte elements), pitch {pitch}\n")
+        print("| cols (row bytes) | c0 | pack | unpack |")
+        print("|---|---:|---:|---:|")
+        for row_bytes in (1788, 1792, 3580, 3584, 7160, 7168, 14332, 14336):
+            cols = row_bytes // es
+            for c0 in (0, 1, 16 // es):
+                if c0 + cols > pitch:
+                    continue
+                s = Slice.of_tensor(bufs[0][0][:, c0:c0 + cols])
+                cell = []
+                for sym in ("mhip_slice_pack", "mhip_slice_unpack"):
+                    if sym.endswith("unpack"):
+                        calls = [prepared(sym, x.data_ptr(), st.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+                    else:
+                        calls = [prepared(sym, st.data_ptr(), x.data_ptr(), C.byref(s.c), es, STREAM()) for x, st in bufs]
+                    res = []
+                    for _ in range(3):
+                        for i in range(3):
+                            assert calls[i % 3]() == 0
+                        torch.cuda.synchronize()
+                        ev = Events(lib, stream)
+                        ev.start()
+                        for i in range(launches):
+                            calls[i % 3]()
+                        res.append(2 * rows * cols * es / (ev.stop_ms() / launches) / 1e6 / HBM_PEAK_GBS)
+                    cell.append(sorted(res)[1])
+                print(f"| {cols} ({cols * es}) | {c0} | {cell[0]:.3f} | {cell[1]:.3f} |", flush=True)
+        del bufs, calls
+        torch.cuda.empty_cache()
+
+
 # The default run reports these beside the headline workload, measured in the same process:
 # workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
 SUMMARY = {
@@ -983,11 +1050,14 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", choices=sorted(SWEEPS), help="print an A/B table instead of the bench line")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views"], help="print an A/B table instead of the bench line")
     ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep == "strided_views":
+        sweep_strided_views([d for d in args.dtypes.split(",") if d != "f64"])
+        return
     if args.sweep:
         sweep_transpose(args.sweep, args.dtypes.split(","))
         return

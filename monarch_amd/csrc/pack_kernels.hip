@@ -718,6 +718,20 @@ static void launch_whole_chunks(bool wide, bool large, int ndim, dim3 grid, hipS
 template <int U, bool PACK>
 static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, dim3 grid, hipStream_t stream, const PackArgs& a) {
     const dim3 block(kPackThreads);
+    if (form == kUnpackLines) {
+        if constexpr (!PACK) {
+            if (wide) {
+                MHIP_LAUNCH((slice_unpack_lines_kernel<U, true, -1>), grid, block, 0, stream, a);
+                return;
+            }
+            switch (ndim) {
+                case 1: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 1>), grid, block, 0, stream, a); break;
+                case 2: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 2>), grid, block, 0, stream, a); break;
+                default: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, -1>), grid, block, 0, stream, a); break;
+            }
+        }
+        return;
+    }
     if constexpr (U < 16) {
         if (form == kShortRuns) {
             if (wide) {
@@ -728,20 +742,6 @@ static void launch_slice_copy_u(bool wide, bool large, CopyForm form, int ndim, 
                 case 1: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 1>), grid, block, 0, stream, a); break;
                 case 2: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, 2>), grid, block, 0, stream, a); break;
                 default: MHIP_LAUNCH((slice_gather_kernel<U, PACK, false, -1>), grid, block, 0, stream, a); break;
-            }
-            return;
-        }
-        if (form == kUnpackLines) {
-            if constexpr (!PACK) {
-                if (wide) {
-                    MHIP_LAUNCH((slice_unpack_lines_kernel<U, true, -1>), grid, block, 0, stream, a);
-                    return;
-                }
-                switch (ndim) {
-                    case 1: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 1>), grid, block, 0, stream, a); break;
-                    case 2: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, 2>), grid, block, 0, stream, a); break;
-                    default: MHIP_LAUNCH((slice_unpack_lines_kernel<U, false, -1>), grid, block, 0, stream, a); break;
-                }
             }
             return;
         }
@@ -768,7 +768,7 @@ static void launch_slice_copy(uint32_t unit, bool wide, bool large, CopyForm for
         case 2: launch_slice_copy_u<2, PACK>(wide, large, form, a.dims.ndim, grid, stream, a); break;
         case 4: launch_slice_copy_u<4, PACK>(wide, large, form, a.dims.ndim, grid, stream, a); break;
         case 8: launch_slice_copy_u<8, PACK>(wide, large, form, a.dims.ndim, grid, stream, a); break;
-        default: launch_slice_copy_u<16, PACK>(wide, large, kWholeChunks, a.dims.ndim, grid, stream, a); break;
+        default: launch_slice_copy_u<16, PACK>(wide, large, form == kUnpackLines ? kUnpackLines : kWholeChunks, a.dims.ndim, grid, stream, a); break;
     }
 }
 
@@ -810,9 +810,10 @@ static int copy_deep_view(char* base, char* packed, const mhip_slice_t& s, uint3
 // before they go to HBM: bf16 columns 1:7169 0.66 -> 0.73, 1:3585 0.60 -> 0.68, 1:1793 0.53 -> 0.59.  16-byte units
 // store write-through while the copy is small enough to stay in the Infinity Cache (58 MB views: 0.87-0.89 in a
 // rotation of 350 MB, 0.54-0.68 with non-temporal stores); from 96 MiB on they stream with non-temporal stores
-// (one column block of 235 MB: 0.70 -> 0.81; 117 MB: 0.70 -> 0.755), and take the shares when rows do not start and
-// end on cache lines (columns 8:7176 0.59 -> 0.73; rows of 14320 bytes 0.545 -> 0.74).  Several views in one launch
-// keep write-through stores at any size (the eight column blocks of a 117 MB tensor: 0.794 against 0.777).
+// (one column block of 235 MB: 0.70 -> 0.81; 117 MB: 0.70 -> 0.755); when their rows do not start and end on cache
+// lines they are unpacked line by line instead (rows of 256 bytes and more; columns 8:7176 0.59 -> 0.76), or take the
+// shares (shorter rows).  Several views in one launch keep write-through stores at any size (the eight column blocks
+// of a 117 MB tensor: 0.794 against 0.777).
 constexpr uint64_t kSharesFromRowBytes = 6144;
 constexpr uint64_t kStreamUnpackFromBytes = 96ull << 20;
 template <bool PACK>
@@ -903,10 +904,19 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             else if (first.run >= vu) form = kRaggedRows;
         }
         // Unpacking ragged rows of 256 bytes and more line by line of the written side (see slice_unpack_lines_kernel).
-        // Shorter rows keep the two-vector form: their two or three lines would leave half the lanes idle.
+        // Shorter rows keep the two-vector form: their two or three lines would leave half the lanes idle.  Rows of
+        // whole chunks that do not start and end on cache lines go the same way once a single view is too large to
+        // stay in the Infinity Cache (bf16 columns 8:7176 of [16384, 14336]: 0.73 with the chunk grid, streamed stores
+        // and XCD shares, 0.76 line by line; below that size write-through stores on the chunk grid win, 0.85 against 0.58).
         uint64_t line_blocks = 0;
         bool wide = !fits32;
-        if (!PACK && form == kRaggedRows && first.run * unit >= 256) {
+        bool lines_of_whole_chunks = false;
+        if (!PACK && form == kWholeChunks && nbatch == 1 && first.total * unit >= kStreamUnpackFromBytes) {
+            uint64_t mask = (uint64_t)(uintptr_t)(a.base + first.offset * unit) | (first.run * unit);
+            for (int d = 0; d < first.ndim; ++d) mask |= first.dims[d].stride * unit;
+            lines_of_whole_chunks = (mask & 127u) != 0;
+        }
+        if (!PACK && (form == kRaggedRows || lines_of_whole_chunks) && first.run * unit >= 256) {
             const uint64_t run_bytes = first.run * unit;
             uint64_t pitch_mask = 0;
             for (int d = 0; d < first.ndim; ++d) pitch_mask |= first.dims[d].stride * unit;
