@@ -920,9 +920,17 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             const uint64_t run_bytes = first.run * unit;
             uint64_t pitch_mask = 0;
             for (int d = 0; d < first.ndim; ++d) pitch_mask |= first.dims[d].stride * unit;
-            // lines a row overlaps: every row starts at the same place in its line when all pitches are whole lines
+            // lines a row overlaps: all rows of a view start at the same place in their lines when all pitches are
+            // whole lines (the views of one launch each at their own)
             uint64_t lines = (run_bytes + 128 - unit + 127) / 128;
-            if ((pitch_mask & 127u) == 0) lines = (((uintptr_t)(a.base + first.offset * unit) & 127u) + run_bytes + 127) / 128;
+            if ((pitch_mask & 127u) == 0) {
+                uint64_t lead = 0;
+                for (uint32_t v = 0; v < nbatch; ++v) {
+                    const uint64_t l = (uintptr_t)(a.base + a.offset[v] * unit) & 127u;
+                    lead = l > lead ? l : lead;
+                }
+                lines = (lead + run_bytes + 127) / 128;
+            }
             const uint64_t nrows = first.total / first.run;
             if (lines < kFastDivLimit && nrows <= UINT64_MAX / 8 / lines) {
                 form = kUnpackLines;

@@ -210,6 +210,19 @@ def test_unpack_of_ragged_rows_by_cache_lines_of_the_written_side(elem_size):
     for v in views:
         want[:, (v.offset) * nbytes: (v.offset + 1201) * nbytes] = x[:, v.offset * nbytes: (v.offset + 1201) * nbytes]
     assert torch.equal(back.cpu(), want)
+    # the same with a pitch of whole cache lines: every view's rows then sit at one place in their lines, each view
+    # at its own, and the number of lines a row overlaps differs between the views of the launch
+    x = torch.randint(0, 256, (40, 4096 * nbytes), dtype=torch.uint8, generator=g)
+    dev = x.to(DEV)
+    views = [Slice(offset=k * 1201, sizes=[40, 1201], strides=[4096, 1]) for k in range(3)]
+    arr = slice_array(views)
+    check(lib().mhip_slice_pack_many(ptr_array([o.data_ptr() for o in outs]), dev.data_ptr(), arr, len(views), nbytes, stream))
+    back = torch.full_like(dev, 0x3C)
+    check(lib().mhip_slice_unpack_many(back.data_ptr(), ptr_array([o.data_ptr() for o in outs]), arr, len(views), nbytes, stream))
+    sync()
+    want = torch.full_like(x, 0x3C)
+    want[:, :3 * 1201 * nbytes] = x[:, :3 * 1201 * nbytes]
+    assert torch.equal(back.cpu(), want)
 
 
 def test_wide_index_unpack_of_long_ragged_rows():
