@@ -922,7 +922,8 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
             for (int d = 0; d < first.ndim; ++d) pitch_mask |= first.dims[d].stride * unit;
             // lines a row overlaps: all rows of a view start at the same place in their lines when all pitches are
             // whole lines (the views of one launch each at their own)
-            uint64_t lines = (run_bytes + 128 - unit + 127) / 128;
+            const uint64_t row_align = any_base ? 1 : unit;  // what every row's address is a multiple of
+            uint64_t lines = (run_bytes + 128 - row_align + 127) / 128;
             if ((pitch_mask & 127u) == 0) {
                 uint64_t lead = 0;
                 for (uint32_t v = 0; v < nbatch; ++v) {

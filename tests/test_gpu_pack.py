@@ -153,6 +153,9 @@ def test_views_that_start_off_the_unit_of_their_shape(elem_size):
         for misalign in (0, e, 3 * e):
             for dst_misalign in (0, 16):
                 _roundtrip(s, e, seed=40 + i, misalign=misalign, dst_misalign=dst_misalign)
+    # rows of 8-byte-granular shape from a base that is 2 bytes off: some rows start 122 bytes into a cache line, deeper
+    # than any address that is a multiple of the unit, and overlap one line more
+    _roundtrip(Slice(offset=0, sizes=[56, 776 // e], strides=[792 // e, 1]), e, seed=47, misalign=2 if e <= 2 else e, dst_misalign=0)
     # several views in one launch: equal skews batch, different ones do not
     g = torch.Generator().manual_seed(41)
     x = torch.randint(0, 256, (64, 8192 * e), dtype=torch.uint8, generator=g)
