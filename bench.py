@@ -387,6 +387,42 @@ def wl_c3(torch, unpack=False, sets=3):
     return ("c3_column_block_unpack" if unpack else "c3_column_block_pack"), nbytes, launch, cpu, "slice_copy_kernel<16>", "u8"
 
 
+def wl_ragged(torch, unpack=False, sets=3):
+    """A column block that fits no 16-byte grid: columns 1:7167 of a bf16 [16384, 14336] matrix (rows of 14332 bytes that
+    start 2 bytes into a 16-byte vector), packed to / unpacked from one contiguous buffer.  The view is moved in 4-byte
+    units from a base that is 2 bytes off: the two-vector form packing, the line-by-line form unpacking."""
+    from monarch_amd import Slice
+    g = torch.Generator(device="cuda:0").manual_seed(3100)
+    rows, pitch, c0, cols = 16384, 14336, 1, 7166
+    view = Slice(offset=c0, sizes=[rows, cols], strides=[pitch, 1])
+    bufs = []
+    for _ in range(sets):
+        w = (torch.randn(rows, pitch, generator=g, device="cuda:0") * 0.02).bfloat16()
+        out = w[:, c0:c0 + cols].contiguous().reshape(-1)
+        bufs.append((w, out))
+    nbytes = 2 * rows * cols * 2
+    if unpack:
+        calls = [prepared("mhip_slice_unpack", w.data_ptr(), o.data_ptr(), C.byref(view.c), 2, STREAM()) for w, o in bufs]
+    else:
+        calls = [prepared("mhip_slice_pack", o.data_ptr(), w.data_ptr(), C.byref(view.c), 2, STREAM()) for w, o in bufs]
+
+    def launch(i):
+        return calls[i % sets]()
+
+    def cpu():
+        import oracle
+        h = bufs[0][0][:2048].cpu().view(torch.uint16).numpy().reshape(-1)
+        ov = oracle.OSlice(c0, [2048, cols], [pitch, 1])
+        t0 = time.perf_counter()
+        oracle.pack(h, ov)
+        dt = time.perf_counter() - t0
+        return {"value": nbytes / 8 / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "2048 of the 16384 rows through the per-element Slice::get walk"}
+
+    kernel = "slice_unpack_lines_kernel<4>" if unpack else "slice_copy_ragged_kernel<4>"
+    return ("ragged_column_block_unpack" if unpack else "ragged_column_block_pack"), nbytes, launch, cpu, kernel, "u8"
+
+
 def wl_c3_reshard(torch, sets=3, one_by_one=False):
     """Configuration 3 end to end (SendTensor / to_mesh of a column-sharded weight): the 8 column blocks are packed
     into 8 staging buffers in one launch, and the buffers are transferred into their receivers' contiguous tensors
@@ -747,6 +783,7 @@ WORKLOADS = {
     "c2_inplace_separate": lambda t: wl_c2(t, True, separate=True),
     "c2p_pack": lambda t: wl_c2p(t, False),
     "c2p_unpack": lambda t: wl_c2p(t, True),
+    "ragged_pack": lambda t: wl_ragged(t, False), "ragged_unpack": lambda t: wl_ragged(t, True),
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
     "c3_reshard_e2e": wl_c3_reshard,
@@ -954,7 +991,8 @@ def sweep_strided_views(dtypes, launches=20):
 # workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
 SUMMARY = {
     "c2": 0.75, "c2_inplace": 0.75, "c2_separate": 0.75, "c2_cold": 0.75, "c2p_pack": 0.75, "c2p_unpack": 0.75,
-    "c3_pack": 0.60, "c3_unpack": 0.60, "c3_reshard_e2e": 0.60, "c4": 0.60, "c4_slots": 0.60, "c4_cold": 0.60,
+    "c3_pack": 0.60, "c3_unpack": 0.60, "c3_reshard_e2e": 0.60, "ragged_pack": 0.60, "ragged_unpack": 0.60,
+    "c4": 0.60, "c4_slots": 0.60, "c4_cold": 0.60,
     "c5_flat_pack": 0.60, "c5_quantize": 0.60, "c5_dequant": 0.60, "c5_flat_unpack": 0.60,
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
