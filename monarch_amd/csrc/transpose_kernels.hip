@@ -522,6 +522,19 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
                (((uintptr_t)base | (uintptr_t)packed) & 511u) == 0;
     for (int k = 0; big && k < c.ndim; ++k)
         if (k != cd && c.dims[k].stride % 128 != 0) big = false;
+    // 2-byte elements get the 512-byte-row tile too (256 x 256 elements, 128 KiB of LDS, one workgroup per CU) where
+    // 256-byte runs do worst: matrices of 120 MiB and more whose rows are multiples of 16 KiB apart on both sides
+    // (every row of a tile then falls on the same position of HBM's address interleave, and a 512-byte run halves
+    // the number of pieces that meet there).  bf16, same GPU, both tiles in turn: 8192^2 pack / unpack 0.68 / 0.68 ->
+    // 0.71 / 0.735 of peak, 16384 x 8192 0.67 / 0.67 -> 0.70 / 0.745, 8192 x 16384 0.69 / 0.67 -> 0.75 / 0.77,
+    // 8 x 2048 x 8192 0.70 / 0.69 -> 0.73 / 0.74.  Smaller matrices lose with it (6144^2 0.80 -> 0.73, 4096 x 8192
+    // unpack 0.79 -> 0.70), other pitches gain or lose 0.01 (12288^2), so they keep the 128 x 128 tile.
+    if (unit == 2) {
+        big = Sc % 256 == 0 && Q % 8192 == 0 && c.offset % 256 == 0 && nbatch * Sc * Q * 2 >= (120ull << 20) &&
+              (((uintptr_t)base | (uintptr_t)packed) & 511u) == 0;
+        for (int k = 0; big && k < c.ndim; ++k)
+            if (k != cd && c.dims[k].stride % 8192 != 0) big = false;
+    }
     const uint32_t tile = vec ? (big ? 512 : 256) / unit : 32;
     a.base = base;
     a.packed = packed;
@@ -536,7 +549,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     // 16 0.65 of peak; 2-byte elements do best at 8.
     // 1-byte elements (256 x 256 tiles, two workgroups per CU) do best at 4: 8200^2 0.40 -> 0.47, 5000 x 7000 0.51 -> 0.57,
     // never lower than 8 on the shapes of the walk table.
-    a.group = big ? 8 : (unit == 4 || unit == 8) ? 16 : unit == 2 ? 8 : 4;
+    a.group = big ? (unit == 2 ? 4 : 8) : (unit == 4 || unit == 8) ? 16 : unit == 2 ? 8 : 4;
     a.cgroups = (a.ctiles + a.group - 1) / a.group;
     bool stream_loads = false;
     if (vec) {
@@ -582,7 +595,10 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
             if (stream_loads) {
                 switch (unit) {
                     case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a); break;
-                    case 2: MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a); break;
+                    case 2:
+                        if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 1024, PACK, 512, true>), grid, dim3(1024), 0, stream, a);
+                        else MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a);
+                        break;
                     case 4:
                         if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512, true>), grid, dim3(1024), 0, stream, a);
                         else MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a);
@@ -593,7 +609,10 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
             }
             switch (unit) {
                 case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
-                case 2: MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                case 2:
+                    if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a);
+                    else MHIP_LAUNCH((slice_transpose_vec_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a);
+                    break;
                 case 4:
                     if (big) MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 1024, PACK, 512>), grid, dim3(1024), 0, stream, a);
                     else MHIP_LAUNCH((slice_transpose_vec_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a);

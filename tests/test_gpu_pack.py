@@ -690,6 +690,23 @@ def test_transpose_large_aligned_bf16_tiles():
         assert torch.equal(back.view(torch.int16), x.view(torch.int16)), shape
 
 
+def test_transpose_bf16_matrices_of_120_mib_and_more_with_rows_16_kib_apart():
+    # the 256 x 256 tile form of two-byte elements, with and without a batch dimension and with more rows than columns
+    g = torch.Generator(device=DEV).manual_seed(16)
+    for shape in [(1, 8192, 8192), (2, 8192, 8192), (1, 16384, 8192)]:
+        x = torch.randint(-32768, 32767, shape, dtype=torch.int16, generator=g, device=DEV)
+        view = x.transpose(1, 2)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.view(view.shape), view.contiguous()), shape
+        back = torch.zeros_like(x)
+        staging.unpack(back, s, out)
+        sync()
+        assert torch.equal(back, x), shape
+        del x, view, out, back
+
+
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.float32, torch.float64])
 def test_transposes_whose_rows_are_a_multiple_of_8k_apart(dtype):
     # at these pitches the tile walk is rotated per eighth of the tiles; shapes with ragged edges, batches,
