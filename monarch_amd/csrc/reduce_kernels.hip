@@ -300,15 +300,23 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_kernel(ScatterA
             acc_t acc[V];
             VT::widen(load16_unaligned(static_cast<const char*>(a.in[0]) + loc * 16), acc);
             uint32_t g = 1;
-            for (; g + 7 <= a.n_in; g += 7) add_group<T, 7, MODE>(acc, a.in, g, loc, a.op);
-            switch (a.n_in - g) {  // wave-uniform: what is left after the groups of 7, its loads hoisted as well
-                case 6: add_group<T, 6, MODE>(acc, a.in, g, loc, a.op); break;
-                case 5: add_group<T, 5, MODE>(acc, a.in, g, loc, a.op); break;
-                case 4: add_group<T, 4, MODE>(acc, a.in, g, loc, a.op); break;
-                case 3: add_group<T, 3, MODE>(acc, a.in, g, loc, a.op); break;
-                case 2: add_group<T, 2, MODE>(acc, a.in, g, loc, a.op); break;
-                case 1: add_group<T, 1, MODE>(acc, a.in, g, loc, a.op); break;
-                default: break;
+            for (; g + 7 <= a.n_in; g += 7) {
+                uint4 raw[7];
+#pragma unroll
+                for (int j = 0; j < 7; ++j) raw[j] = load16_unaligned(static_cast<const char*>(a.in[g + j]) + loc * 16);
+#pragma unroll
+                for (int j = 0; j < 7; ++j) {
+                    acc_t x[V];
+                    VT::widen(raw[j], x);
+#pragma unroll
+                    for (int e = 0; e < V; ++e) acc[e] = combine<MODE>(acc[e], x[e], a.op);
+                }
+            }
+            for (; g < a.n_in; ++g) {
+                acc_t x[V];
+                VT::widen(load16_unaligned(static_cast<const char*>(a.in[g]) + loc * 16), x);
+#pragma unroll
+                for (int e = 0; e < V; ++e) acc[e] = combine<MODE>(acc[e], x[e], a.op);
             }
 #pragma unroll
             for (int e = 0; e < V; ++e) acc[e] = finish(acc[e], MODE == kAvg, a.scale, a.divisor);
