@@ -202,9 +202,9 @@ def test_reduce_over_staging_area_slots():
 
 @pytest.mark.parametrize("numel", [1, 1023, 128 * 8 * 8 * 3, 128 * 8 * 61 + 777, 1_000_003])
 def test_reduce_both_block_mappings(numel):
-    # inputs that share a 16 KiB phase take the XCD-contiguous block mapping, inputs at different
-    # phases the plain one; both must cover every element exactly once, for grids that are and
-    # are not a multiple of 8 workgroups
+    # inputs that share a 16 KiB phase take the rotated block mapping (workgroup i takes chunk i + i / 8 of its
+    # group of 8), inputs at different phases the plain one; both must cover every element exactly once, for
+    # grids that are and are not a multiple of 8 workgroups
     n = 8
     hosts = [_rand(torch.float32, numel, 900 + r) for r in range(n)]
     want = oracle.reduce([h.numpy() for h in hosts], SUM)
