@@ -316,18 +316,18 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
                 // Half the LDS instructions of the element-wise form, and no sub-dword accesses.
 #pragma unroll
                 for (int p = 0; p < PASSES / 2; ++p) {
-                    const int c = 2 * (r16 + ROWS * p);
+                    const int c = 2 * (cc0 + CSTEP * p);
                     uint32_t w[E];
 #pragma unroll
-                    for (int j = 0; j < E; ++j) w[j] = *reinterpret_cast<const uint32_t*>(&tile[at(v16 * E + j, c)]);
+                    for (int j = 0; j < E; ++j) w[j] = *reinterpret_cast<const uint32_t*>(&tile[at(qv * E + j, c)]);
                     u32x4 lo, hi;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         lo[k] = (w[2 * k] & 0xffffu) | (w[2 * k + 1] << 16);
                         hi[k] = (w[2 * k] >> 16) | (w[2 * k + 1] & 0xffff0000u);
                     }
-                    tstore(packed_tile + (uint64_t)c * a.Q + v16 * E, lo, a.aligned_stores);
-                    tstore(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E, hi, a.aligned_stores);
+                    tstore(packed_tile + (uint64_t)c * a.Q + qv * E, lo, a.aligned_stores);
+                    tstore(packed_tile + (uint64_t)(c + 1) * a.Q + qv * E, hi, a.aligned_stores);
                 }
             } else {
 #pragma unroll
@@ -345,20 +345,20 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
                 // halves interleaved into eight 32-bit LDS writes
 #pragma unroll
                 for (int p = 0; p < PASSES / 2; ++p) {
-                    const int c = 2 * (r16 + ROWS * p);
-                    d[2 * p].v = tload<STREAM>(packed_tile + (uint64_t)c * a.Q + v16 * E);
-                    d[2 * p + 1].v = tload<STREAM>(packed_tile + (uint64_t)(c + 1) * a.Q + v16 * E);
+                    const int c = 2 * (cc0 + CSTEP * p);
+                    d[2 * p].v = tload<STREAM>(packed_tile + (uint64_t)c * a.Q + qv * E);
+                    d[2 * p + 1].v = tload<STREAM>(packed_tile + (uint64_t)(c + 1) * a.Q + qv * E);
                 }
 #pragma unroll
                 for (int p = 0; p < PASSES / 2; ++p) {
-                    const int c = 2 * (r16 + ROWS * p);
+                    const int c = 2 * (cc0 + CSTEP * p);
                     const u32x4 lo = d[2 * p].v, hi = d[2 * p + 1].v;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         const uint32_t w0 = (lo[k] & 0xffffu) | (hi[k] << 16);
                         const uint32_t w1 = (lo[k] >> 16) | (hi[k] & 0xffff0000u);
-                        *reinterpret_cast<uint32_t*>(&tile[at(v16 * E + 2 * k, c)]) = w0;
-                        *reinterpret_cast<uint32_t*>(&tile[at(v16 * E + 2 * k + 1, c)]) = w1;
+                        *reinterpret_cast<uint32_t*>(&tile[at(qv * E + 2 * k, c)]) = w0;
+                        *reinterpret_cast<uint32_t*>(&tile[at(qv * E + 2 * k + 1, c)]) = w1;
                     }
                 }
             } else {
