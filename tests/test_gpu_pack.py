@@ -690,6 +690,24 @@ def test_transpose_large_aligned_bf16_tiles():
         assert torch.equal(back.view(torch.int16), x.view(torch.int16)), shape
 
 
+def test_transpose_large_aligned_f64_tiles():
+    # 2^24 and more eight-byte elements with 512-byte aligned rows: the 64 x 64 tile form with 512 lanes (a row
+    # length of 4096 or less) and with 1024 lanes, with a batch dimension
+    g = torch.Generator(device=DEV).manual_seed(17)
+    for shape in [(1, 4096, 4096), (2, 4096, 2048), (1, 4160, 8192 + 64)]:
+        x = torch.randint(-2**62, 2**62, shape, dtype=torch.int64, generator=g, device=DEV)
+        view = x.transpose(1, 2)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.view(view.shape), view.contiguous()), shape
+        back = torch.zeros_like(x)
+        staging.unpack(back, s, out)
+        sync()
+        assert torch.equal(back, x), shape
+        del x, view, out, back
+
+
 def test_transpose_bf16_matrices_of_120_mib_and_more_with_rows_16_kib_apart():
     # the 256 x 256 tile form of two-byte elements, with and without a batch dimension and with more rows than columns
     g = torch.Generator(device=DEV).manual_seed(16)
