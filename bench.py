@@ -842,7 +842,7 @@ SWEEP_HEADERS = {
 further on); `packed fastest` / `memory fastest`: plain row-major walks; `diagonal`: consecutive workgroups step one
 tile along both axes.  The selection rule (`choose_walk` in `monarch_amd/csrc/transpose_kernels.hip`): 1/2/4-byte
 elements whose row pitches are multiples of 4 KiB on both sides take the diagonal walk, everything else the blocked
-walk (block 4 for 1-byte, 8 for 2-byte, 16 for 4/8-byte elements; 8 with the 512-byte-row tile of fp32).  Every walk
+walk (block 4 for 1-byte, 8 for 2-byte, 16 for 4/8-byte elements; 8 with the 512-byte-row tiles of 4- and 8-byte elements, 4 with that of 2-byte elements).  Every walk
 runs with the cache policy the library picks for the element size.""",
     "transpose_policies": "# Transposing pack / unpack: A/B of the cache policies of its loads and stores (MI355X)\n\n"
     + _SWEEP_COMMON.format(which="transpose_policies", file="transpose_cache_policy_ab.md") + """\
