@@ -178,6 +178,56 @@ __global__ __launch_bounds__(kThreads) void slice_transpose_kernel(TransArgs a) 
     }
 }
 
+// The tile (batch b, q-tile qt, c-tile ct) this workgroup takes, in the order the host chose (see choose_walk); false when
+// the workgroup is padding of the walk.  Uniform over the workgroup.
+__device__ __forceinline__ bool walk_tile(const TransArgs& a, uint64_t* b_out, uint32_t* qt_out, uint32_t* ct_out) {
+    const uint64_t per_batch = (uint64_t)a.cgroups * ((a.qtiles + a.group - 1) / a.group) * a.group * a.group;
+
+    // workgroup w runs on XCD w % 8
+    const uint64_t per_xcd = (a.ntiles + 7) / 8;
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t tile_id = a.xcd_ranges ? (wg % 8) * per_xcd + wg / 8 : wg;
+    if (tile_id >= a.ntiles) return false;
+
+    uint64_t b;
+    uint32_t qt, ct;
+    if (a.walk == kWalkBlocked) {
+        b = tile_id / per_batch;
+        const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
+        const uint32_t gsz = a.group * a.group;
+        const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
+        const uint32_t gq = grp / a.cgroups;
+        uint32_t gc = grp - gq * a.cgroups;
+        if (a.rotate) {
+            // a function of the row of groups alone, so that every row still visits each of its c-groups once
+            const uint32_t eighth = (uint32_t)((b * a.qgroups + gq) / a.rows_per_eighth);  // 0..7: the XCD, when ranges hold whole rows
+            gc = (gc + eighth * a.cgroups / 8) % a.cgroups;
+        }
+        qt = gq * a.group + within / a.group;
+        ct = gc * a.group + within % a.group;
+        if (qt >= a.qtiles || ct >= a.ctiles) return false;  // padding of the blocked walk (uniform per workgroup)
+    } else {
+        const uint64_t plain = (uint64_t)a.qtiles * a.ctiles;
+        b = tile_id / plain;
+        const uint32_t t = (uint32_t)(tile_id - b * plain);
+        if (a.walk == kWalkPackedFastest) {          // neighbours write neighbouring pieces of the same packed rows
+            ct = t / a.qtiles;
+            qt = t - ct * a.qtiles;
+        } else if (a.walk == kWalkMemoryFastest) {   // neighbours read neighbouring pieces of the same memory rows
+            qt = t / a.ctiles;
+            ct = t - qt * a.ctiles;
+        } else {                                     // kWalkDiagonal: neighbours differ in both coordinates
+            const uint32_t d = t / a.qtiles;
+            qt = t - d * a.qtiles;
+            ct = (d + qt) % a.ctiles;
+        }
+    }
+    *b_out = b;
+    *qt_out = qt;
+    *ct_out = ct;
+    return true;
+}
+
 // ---- 16-byte-per-lane variant for elements of 1, 2, 4 and 8 bytes ----
 // A tile is TQ x TC elements with TQ * sizeof(T) == TC * sizeof(T) == 256 bytes, so that every
 // row of the tile is a 256-byte run on BOTH HBM sides and every lane moves 16 bytes
@@ -211,47 +261,9 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 
     T* __restrict__ mem = reinterpret_cast<T*>(a.base) + a.offset;
     T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
-    const uint64_t per_batch = (uint64_t)a.cgroups * ((a.qtiles + a.group - 1) / a.group) * a.group * a.group;
-
-    // workgroup w runs on XCD w % 8
-    const uint64_t per_xcd = (a.ntiles + 7) / 8;
-    const uint64_t wg = a.wg0 + blockIdx.x;
-    const uint64_t tile_id = a.xcd_ranges ? (wg % 8) * per_xcd + wg / 8 : wg;
-    if (tile_id >= a.ntiles) return;
-
     uint64_t b;
     uint32_t qt, ct;
-    if (a.walk == kWalkBlocked) {
-        b = tile_id / per_batch;
-        const uint32_t in_batch = (uint32_t)(tile_id - b * per_batch);
-        const uint32_t gsz = a.group * a.group;
-        const uint32_t grp = in_batch / gsz, within = in_batch - grp * gsz;
-        const uint32_t gq = grp / a.cgroups;
-        uint32_t gc = grp - gq * a.cgroups;
-        if (a.rotate) {
-            // a function of the row of groups alone, so that every row still visits each of its c-groups once
-            const uint32_t eighth = (uint32_t)((b * a.qgroups + gq) / a.rows_per_eighth);  // 0..7: the XCD, when ranges hold whole rows
-            gc = (gc + eighth * a.cgroups / 8) % a.cgroups;
-        }
-        qt = gq * a.group + within / a.group;
-        ct = gc * a.group + within % a.group;
-        if (qt >= a.qtiles || ct >= a.ctiles) return;  // padding of the blocked walk (uniform per workgroup)
-    } else {
-        const uint64_t plain = (uint64_t)a.qtiles * a.ctiles;
-        b = tile_id / plain;
-        const uint32_t t = (uint32_t)(tile_id - b * plain);
-        if (a.walk == kWalkPackedFastest) {          // neighbours write neighbouring pieces of the same packed rows
-            ct = t / a.qtiles;
-            qt = t - ct * a.qtiles;
-        } else if (a.walk == kWalkMemoryFastest) {   // neighbours read neighbouring pieces of the same memory rows
-            qt = t / a.ctiles;
-            ct = t - qt * a.ctiles;
-        } else {                                     // kWalkDiagonal: neighbours differ in both coordinates
-            const uint32_t d = t / a.qtiles;
-            qt = t - d * a.qtiles;
-            ct = (d + qt) % a.ctiles;
-        }
-    }
+    if (!walk_tile(a, &b, &qt, &ct)) return;
     // A tile that would hang over the edge is moved back inside when the extent allows it: it
     // then overlaps its neighbour, and both write the same bytes to the overlap.
     uint32_t q0 = qt * TQ, c0 = ct * TC;
@@ -432,6 +444,122 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
     }
 }
 
+// ---- the same tile when the rows of the side that is WRITTEN do not start on cache lines ----
+// With 256-byte tile rows cut at fixed element positions, a written row piece that starts inside a 128-byte line shares
+// its first and last line with the neighbouring tiles, and such a line reaches HBM as two partial writes (bf16 8200^2:
+// 0.42 of peak against 0.68 at 8064^2, whose rows are whole lines).  Here every written row gets its own window of the
+// tile's TX positions, moved back by d_w < 128 / sizeof(T) elements so that it starts on a line: the windows of one row
+// still tile the row (256 bytes are two lines, so d_w is the same in every tile), every vector store is aligned and
+// every line is written whole by one workgroup, except at the two ends of a row.  The windows of a tile's rows start
+// at different places, so the tile reads up to D more rows of the other side than it writes positions: TX + D rows go
+// through LDS (the same XOR-permuted layout), the surplus coming out of L2, where the neighbouring tile has just put it.
+// Both kernels in turn on one GPU, pack / unpack: bf16 8200^2 0.42 / 0.42 -> 0.58 / 0.585 of peak, 5000 x 7000
+// 0.53 / 0.55 -> 0.69 / 0.70; fp32 0.53 / 0.54 -> 0.65 / 0.645 and 0.46 / 0.46 -> 0.61 / 0.60; f64 0.64 / 0.63 ->
+// 0.67 / 0.67 and 0.60 / 0.58 -> 0.63 / 0.62.  Rows that do start on lines keep the kernel above.
+// W is the index of a written row (c when packing, q when unpacking), X the position along it.
+template <typename T, int THREADS, bool PACK>
+__global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArgs a) {
+    constexpr int ES = sizeof(T), E = 16 / ES;
+    constexpr int TW = 256 / ES, TX = 256 / ES, D = 128 / ES, XR = TX + D;
+    constexpr int ROWS = THREADS / 16;
+    static_assert(XR <= THREADS && TW <= THREADS, "one lane per decoded row");
+    __shared__ __attribute__((aligned(16))) T tile[XR * TW];  // [read row][written row]
+    __shared__ uint64_t s_off[PACK ? XR : TW];
+    union Vec {
+        u32x4 v;
+        T e[E];
+    };
+    auto at = [](int xr, int wc) { return xr * TW + (wc ^ (E * ((xr / E) % 16))); };
+
+    uint64_t b;
+    uint32_t qt, ct;
+    if (!walk_tile(a, &b, &qt, &ct)) return;
+    const uint32_t Wn = PACK ? a.Sc : a.Q, Xn = PACK ? a.Q : a.Sc;
+    uint32_t w0 = (PACK ? ct : qt) * TW;
+    if (w0 + TW > Wn) w0 = Wn - TW;  // the host sends extents of at least a tile; the overlap is written twice, same bytes
+    const int64_t x0 = (int64_t)(PACK ? qt : ct) * TX;
+
+    T* __restrict__ mem = reinterpret_cast<T*>(a.base) + a.offset;
+    T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
+    uint64_t batch_off = 0;
+    {
+        uint64_t rem = b;
+        for (int k = a.n_outer - 1; k >= 0; --k) {
+            const uint64_t qd = rem / a.outer_size[k];
+            batch_off += (rem - qd * a.outer_size[k]) * a.outer_stride[k];
+            rem = qd;
+        }
+    }
+    // memory offsets of the q rows this tile touches: the read rows when packing (clamped into the extent: what a
+    // clamped row holds is never written), the written rows when unpacking
+    if (threadIdx.x < (PACK ? XR : TW)) {
+        int64_t qi = PACK ? x0 - D + (int64_t)threadIdx.x : (int64_t)w0 + threadIdx.x;
+        if (qi < 0) qi = 0;
+        if (qi > (int64_t)a.Q - 1) qi = (int64_t)a.Q - 1;
+        uint32_t q = (uint32_t)qi;
+        uint64_t off = 0;
+        for (int k = a.n_inner - 1; k > 0; --k) {
+            uint32_t qd, r;
+            a.inner_div[k].divmod(q, qd, r);
+            off += (uint64_t)r * a.inner_stride[k];
+            q = qd;
+        }
+        off += (uint64_t)q * a.inner_stride[0];
+        s_off[threadIdx.x] = off;
+    }
+    __syncthreads();
+
+    // ---- read side -> LDS: rows x0 - D .. x0 + TX - 1, TW consecutive written-row indices of each ----
+    const int v16 = threadIdx.x % 16, r16 = threadIdx.x / 16;
+    constexpr int LPASSES = (XR + ROWS - 1) / ROWS;
+    Vec d[LPASSES];
+#pragma unroll
+    for (int p = 0; p < LPASSES; ++p) {
+        int xr = r16 + ROWS * p;
+        if (xr > XR - 1) xr = XR - 1;  // surplus lanes of the last pass repeat its last row
+        const T* src;
+        if constexpr (PACK) {
+            src = mem + batch_off + s_off[xr] + w0 + v16 * E;
+        } else {
+            int64_t c = x0 - D + xr;
+            if (c < 0) c = 0;
+            if (c > (int64_t)a.Sc - 1) c = (int64_t)a.Sc - 1;
+            src = packed + (b * a.Sc + (uint64_t)c) * (uint64_t)a.Q + w0 + v16 * E;
+        }
+        d[p].v = tload<false>(src);
+    }
+#pragma unroll
+    for (int p = 0; p < LPASSES; ++p) {
+        const int xr = r16 + ROWS * p;
+        if (xr < XR) *reinterpret_cast<u32x4*>(&tile[xr * TW + E * (v16 ^ ((xr / E) % 16))]) = d[p].v;
+    }
+    __syncthreads();
+
+    // ---- LDS -> written side: row w takes positions x0 - d_w .. x0 - d_w + TX - 1, a window that starts on a line ----
+    constexpr int WPASSES = TW / ROWS;
+    static_assert(TW % ROWS == 0, "whole passes");
+#pragma unroll
+    for (int p = 0; p < WPASSES; ++p) {
+        const int wr = r16 + ROWS * p;
+        T* row;  // position 0 of the written row
+        if constexpr (PACK) row = packed + (b * a.Sc + w0 + wr) * (uint64_t)a.Q;
+        else row = mem + batch_off + s_off[wr];
+        const int dw = (int)((((uintptr_t)row + (uint64_t)x0 * ES) & 127u) / ES);
+        const int64_t xs = x0 - dw + v16 * E;  // first position of this lane's vector
+        const int xr0 = D - dw + v16 * E;      // and the LDS row that holds it
+        Vec o;
+#pragma unroll
+        for (int j = 0; j < E; ++j) o.e[j] = tile[at(xr0 + j, wr)];
+        if (xs >= 0 && xs + E <= (int64_t)Xn) {
+            tstore(row + xs, o.v, kStoreStreaming);
+        } else {
+#pragma unroll
+            for (int j = 0; j < E; ++j)
+                if (xs + j >= 0 && xs + j < (int64_t)Xn) row[xs + j] = o.e[j];
+        }
+    }
+}
+
 // Cache policy of a launch, from an A/B over sixteen shapes, both directions and four element sizes (fractions of the
 // HBM peak; "cached" = plain loads, write-through stores on aligned rows; the table is
 // profiles/transpose_cache_policy_ab.md):
@@ -562,13 +690,26 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         }
     }
     const uint32_t tile = vec ? (big ? 512 : 256) / unit : 32;
+    // Written rows that do not start on cache lines take the kernel whose windows do (slice_transpose_lines_kernel):
+    // the extent along the written rows grows by the most a window can start early.
+    // MONARCH_HIP_TRANSPOSE_LINES=0 / 1 overrides the choice (a tuning aid, read at every call).
+    bool lines = false;
+    if (vec && !big && unit >= 2 && (PACK ? Sc : Q) >= tile) {  // 1-byte elements lose with it (8200^2 0.475 -> 0.36: 96 KiB of LDS, byte-wise LDS reads)
+        uint64_t written = PACK ? ((uint64_t)(uintptr_t)packed | Q * unit) : ((uint64_t)(uintptr_t)base + c.offset * unit);
+        if (!PACK)
+            for (int k = 0; k < c.ndim; ++k)
+                if (k != cd) written |= c.dims[k].stride * unit;
+        lines = (written & 127u) != 0;
+        if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_LINES")) lines = std::atoi(e) != 0;
+    }
+    const uint32_t early = lines ? 128 / unit - 1 : 0;
     a.base = base;
     a.packed = packed;
     a.offset = c.offset;
     a.Sc = (uint32_t)Sc;
     a.Q = (uint32_t)Q;
-    a.ctiles = (uint32_t)((Sc + tile - 1) / tile);
-    a.qtiles = (uint32_t)((Q + tile - 1) / tile);
+    a.ctiles = (uint32_t)((Sc + (PACK ? 0 : early) + tile - 1) / tile);
+    a.qtiles = (uint32_t)((Q + (PACK ? early : 0) + tile - 1) / tile);
     // Tiles are walked in group x group blocks, and a block is about what one XCD runs at a time
     // (8 workgroups per CU of 4-byte tiles, 4 of 2-byte tiles), so that the eight XCDs each stream
     // runs of group * 256 bytes on both sides.  Measured at 8192^2 fp32 pack: group 1 0.47, 4 0.52,
@@ -618,6 +759,15 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         *rc = launch_in_pieces(nblocks, lanes, 8, [&](uint64_t wg0, uint32_t count) {
             a.wg0 = wg0;
             const dim3 grid(count);
+            if (lines) {
+                switch (unit) {
+                    case 1: MHIP_LAUNCH((slice_transpose_lines_kernel<uint8_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                    case 2: MHIP_LAUNCH((slice_transpose_lines_kernel<uint16_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                    case 4: MHIP_LAUNCH((slice_transpose_lines_kernel<uint32_t, 512, PACK>), grid, dim3(512), 0, stream, a); break;
+                    default: MHIP_LAUNCH((slice_transpose_lines_kernel<uint64_t, 256, PACK>), grid, dim3(256), 0, stream, a); break;
+                }
+                return;
+            }
             if (stream_loads) {
                 switch (unit) {
                     case 1: MHIP_LAUNCH((slice_transpose_vec_kernel<uint8_t, 512, PACK, 256, true>), grid, dim3(512), 0, stream, a); break;

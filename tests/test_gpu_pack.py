@@ -645,6 +645,35 @@ def test_transposing_views_interior_and_edge_tiles(dtype):
         assert torch.equal(back.cpu(), ref), (shape, dtype)
 
 
+@pytest.mark.parametrize("lines", ["0", "1"])
+@pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+def test_transposes_with_line_aligned_windows_and_without(dtype, lines, monkeypatch):
+    # written rows that start anywhere in a cache line, through the kernel whose windows start on lines and through
+    # the fixed-position tiles: extents of exactly one tile, of a tile and a bit, shorter than the early start of a
+    # window, batches, offsets, a packed side spanning two dimensions
+    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_LINES", lines)
+    g = torch.Generator().manual_seed(18)
+    info = torch.iinfo(dtype)
+    t = 256 // torch.empty(0, dtype=dtype).element_size()
+    cases = [((t, t + 1), lambda x: x.t()), ((t + 3, t), lambda x: x.t()), ((2 * t + 5, 3 * t + 7), lambda x: x[1:, 2:].t()),
+             ((7, t + 9), lambda x: x.t()), ((t + 9, 7), lambda x: x.t()), ((3, t + 2, t + 1), lambda x: x.transpose(1, 2)),
+             ((2, t + 1, 2, 300 // (t // 32 + 1) + t), lambda x: x.permute(0, 3, 2, 1)[:, 1:]), ((1100, 1031), lambda x: x[:, 5:].t())]
+    for shape, view_of in cases:
+        host = torch.randint(info.min, info.max, shape, dtype=dtype, generator=g)
+        dev = host.to(DEV)
+        view, hview = view_of(dev), view_of(host)
+        s = Slice.of_tensor(view)
+        out = staging.pack(view, s)
+        sync()
+        assert torch.equal(out.cpu(), hview.contiguous().flatten()), (shape, dtype)
+        back = torch.full_like(dev, 7)
+        staging.unpack(back, s, out)
+        sync()
+        ref = torch.full_like(host, 7)
+        view_of(ref).copy_(hview)
+        assert torch.equal(back.cpu(), ref), (shape, dtype)
+
+
 def test_transpose_large_square():
     g = torch.Generator(device=DEV).manual_seed(12)
     x = (torch.randn(4096, 4096, generator=g, device=DEV)).bfloat16()
