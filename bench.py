@@ -833,7 +833,8 @@ Every cell is the fraction of the 8 TB/s HBM peak that `mhip_slice_pack` / `mhip
 view (`x[:, :, :cols].transpose(1, 2)` of a `[batch, rows, pitch]` tensor; algorithmic bytes = 2 x elements x element
 size) with one variant forced through `{{envvar}}`; `library` is what the host code picks by itself.  All variants of a
 row are switched in turn inside one process on one GPU: medians of {{reps}} alternations of {{launches}} launches, 3 rotating
-buffer sets.  Matrices of 4096 x 4096 and smaller partly live in the 256 MB Infinity Cache across the three buffer sets.
+buffer sets.  Matrices of 4096 x 4096 and smaller partly live in the 256 MB Infinity Cache across the three buffer sets.  Shapes whose written rows do not start on cache lines (8200 x 8200, 5000 x 7000) run the kernel with
+line-aligned windows for 2-, 4- and 8-byte elements, under every variant of this table.
 """
 SWEEP_HEADERS = {
     "transpose_walks": "# Transposing pack / unpack: A/B of the tile walks (MI355X)\n\n"
