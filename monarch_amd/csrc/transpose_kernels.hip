@@ -455,7 +455,8 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_vec_kernel(TransArgs 
 // through LDS (the same XOR-permuted layout), the surplus coming out of L2, where the neighbouring tile has just put it.
 // Both kernels in turn on one GPU, pack / unpack: bf16 8200^2 0.42 / 0.42 -> 0.58 / 0.585 of peak, 5000 x 7000
 // 0.53 / 0.55 -> 0.69 / 0.70; fp32 0.53 / 0.54 -> 0.65 / 0.645 and 0.46 / 0.46 -> 0.61 / 0.60; f64 0.64 / 0.63 ->
-// 0.67 / 0.67 and 0.60 / 0.58 -> 0.63 / 0.62.  Rows that do start on lines keep the kernel above.
+// 0.67 / 0.67 and 0.60 / 0.58 -> 0.63 / 0.62.  Rows that do start on lines keep the kernel above.  Loads go through
+// the cache at every size: streaming (nt) loads lose what the neighbouring tile left in L2 (bf16 5000 x 7000 0.70 -> 0.49).
 // W is the index of a written row (c when packing, q when unpacking), X the position along it.
 template <typename T, int THREADS, bool PACK>
 __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArgs a) {
