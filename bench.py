@@ -521,9 +521,9 @@ def wl_stack(torch, scatter=False, sets=None):
     return ("stack_scatter_bf16_8" if scatter else "stack_bf16_8"), nbytes, launch, cpu, "copy_many_kernel", "u8"
 
 
-def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
+def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3, n=None):
     from monarch_amd import Slice, staging
-    n = int(os.environ.get("MONARCH_BENCH_TRANSPOSE_N", "8192"))
+    n = n or int(os.environ.get("MONARCH_BENCH_TRANSPOSE_N", "8192"))
     dt = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
     g = torch.Generator(device="cuda:0").manual_seed(6000)
     s = Slice(offset=0, sizes=[n, n], strides=[1, n])  # iterate columns first: packs x.T
@@ -552,7 +552,8 @@ def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3):
                 "sample": f"{m}x{m} corner through the per-element Slice::get walk, scaled to {n}x{n}"}
 
     name = f"transpose_{dtype_name}_{n}x{n}_" + ("unpack" if unpack else "pack")
-    return name, nbytes, launch, cpu, "slice_transpose_vec_kernel", "u8"
+    kernel = "slice_transpose_vec_kernel" if n * es % 128 == 0 else "slice_transpose_lines_kernel"
+    return name, nbytes, launch, cpu, kernel, "u8"
 
 
 def wl_c4(torch, sets=2, slots=False):
@@ -796,6 +797,9 @@ WORKLOADS = {
     "tr_f32_unpack": lambda t: wl_transpose(t, "f32", True),
     "tr_bf16_pack": lambda t: wl_transpose(t, "bf16", False),
     "tr_bf16_unpack": lambda t: wl_transpose(t, "bf16", True),
+    # rows of 16400 bytes: no written row starts on a cache line
+    "tr_bf16_8200_pack": lambda t: wl_transpose(t, "bf16", False, n=8200),
+    "tr_bf16_8200_unpack": lambda t: wl_transpose(t, "bf16", True, n=8200),
     "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
     "c5_quantize": lambda t: wl_c5(t, "quantize"),
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
@@ -998,6 +1002,7 @@ SUMMARY = {
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
     "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
+    "tr_bf16_8200_pack": None, "tr_bf16_8200_unpack": None,
     # configuration 1 (1 MiB views): launch-bound, reported as time per call
     "c1_pack": None, "c1_unpack": None, "c1_reduce": None, "c1_pipeline": None, "c1_pipeline_fused": None,
 }

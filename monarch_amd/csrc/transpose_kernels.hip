@@ -541,7 +541,13 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
     static_assert(TW % ROWS == 0, "whole passes");
 #pragma unroll
     for (int p = 0; p < WPASSES; ++p) {
-        const int wr = r16 + ROWS * p;
+        // The four written rows of a wavefront take elements that sit in four different 32-bit words of one 16-byte
+        // group: each row reads its own LDS rows (its window starts at its own place), so rows whose elements share
+        // a word would meet in one bank at different addresses.
+        constexpr int S = ES >= 4 ? 1 : 4 / ES;
+        const int logical = r16 + ROWS * p;
+        const int in_block = logical % (4 * S);
+        const int wr = logical - in_block + (in_block % 4) * S + in_block / 4;
         T* row;  // position 0 of the written row
         if constexpr (PACK) row = packed + (b * a.Sc + w0 + wr) * (uint64_t)a.Q;
         else row = mem + batch_off + s_off[wr];
