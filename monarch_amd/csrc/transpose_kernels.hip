@@ -470,7 +470,7 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
         u32x4 v;
         T e[E];
     };
-    auto at = [](int xr, int wc) { return xr * TW + (wc ^ (E * ((xr / E) % 16))); };
+    // LDS position of (read row xr, written row wc): xr * TW + (wc ^ (E * ((xr / E) % 16)))
 
     uint64_t b;
     uint32_t qt, ct;
@@ -554,9 +554,16 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
         const int dw = (int)((((uintptr_t)row + (uint64_t)x0 * ES) & 127u) / ES);
         const int64_t xs = x0 - dw + v16 * E;  // first position of this lane's vector
         const int xr0 = D - dw + v16 * E;      // and the LDS row that holds it
+        // The E rows xr0 .. xr0 + E - 1 lie in at most two groups of E rows, i.e. see two XOR permutations: one base
+        // address for each, and a compare per element instead of the permutation's arithmetic (which is what made the
+        // kernel ALU-bound for narrow elements: 8 or 16 elements per vector).
+        const int first = E - xr0 % E;         // elements in the first group
+        const int k0 = (xr0 / E) % 16, k1 = (xr0 / E + 1) % 16;
+        const T* __restrict__ p0 = tile + xr0 * TW + (wr ^ (E * k0));
+        const T* __restrict__ p1 = tile + xr0 * TW + (wr ^ (E * k1));
         Vec o;
 #pragma unroll
-        for (int j = 0; j < E; ++j) o.e[j] = tile[at(xr0 + j, wr)];
+        for (int j = 0; j < E; ++j) o.e[j] = (j < first ? p0 : p1)[j * TW];
         if (xs >= 0 && xs + E <= (int64_t)Xn) {
             tstore(row + xs, o.v, kStoreStreaming);
         } else {
