@@ -148,3 +148,61 @@ def test_memset_every_alignment_and_in_a_graph():
         want = ((torch.zeros(n) + hosts[0]) + hosts[1]) + hosts[2]
         assert torch.equal(acc.cpu(), want), rep
         assert torch.isfinite(junk)
+
+
+def test_strided_copy_forms_replay():
+    # the forms whose launch geometry the host derives from addresses (XCD shares, line-by-line unpack, units on a
+    # skewed base, line-aligned transposing windows) recorded once and replayed on new data
+    g = torch.Generator(device=DEV).manual_seed(9)
+    cases = [(torch.int16, (300, 4096), lambda x: x[:, 1:3581]),          # ragged rows of 7160 bytes at an odd column
+             (torch.int16, (300, 4096), lambda x: x[:, 1:3585]),          # whole chunks from a skewed base
+             (torch.int32, (257, 1031), lambda x: x[:, 3:].t()),          # transposing, written rows off the cache lines
+             (torch.uint8, (600, 1000), lambda x: x[5:, 7:900])]          # one-byte units
+    views, outs, backs, xs = [], [], [], []
+    for dt, shape, view_of in cases:
+        x = torch.zeros(shape, dtype=dt, device=DEV)
+        v = view_of(x)
+        xs.append(x)
+        views.append((v, Slice.of_tensor(v), view_of))
+        outs.append(torch.empty(v.numel(), dtype=dt, device=DEV))
+        backs.append(torch.zeros_like(x))
+
+    def pipeline():
+        for (v, s, _), o, b in zip(views, outs, backs):
+            staging.pack(v, s, out=o)
+            staging.unpack(b, s, o)
+
+    def fill():
+        for x in xs:
+            info = torch.iinfo(x.dtype)
+            x.copy_(torch.randint(info.min, info.max, x.shape, dtype=x.dtype, generator=g, device=DEV))
+
+    def check(tag):
+        for (v, s, view_of), o, b, x in zip(views, outs, backs, xs):
+            assert torch.equal(o.view(v.shape), v.contiguous()), tag
+            want = torch.zeros_like(x)
+            view_of(want).copy_(v)
+            assert torch.equal(b, want), tag
+
+    fill()
+    pipeline()
+    sync()
+    check("eager")
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        pipeline()
+    torch.cuda.current_stream().wait_stream(side)
+    sync()
+    with torch.cuda.graph(graph, stream=side):
+        pipeline()
+    for rep in range(3):
+        fill()
+        for b in backs:
+            b.zero_()
+        scratch = torch.randn(1 << 20, device=DEV).sum()  # unrelated eager work between replays
+        graph.replay()
+        sync()
+        check(rep)
+        assert torch.isfinite(scratch)
