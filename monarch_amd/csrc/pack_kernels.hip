@@ -43,7 +43,8 @@ struct PackArgs {
     uint64_t nrows;              //   rows per view
     uint64_t per_xcd;            // copies whose pieces share cache lines: workgroups in each XCD's contiguous
     uint64_t nwg;                //   share of the nwg workgroups (0: workgroup i takes tile i)
-    uint32_t stream_stores;      // slice_copy_kernel unpacking 16-byte units: non-temporal instead of write-through stores
+    uint32_t stream_stores;      // slice_copy_kernel unpacking 16-byte units, slice_unpack_lines_kernel: non-temporal
+                                 //   instead of write-through stores
     DimsArg dims;
 };
 
@@ -295,6 +296,10 @@ __global__ __launch_bounds__(kPackThreads) void slice_copy_ragged_kernel(PackArg
 // 1790 0.58 -> 0.62, of 3580 0.66 -> 0.70; u8 rows of 3581 0.51 -> 0.60, of 14333 0.645 -> 0.75; fp32 rows of 447
 // 0.36 -> 0.42, of 1791 0.67 -> 0.71.  (A form with one 1 KiB-aligned piece of one row per wavefront, which this one
 // replaces, gave 0.59 / 0.66 on bf16 rows of 1790 / 3580 and lost on rows around 1 KiB, whose pieces are half empty.)
+// Launches that write less than 96 MiB store write-through, cut vectors included, as the whole-chunk form does at those
+// sizes (u8 rows of 1788 0.41-0.44 -> 0.54-0.58, of 3580 0.59-0.63 -> 0.66-0.80, 82 MB 0.64 -> 0.76; eight bf16 column
+// blocks of 1790 in one launch, 59 MB together, 0.70 -> 0.76); larger ones stream (117 MB in eight views 0.72 against
+// 0.70 write-through, one view of 117 MB 0.71 against 0.66, of 235 MB 0.76 against 0.66).
 template <int U, bool WIDE, int NDIM>
 __global__ __launch_bounds__(kPackThreads) void slice_unpack_lines_kernel(PackArgs a) {
     uint64_t wg = a.wg0 + blockIdx.x;
@@ -329,7 +334,10 @@ __global__ __launch_bounds__(kPackThreads) void slice_unpack_lines_kernel(PackAr
     int64_t o = at < 0 ? 0 : at;
     if (o > run_bytes - 16) o = run_bytes - 16;
     const uint4 d = load16_unaligned(prow + o);
-    if (active) store16_unaligned(row + o, d);
+    if (active) {
+        if (a.stream_stores) store16_unaligned(row + o, d);  // wave-uniform
+        else store16_writethrough(row + o, d);
+    }
 }
 
 // Views whose contiguous runs are shorter than a chunk (element-strided selections such as
@@ -940,6 +948,7 @@ static int copy_views(char* base, char* const* packed, const mhip_slice_t* views
                 a.nrows = nrows;
                 if (nrows * lines + kPackThreads >= kFastDivLimit) wide = true;
                 line_blocks = (nrows * lines + kPackThreads / 8 - 1) / (kPackThreads / 8);
+                a.stream_stores = nbatch * first.total * unit >= kStreamUnpackFromBytes;  // by the bytes the launch writes
             }
         }
         const bool large = a.nchunks >= kLargeCopyChunks;
