@@ -8,10 +8,12 @@
 //
 // Blocks of 1024 are still counted over the flat index space of the bucket, so codes and
 // scales are bit-identical to the two-step pipeline.  A wavefront finds the tensors that
-// hold the first and the last element of its span with two cooperative 65-ary searches over
-// the offsets table; a span inside one tensor (the common case: tensors are >= 1K
-// elements) then costs nothing extra; a block that straddles tensors is walked tensor by
-// tensor, the lanes taking consecutive elements of each segment.
+// hold the first and the last element of its span from the bucket's block index (or with two
+// cooperative 65-ary searches over the offsets table); a span inside one tensor (the common
+// case: tensors are >= 1K elements) then costs nothing extra; a span or block that one
+// boundary between two tensors cuts is loaded in one go as well, each lane's vector from the
+// tensor it lies in; what is left (more boundaries, the short last block, blocks with Inf or
+// NaN) is walked tensor by tensor, the lanes taking consecutive elements of each segment.
 #include <mutex>
 
 #include "fp8_common.h"
@@ -51,33 +53,57 @@ __device__ __forceinline__ void span_tensors(const BucketArgs& a, uint64_t begin
 }
 
 // Careful path for one block that straddles tensors, holds NaN / Inf, or is the short last block of
-// the bucket, whole wavefront.  [t_lo, t_hi] are the tensors of its first and last element.  The block
-// is walked tensor by tensor (a wave-uniform loop whose table reads are scalar loads), so that inside a
-// segment the lanes take consecutive elements from one base pointer and no lane searches the table.
-__device__ void quantize_bucket_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
+// the bucket, whole wavefront.  [t_lo, t_hi] are the tensors of its first and last element (t_hi may be an
+// upper bound).  Lane l owns elements l, 64 + l, ... of the block, sixteen at most.  The block is walked tensor by
+// tensor (a wave-uniform loop whose table reads are scalar loads): inside a segment the lanes read consecutive
+// elements from one base pointer, no lane searches the table, and all loads of a segment are issued before any
+// value is used, so the block costs a few memory latencies.  (Sixteen dependent 64-element steps per pass, as
+// this path was first written, made a straddling span cost its wavefront about 10 us: invisible behind a 1.5 GB
+// bucket, but most of the run time of a bucket of 4 M elements.)
+constexpr int kCarefulSlots = kBlock / 64;
+
+__device__ __forceinline__ void quantize_bucket_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                            char* const* tensors, const uint64_t* offsets, uint32_t t_lo,
                                                            uint32_t t_hi, uint64_t begin, uint32_t count, uint64_t b,
                                                            int lane) {
     const uint64_t end = begin + count;
-    uint32_t m = 0;
+    uint16_t x[kCarefulSlots];
+#pragma unroll
+    for (int j = 0; j < kCarefulSlots; ++j) x[j] = 0;  // elements past a short block's end count as zeros
     for (uint32_t t = t_lo; t <= t_hi; ++t) {
         const uint64_t off = offsets[t], next = offsets[t + 1];
         const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
-        const uint16_t* __restrict__ p = reinterpret_cast<const uint16_t*>(tensors[t]) - off;  // p[e] is bucket element e
-        for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
-            const uint32_t v = p[e] & 0x7fffu;
-            if (v <= 0x7f80u && v > m) m = v;
+        if (seg_b >= seg_e) continue;  // an empty tensor, or one past the block
+        // The segment is elements [lo, hi) of the block, read from p.  No load is predicated (a lane outside the
+        // segment reads the segment's nearest element and drops it), so all of them are in flight together.
+        const uint16_t* __restrict__ p = reinterpret_cast<const uint16_t*>(tensors[t]) + (begin - off);
+        const uint32_t lo = (uint32_t)(seg_b - begin), hi = (uint32_t)(seg_e - begin);
+        uint16_t v[kCarefulSlots];
+#pragma unroll
+        for (int j = 0; j < kCarefulSlots; ++j) {
+            const uint32_t i = j * 64 + lane;
+            v[j] = p[i < lo ? lo : i >= hi ? hi - 1 : i];
         }
+#pragma unroll
+        for (int j = 0; j < kCarefulSlots; ++j) {
+            const uint32_t i = j * 64 + lane;
+            if (i >= lo && i < hi) x[j] = v[j];
+        }
+    }
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < kCarefulSlots; ++j) {
+        const uint32_t v = x[j] & 0x7fffu;
+        if (v <= 0x7f80u && v > m) m = v;
     }
     m = wave_max_u32(m);
     float scale, inv;
     block_factors(m, &scale, &inv);
     if (lane == 0) scales[b] = scale;
-    for (uint32_t t = t_lo; t <= t_hi; ++t) {
-        const uint64_t off = offsets[t], next = offsets[t + 1];
-        const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
-        const uint16_t* __restrict__ p = reinterpret_cast<const uint16_t*>(tensors[t]) - off;
-        for (uint64_t e = seg_b + lane; e < seg_e; e += 64) q[e] = quant_one_careful(p[e], inv);
+#pragma unroll
+    for (int j = 0; j < kCarefulSlots; ++j) {
+        const uint64_t e = begin + j * 64 + lane;
+        if (e < end) q[e] = quant_one_careful(x[j], inv);
     }
 }
 
@@ -120,12 +146,56 @@ __device__ __forceinline__ bool quantize_loaded_block(uint8_t* __restrict__ q, f
     return true;
 }
 
-// The rare span that touches several tensors or holds the short last block: block by block, each
-// block narrowed to its own tensors by a wave-uniform walk over the table.
-__device__ void quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __restrict__ scales,
-                                                       char* const* tensors, const uint64_t* offsets, uint64_t total,
-                                                       uint64_t nblocks, uint32_t t_first, uint32_t t_last, uint64_t b0,
-                                                       int lane) {
+// R rows of 1 KiB (512 elements each) that two tensors share: elements [0, cut) are the last ones of the first tensor,
+// starting at `head`, the others the first ones of the second tensor, which starts at `next`; 0 < cut < 512 R.  A lane's
+// vector comes from one of the two with the same unaligned load as in a span inside one tensor; the one vector that the
+// cut goes through is fetched element by element - by every lane for its own vector of that row, which needs no
+// branch - and all loads are in flight together.  (Through the careful path below a straddling block takes several
+// round trips one after the other: a span of three tensors cost its wavefront about 10 us, invisible behind a 1.5 GB
+// bucket and twice the rest of the run time of a bucket of 4 M elements.)
+template <int R>
+struct Rows {
+    uint4 row[R];
+};
+
+template <int R>
+__device__ __forceinline__ Rows<R> load_rows_of_two_tensors(const char* head, const char* next, uint32_t cut, int lane) {
+    Rows<R> out;
+    uint4 (&row)[R] = out.row;
+    const char* rest = reinterpret_cast<const char*>(reinterpret_cast<uintptr_t>(next) - (uintptr_t)cut * 2);  // element e >= cut at rest + 2 e
+#pragma unroll
+    for (int k = 0; k < R; ++k) {
+        uint32_t v0 = k * 512 + lane * 8;
+        if (v0 < cut && v0 + 8 > cut) v0 = v0 >= 8 ? v0 - 8 : 8;  // the cut vector: a valid neighbour instead, replaced below
+        if (v0 < cut) row[k] = load16_unaligned(head + v0 * 2);
+        else row[k] = load16_unaligned(rest + v0 * 2);
+    }
+    if (cut % 8 != 0) {
+        const uint32_t cut_row = cut / 512;
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t e = cut_row * 512 + lane * 8 + i;
+            uint32_t x;
+            if (e < cut) x = *reinterpret_cast<const uint16_t*>(head + e * 2);
+            else x = *reinterpret_cast<const uint16_t*>(rest + e * 2);
+            w[i / 2] = i % 2 ? w[i / 2] | (x << 16) : x;
+        }
+#pragma unroll
+        for (int k = 0; k < R; ++k)
+            if (k == (int)cut_row) row[k] = make_uint4(w[0], w[1], w[2], w[3]);  // wave-uniform
+    }
+    return out;
+}
+
+// The rare span that touches more than two tensors or holds the short last block: block by block, each block
+// narrowed to its own tensors by a wave-uniform walk over the table.  Returns the blocks (bit j: block b0 + j) that
+// are left for the careful path.
+__device__ __forceinline__ uint32_t quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                              char* const* tensors, const uint64_t* offsets, uint64_t total,
+                                                              uint64_t nblocks, uint32_t ntensors, uint32_t t_first, uint32_t t_last,
+                                                              uint64_t b0, int lane) {
+    uint32_t redo = 0;
     uint32_t tb = t_first;
     for (int j = 0; j < kBucketBlocks; ++j) {
         const uint64_t b = b0 + j;
@@ -133,19 +203,37 @@ __device__ void quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __rest
         const uint64_t begin = b * kBlock;
         const uint64_t end = begin + kBlock < total ? begin + kBlock : total;
         while (tb < t_last && offsets[tb + 1] <= begin) ++tb;
-        uint32_t te = tb;
-        while (te < t_last && offsets[te + 1] < end) ++te;
-        if (tb == te && end - begin == kBlock) {
+        if (end - begin == kBlock) {
+            const uint64_t next = offsets[tb + 1];
             const char* src = tensors[tb] + (begin - offsets[tb]) * 2;
-            const uint4 lo = load16_unaligned(src + lane * 16);
-            const uint4 hi = load16_unaligned(src + 1024 + lane * 16);
-            if (quantize_loaded_block(q, scales, lo, hi, begin, b, lane)) continue;
+            if (next >= end) {  // a full block inside one tensor
+                const uint4 lo = load16_unaligned(src + lane * 16);
+                const uint4 hi = load16_unaligned(src + 1024 + lane * 16);
+                if (quantize_loaded_block(q, scales, lo, hi, begin, b, lane)) continue;
+            } else if (tb + 2 <= ntensors && offsets[tb + 2] >= end) {  // a full block that two tensors share
+                const Rows<2> both = load_rows_of_two_tensors<2>(src, tensors[tb + 1], (uint32_t)(next - begin), lane);
+                if (quantize_loaded_block(q, scales, both.row[0], both.row[1], begin, b, lane)) continue;
+            }
         }
-        quantize_bucket_block_careful(q, scales, tensors, offsets, tb, te, begin, (uint32_t)(end - begin), b, lane);
+        redo |= 1u << j;
     }
+    return redo;
 }
 
-__global__ __launch_bounds__(kBucketThreads) void fp8_quantize_bucket_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
+// The kBucketBlocks blocks of a span whose elements are in registers, row[2j] and row[2j + 1] holding block j.
+// Returns the blocks (bit j: block b0 + j) that hold Inf or NaN and are left for the careful path.
+__device__ __forceinline__ uint32_t quantize_loaded_span(uint8_t* __restrict__ q, float* __restrict__ scales,
+                                                         const uint4 (&row)[2 * kBucketBlocks], uint64_t b0, int lane) {
+    uint32_t redo = 0;
+#pragma unroll
+    for (int j = 0; j < kBucketBlocks; ++j) {
+        const uint64_t b = b0 + j;
+        if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane)) redo |= 1u << j;
+    }
+    return redo;
+}
+
+__global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(4))) void fp8_quantize_bucket_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                        BucketArgs a) {
     const int lane = threadIdx.x & 63;
     const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (threadIdx.x >> 6);
@@ -156,37 +244,210 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_quantize_bucket_kernel(uin
                                       ? span_begin + (uint64_t)kBucketBlocks * kBlock : a.total;
         uint32_t t_first, t_last;
         span_tensors(a, span_begin, span_end, &t_first, &t_last);
-        if (t_first != t_last || span_end - span_begin != (uint64_t)kBucketBlocks * kBlock) {  // wave-uniform, rare
-            quantize_bucket_span_slow(q, scales, a.tensors, a.offsets, a.total, a.nblocks, t_first, t_last, b0, lane);
-            continue;
-        }
-        // the whole span lies in one tensor: all loads of the lane back to back from one base pointer
-        const uint64_t t_begin = a.offsets[t_first], t_end = a.offsets[t_first + 1];
-        const char* src = a.tensors[t_first] + (span_begin - t_begin) * 2;
-        const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
+        const bool full = span_end - span_begin == (uint64_t)kBucketBlocks * kBlock;
+        // Blocks that need the careful path are only noted (bit j: block b0 + j; wave-uniform) and worked off in one
+        // place at the end of the step, where the span's registers are free: inlined where the rows are live, that
+        // path costs the whole kernel a quarter of its wavefronts; as a function that is not inlined, its table reads
+        // become vector loads with a round trip each (6 us for one short block).
+        uint32_t redo = 0;
+        uint32_t t_redo = t_first;     // last tensor those blocks can touch
         uint4 row[2 * kBucketBlocks];  // row[2j] = first, row[2j + 1] = second 1 KiB of block j
-        if (shift != 0 && (span_begin - t_begin) * 2 >= shift && (t_end - span_end) * 2 >= 16 - shift) {
-            const char* base = src - shift;  // 16-byte aligned, and [base, base + 8 KiB + 16) lies inside the tensor
+        if (t_first == t_last && full) {
+            // the whole span lies in one tensor (the common case): all loads of the lane back to back from one base pointer
+            const uint64_t t_begin = a.offsets[t_first], t_end = a.offsets[t_first + 1];
+            const char* src = a.tensors[t_first] + (span_begin - t_begin) * 2;
+            const uint32_t shift = (uint32_t)((uintptr_t)src & 15u);
+            if (shift != 0 && (span_begin - t_begin) * 2 >= shift && (t_end - span_end) * 2 >= 16 - shift) {
+                const char* base = src - shift;  // 16-byte aligned, and [base, base + 8 KiB + 16) lies inside the tensor
 #pragma unroll
-            for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_aligned(base + k * 1024 + lane * 16);
-            const uint4 tail = load16_aligned(base + 2 * kBucketBlocks * 1024);
-            shift_rows_into_place<2 * kBucketBlocks>(row, tail, shift);
+                for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_aligned(base + k * 1024 + lane * 16);
+                const uint4 tail = load16_aligned(base + 2 * kBucketBlocks * 1024);
+                shift_rows_into_place<2 * kBucketBlocks>(row, tail, shift);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_unaligned(src + k * 1024 + lane * 16);
+            }
+            redo = quantize_loaded_span(q, scales, row, b0, lane);
+        } else if (full && t_first + 2 <= a.ntensors && a.offsets[t_first + 2] >= span_end) {
+            // one tensor ends inside the span and the next one holds the rest (every span that straddles tensors of
+            // 4096 elements and more)
+            const uint32_t cut = (uint32_t)(a.offsets[t_first + 1] - span_begin);  // 0 < cut < span length
+            const char* head = a.tensors[t_first] + (span_begin - a.offsets[t_first]) * 2;
+            const char* rest = reinterpret_cast<const char*>(reinterpret_cast<uintptr_t>(a.tensors[t_first + 1]) - (uintptr_t)cut * 2);
+            // as in load_rows_of_two_tensors, on the span's own registers
+#pragma unroll
+            for (int k = 0; k < 2 * kBucketBlocks; ++k) {
+                uint32_t v0 = k * 512 + lane * 8;
+                if (v0 < cut && v0 + 8 > cut) v0 = v0 >= 8 ? v0 - 8 : 8;
+                if (v0 < cut) row[k] = load16_unaligned(head + v0 * 2);
+                else row[k] = load16_unaligned(rest + v0 * 2);
+            }
+            if (cut % 8 != 0) {
+                const uint32_t cut_row = cut / 512;
+                uint32_t w[4];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t e = cut_row * 512 + lane * 8 + i;
+                    uint32_t x;
+                    if (e < cut) x = *reinterpret_cast<const uint16_t*>(head + e * 2);
+                    else x = *reinterpret_cast<const uint16_t*>(rest + e * 2);
+                    w[i / 2] = i % 2 ? w[i / 2] | (x << 16) : x;
+                }
+#pragma unroll
+                for (int k = 0; k < 2 * kBucketBlocks; ++k)
+                    if (k == (int)cut_row) row[k] = make_uint4(w[0], w[1], w[2], w[3]);  // wave-uniform
+            }
+            redo = quantize_loaded_span(q, scales, row, b0, lane);
+            t_redo = t_first + 1;
+        } else {  // more than two tensors, or the short last span of the bucket
+            redo = quantize_bucket_span_slow(q, scales, a.tensors, a.offsets, a.total, a.nblocks, a.ntensors, t_first, t_last, b0, lane);
+            t_redo = t_last;
+        }
+        for (uint64_t b = b0; redo != 0; ++b, redo >>= 1) {
+            if (redo & 1u) {
+                const uint64_t begin = b * kBlock;
+                const uint32_t count = a.total - begin < kBlock ? (uint32_t)(a.total - begin) : (uint32_t)kBlock;
+                quantize_bucket_block_careful(q, scales, a.tensors, a.offsets, t_first, t_redo, begin, count, b, lane);
+            }
+        }
+    }
+}
+
+// The dequantisers' path for a block that straddles tensors or is the short last block of the bucket, whole
+// wavefront: the accumulator elements of the block are read tensor by tensor with all loads of a segment in
+// flight together (lane l owns elements l, 64 + l, ...), the n peers' codes are added in order, each peer's
+// loads issued together (codes(r) is peer r's code buffer, scale(r) its scale for this block), and the sums are
+// written back tensor by tensor.  [t_lo, t_hi] as in the quantiser's careful path.
+template <typename Codes, typename Scale>
+__device__ __forceinline__ void dequant_bucket_block_careful(const BucketArgs& a, uint32_t t_lo, uint32_t t_hi, uint64_t begin,
+                                                             uint64_t end, int lane, uint32_t n, Codes&& codes, Scale&& scale) {
+    // in two halves of 512 elements, which keeps the registers of this rare path under those of the common one
+    constexpr int H = kCarefulSlots / 2;
+    const uint32_t count = (uint32_t)(end - begin);
+#pragma unroll 1
+    for (uint32_t first = 0; first < count; first += H * 64) {
+        float x[H];
+#pragma unroll
+        for (int j = 0; j < H; ++j) x[j] = 0.0f;
+        for (uint32_t t = t_lo; t <= t_hi; ++t) {
+            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
+            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+            if (seg_b >= seg_e) continue;  // an empty tensor, or one past the block
+            // the segment is elements [lo, hi) of the block, read from p; no load is predicated
+            const float* __restrict__ p = reinterpret_cast<const float*>(a.tensors[t]) + (begin - off);
+            const uint32_t lo = (uint32_t)(seg_b - begin), hi = (uint32_t)(seg_e - begin);
+            float v[H];
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                const uint32_t i = first + j * 64 + lane;
+                v[j] = p[i < lo ? lo : i >= hi ? hi - 1 : i];
+            }
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                const uint32_t i = first + j * 64 + lane;
+                if (i >= lo && i < hi) x[j] = v[j];
+            }
+        }
+        for (uint32_t r = 0; r < n; ++r) {
+            const uint8_t* __restrict__ q = codes(r) + begin;
+            const float s = scale(r);
+            uint8_t c[H];
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                const uint32_t i = first + j * 64 + lane;
+                c[j] = q[i < count ? i : count - 1];
+            }
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                const auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)c[j], false);
+                x[j] = x[j] + v[0] * s;  // product rounded, then added
+            }
+        }
+        for (uint32_t t = t_lo; t <= t_hi; ++t) {
+            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
+            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
+            if (seg_b >= seg_e) continue;
+            float* __restrict__ p = reinterpret_cast<float*>(a.tensors[t]) + (begin - off);
+            const uint32_t lo = (uint32_t)(seg_b - begin), hi = (uint32_t)(seg_e - begin);
+#pragma unroll
+            for (int j = 0; j < H; ++j) {
+                const uint32_t i = first + j * 64 + lane;
+                if (i >= lo && i < hi) p[i] = x[j];
+            }
+        }
+    }
+}
+
+// Accumulator elements of a full block that one tensor boundary cuts (every block that straddles tensors of 1024
+// elements and more): element i of the block is head[i] for i < cut and rest[i] from there on.  Step j of a lane is
+// elements j * 256 + lane * 4 .. + 3: a 128-bit access to one of the two tensors, except in the step that holds the
+// vector the cut goes through, which every lane moves element by element (a wave-uniform choice, no lane branches).
+// All loads of the block are then in flight together as in a block inside one tensor; through the careful path
+// above such a block takes several round trips, which shows in buckets of a few million elements.
+struct CutBlock {
+    float* head;
+    float* rest;
+    uint32_t cut;  // 0 < cut < kBlock
+    __device__ __forceinline__ CutBlock(const BucketArgs& a, uint32_t t, uint64_t begin) {
+        cut = (uint32_t)(a.offsets[t + 1] - begin);
+        head = reinterpret_cast<float*>(a.tensors[t]) + (begin - a.offsets[t]);
+        rest = reinterpret_cast<float*>(reinterpret_cast<uintptr_t>(a.tensors[t + 1]) - (uintptr_t)cut * 4);
+    }
+    __device__ __forceinline__ bool by_elements(int j) const { return cut % 4 != 0 && cut / 256 == (uint32_t)j; }
+    __device__ __forceinline__ float* at(uint32_t i) const { return (i < cut ? head : rest) + i; }
+    __device__ __forceinline__ uint4 load(int j, int lane) const {
+        const uint32_t v0 = j * 256 + lane * 4;
+        if (by_elements(j))
+            return make_uint4(__float_as_uint(*at(v0)), __float_as_uint(*at(v0 + 1)), __float_as_uint(*at(v0 + 2)),
+                              __float_as_uint(*at(v0 + 3)));
+        return load16_unaligned(at(v0));
+    }
+    __device__ __forceinline__ void store(int j, int lane, const uint4& r) const {
+        const uint32_t v0 = j * 256 + lane * 4;
+        if (by_elements(j)) {
+            *at(v0) = __uint_as_float(r.x);
+            *at(v0 + 1) = __uint_as_float(r.y);
+            *at(v0 + 2) = __uint_as_float(r.z);
+            *at(v0 + 3) = __uint_as_float(r.w);
         } else {
-#pragma unroll
-            for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_unaligned(src + k * 1024 + lane * 16);
+            store16_unaligned(at(v0), r);
         }
+    }
+};
+
+// whether the full block [begin, begin + kBlock), whose first element tensor t holds, ends in tensor t + 1
+__device__ __forceinline__ bool block_cut_once(const BucketArgs& a, uint32_t t, uint64_t begin) {
+    return t + 2 <= a.ntensors && a.offsets[t + 1] < begin + kBlock && a.offsets[t + 2] >= begin + kBlock;
+}
+
+// One block of one peer: codes at q + begin, accumulator vectors through load(j) / store(j, r), 4 steps of 256
+// elements, all loads first.
+template <typename Load, typename Store>
+__device__ __forceinline__ void dequant_accumulate_block(const uint8_t* __restrict__ q, float s, uint64_t begin, int lane, Load&& load,
+                                                         Store&& store) {
+    uint32_t codes[4];
+    uint4 acc[4];
 #pragma unroll
-        for (int j = 0; j < kBucketBlocks; ++j) {
-            const uint64_t b = b0 + j;
-            if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane))
-                quantize_bucket_block_careful(q, scales, a.tensors, a.offsets, t_first, t_first, b * kBlock, kBlock, b, lane);
-        }
+    for (int j = 0; j < 4; ++j) {
+        codes[j] = load4_unaligned(q + begin + j * 256 + lane * 4);
+        acc[j] = load(j);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], false);
+        const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], true);
+        uint4 r;
+        r.x = __float_as_uint(__uint_as_float(acc[j].x) + p01[0] * s);
+        r.y = __float_as_uint(__uint_as_float(acc[j].y) + p01[1] * s);
+        r.z = __float_as_uint(__uint_as_float(acc[j].z) + p23[0] * s);
+        r.w = __float_as_uint(__uint_as_float(acc[j].w) + p23[1] * s);
+        store(j, r);
     }
 }
 
 // out_t[j] += float(q[off_t + j]) * scale[(off_t + j) / 1024], accumulators are the bucket's
 // own fp32 tensors.  One wavefront per 1024-element block, 4 lanes-groups of 4 elements each.
-__global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_kernel(const uint8_t* __restrict__ q,
+__global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(7))) void fp8_dequant_accumulate_bucket_kernel(const uint8_t* __restrict__ q,
                                                                                  const float* __restrict__ scales,
                                                                                  BucketArgs a) {
     const int lane = threadIdx.x & 63;
@@ -199,38 +460,20 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_
         span_tensors(a, begin, end, &t_lo, &t_hi);
         const float s = scales[b];
         if (t_lo == t_hi && end - begin == kBlock) {
-            // the whole block lies in one tensor: 4 steps of 256 elements, all loads first
+            // the whole block lies in one tensor
             float* dst = reinterpret_cast<float*>(a.tensors[t_lo]) + (begin - a.offsets[t_lo]);
-            uint32_t codes[4];
-            uint4 acc[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                codes[j] = load4_unaligned(q + begin + j * 256 + lane * 4);
-                acc[j] = load16_unaligned(dst + j * 256 + lane * 4);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], false);
-                const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[j], true);
-                uint4 r;
-                r.x = __float_as_uint(__uint_as_float(acc[j].x) + p01[0] * s);
-                r.y = __float_as_uint(__uint_as_float(acc[j].y) + p01[1] * s);
-                r.z = __float_as_uint(__uint_as_float(acc[j].z) + p23[0] * s);
-                r.w = __float_as_uint(__uint_as_float(acc[j].w) + p23[1] * s);
-                store16_unaligned(dst + j * 256 + lane * 4, r);
-            }
+            dequant_accumulate_block(q, s, begin, lane, [&](int j) { return load16_unaligned(dst + j * 256 + lane * 4); },
+                                     [&](int j, const uint4& r) { store16_unaligned(dst + j * 256 + lane * 4, r); });
             continue;
         }
-        // straddling or short block: tensor by tensor (wave-uniform loop), lanes on consecutive elements
-        for (uint32_t t = t_lo; t <= t_hi; ++t) {
-            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
-            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
-            float* __restrict__ p = reinterpret_cast<float*>(a.tensors[t]) - off;  // p[e] is bucket element e
-            for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
-                const auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[e], false);
-                p[e] = p[e] + v[0] * s;
-            }
+        if (end - begin == kBlock && block_cut_once(a, t_lo, begin)) {
+            const CutBlock c(a, t_lo, begin);
+            dequant_accumulate_block(q, s, begin, lane, [&](int j) { return c.load(j, lane); },
+                                     [&](int j, const uint4& r) { c.store(j, lane, r); });
+            continue;
         }
+        // more than two tensors, or the short last block
+        dequant_bucket_block_careful(a, t_lo, t_hi, begin, end, lane, 1, [&](uint32_t) { return q; }, [&](uint32_t) { return s; });
     }
 }
 
@@ -246,7 +489,49 @@ struct BucketPeersArgs {
     uint32_t n;
 };
 
-__global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_many_kernel(BucketPeersArgs p) {
+// One full block of all peers: accumulator vectors through load(j) / store(j, r), peers four at a time with all
+// their codes loaded before the first add.
+template <typename Load, typename Store>
+__device__ __forceinline__ void dequant_accumulate_block_peers(const BucketPeersArgs& p, uint64_t b, int lane, Load&& load, Store&& store) {
+    const uint64_t begin = b * kBlock;
+    float v[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint4 r = load(j);
+        v[j][0] = __uint_as_float(r.x); v[j][1] = __uint_as_float(r.y);
+        v[j][2] = __uint_as_float(r.z); v[j][3] = __uint_as_float(r.w);
+    }
+    for (uint32_t r0 = 0; r0 < p.n; r0 += 4) {
+        uint32_t codes[4][4];
+        float s[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint32_t r = r0 + g < p.n ? r0 + g : p.n - 1;  // clamped: surplus loads are unused
+            s[g] = p.scales[r][b];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) codes[g][j] = load4_unaligned(p.q[r] + begin + j * 256 + lane * 4);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            if (r0 + g < p.n) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], false);
+                    const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], true);
+                    v[j][0] = v[j][0] + p01[0] * s[g];
+                    v[j][1] = v[j][1] + p01[1] * s[g];
+                    v[j][2] = v[j][2] + p23[0] * s[g];
+                    v[j][3] = v[j][3] + p23[1] * s[g];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        store(j, make_uint4(__float_as_uint(v[j][0]), __float_as_uint(v[j][1]), __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
+}
+
+__global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(7))) void fp8_dequant_accumulate_bucket_many_kernel(BucketPeersArgs p) {
     const BucketArgs& a = p.b;
     const int lane = threadIdx.x & 63;
     const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (threadIdx.x >> 6);
@@ -258,57 +543,19 @@ __global__ __launch_bounds__(kBucketThreads) void fp8_dequant_accumulate_bucket_
         span_tensors(a, begin, end, &t_lo, &t_hi);
         if (t_lo == t_hi && end - begin == kBlock) {
             float* dst = reinterpret_cast<float*>(a.tensors[t_lo]) + (begin - a.offsets[t_lo]);
-            float v[4][4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint4 r = load16_unaligned(dst + j * 256 + lane * 4);
-                v[j][0] = __uint_as_float(r.x); v[j][1] = __uint_as_float(r.y);
-                v[j][2] = __uint_as_float(r.z); v[j][3] = __uint_as_float(r.w);
-            }
-            for (uint32_t r0 = 0; r0 < p.n; r0 += 4) {
-                uint32_t codes[4][4];
-                float s[4];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const uint32_t r = r0 + g < p.n ? r0 + g : p.n - 1;  // clamped: surplus loads are unused
-                    s[g] = p.scales[r][b];
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) codes[g][j] = load4_unaligned(p.q[r] + begin + j * 256 + lane * 4);
-                }
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    if (r0 + g < p.n) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const auto p01 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], false);
-                            const auto p23 = __builtin_amdgcn_cvt_pk_f32_fp8((int)codes[g][j], true);
-                            v[j][0] = v[j][0] + p01[0] * s[g];
-                            v[j][1] = v[j][1] + p01[1] * s[g];
-                            v[j][2] = v[j][2] + p23[0] * s[g];
-                            v[j][3] = v[j][3] + p23[1] * s[g];
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                store16_unaligned(dst + j * 256 + lane * 4, make_uint4(__float_as_uint(v[j][0]), __float_as_uint(v[j][1]),
-                                                                      __float_as_uint(v[j][2]), __float_as_uint(v[j][3])));
+            dequant_accumulate_block_peers(p, b, lane, [&](int j) { return load16_unaligned(dst + j * 256 + lane * 4); },
+                                           [&](int j, const uint4& r) { store16_unaligned(dst + j * 256 + lane * 4, r); });
             continue;
         }
-        for (uint32_t t = t_lo; t <= t_hi; ++t) {  // straddling or short block: tensor by tensor
-            const uint64_t off = a.offsets[t], next = a.offsets[t + 1];
-            const uint64_t seg_b = begin > off ? begin : off, seg_e = end < next ? end : next;
-            float* __restrict__ ptr = reinterpret_cast<float*>(a.tensors[t]) - off;
-            for (uint64_t e = seg_b + lane; e < seg_e; e += 64) {
-                float x = ptr[e];
-                for (uint32_t r = 0; r < p.n; ++r) {
-                    const auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)p.q[r][e], false);
-                    x = x + c[0] * p.scales[r][b];
-                }
-                ptr[e] = x;
-            }
+        if (end - begin == kBlock && block_cut_once(a, t_lo, begin)) {
+            const CutBlock c(a, t_lo, begin);
+            dequant_accumulate_block_peers(p, b, lane, [&](int j) { return c.load(j, lane); },
+                                           [&](int j, const uint4& r) { c.store(j, lane, r); });
+            continue;
         }
+        // more than two tensors, or the short last block
+        dequant_bucket_block_careful(a, t_lo, t_hi, begin, end, lane, p.n, [&](uint32_t r) { return p.q[r]; },
+                                     [&](uint32_t r) { return p.scales[r][b]; });
     }
 }
 

@@ -18,16 +18,30 @@ namespace mhip {
 __device__ __noinline__ void quantize_block_careful(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                     const uint16_t* __restrict__ x, uint64_t begin, uint32_t count,
                                                     uint64_t b, int lane) {
+    // lane l owns elements l, 64 + l, ... of the block; all of its loads are issued before the first use
+    constexpr int kSlots = kBlock / 64;
+    uint16_t v[kSlots];
+#pragma unroll
+    for (int j = 0; j < kSlots; ++j) {
+        const uint32_t i = j * 64 + lane;
+        const uint16_t e = x[begin + (i < count ? i : count - 1)];  // no load is predicated
+        v[j] = i < count ? e : (uint16_t)0;                          // elements past a short block's end count as zeros
+    }
     uint32_t m = 0;
-    for (uint32_t i = lane; i < count; i += 64) {
-        const uint32_t a = x[begin + i] & 0x7fffu;
+#pragma unroll
+    for (int j = 0; j < kSlots; ++j) {
+        const uint32_t a = v[j] & 0x7fffu;
         if (a <= 0x7f80u && a > m) m = a;
     }
     m = wave_max_u32(m);
     float scale, inv;
     block_factors(m, &scale, &inv);
     if (lane == 0) scales[b] = scale;
-    for (uint32_t i = lane; i < count; i += 64) q[begin + i] = quant_one_careful(x[begin + i], inv);
+#pragma unroll
+    for (int j = 0; j < kSlots; ++j) {
+        const uint32_t i = j * 64 + lane;
+        if (i < count) q[begin + i] = quant_one_careful(v[j], inv);
+    }
 }
 
 // Blocks a wavefront quantises per step (all their loads are issued before the first max).  Measured on

@@ -209,6 +209,67 @@ def test_fused_bucket_forms_equal_two_step_pipeline():
         assert st[: i % 3].abs().sum() == 0 and st[i % 3 + n:].abs().sum() == 0  # neighbours untouched
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("indexed", [True, False])
+def test_spans_and_blocks_shared_by_tensors(seed, indexed):
+    # The fused forms load a span (4 blocks) or a block that one boundary between tensors cuts in one go, take the
+    # careful path for more boundaries and for the short last block, and put off blocks with Inf / NaN until the rest
+    # of their span is done.  Random mixes of tensor sizes put boundaries everywhere: on and off multiples of 8
+    # elements, in the first and last vector of a span, several in one block, empty tensors between them; Inf and
+    # NaN land in blocks of every kind; tensors start on 2-byte (4-byte for the accumulators) boundaries only.
+    rng = np.random.default_rng(9000 + seed)
+    kinds = [(1, 9), (9, 600), (600, 1500), (1500, 5000), (5000, 40000)]
+    sizes = []
+    for _ in range(int(rng.integers(12, 40))):
+        lo, hi = kinds[int(rng.integers(0, len(kinds)))]
+        n = int(rng.integers(lo, hi))
+        if rng.random() < 0.3:
+            n = n // 8 * 8                      # cuts on whole vectors too
+        sizes.append(0 if rng.random() < 0.05 else n)
+    if seed % 2:
+        sizes[-1] += (-sum(sizes)) % 1024       # odd seeds: no short last block
+    total = sum(sizes)
+    offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    flat_h = _c5_like(total, seed=seed)
+    for pos in rng.integers(0, total, size=6):  # Inf / NaN in six blocks
+        flat_h[int(pos)] = float("nan") if pos % 2 else float("-inf")
+    store = [torch.zeros(n + 6, dtype=torch.bfloat16, device=DEV) for n in sizes]
+    dev = []
+    for i, (st, n) in enumerate(zip(store, sizes)):
+        v = st[i % 4: i % 4 + n]
+        v.copy_(flat_h[offs[i]: offs[i + 1]])
+        dev.append(v)
+    bucket = fp8.FlatBucket(dev)
+    q1, s1 = fp8.quantize_bucket(bucket, indexed=indexed)
+    sync()
+    wq, ws = oracle.fp8_quantize(bits(flat_h), 1024)
+    assert np.array_equal(q1.cpu().numpy(), wq), (seed, sizes)
+    assert np.array_equal(s1.cpu().numpy().view(np.uint32), ws.view(np.uint32)), (seed, sizes)
+    # receive side: one peer, then three peers in one pass, into staggered fp32 accumulators
+    qf = q1.clone()
+    qf[(qf & 0x7F) == 0x7F] = 0x23              # keep the sums free of NaN
+    peers_q = [qf, qf ^ 0x05, qf ^ 0x40]
+    peers_q = [torch.where((p & 0x7F) == 0x7F, torch.full_like(p, 0x31), p) for p in peers_q]
+    peers_s = [s1, s1 * 0.5, s1 * 1.25]
+    acc_h = rng.normal(size=total).astype(np.float32)
+    astore = [torch.zeros(n + 3, dtype=torch.float32, device=DEV) for n in sizes]
+    accs = [st[i % 3: i % 3 + n] for i, (st, n) in enumerate(zip(astore, sizes))]
+    for a, lo, hi in zip(accs, offs[:-1], offs[1:]):
+        a.copy_(torch.from_numpy(acc_h[lo:hi]))
+    abucket = fp8.FlatBucket(accs)
+    fp8.dequant_accumulate_bucket(abucket, peers_q[0], peers_s[0], indexed=indexed)
+    oracle.fp8_dequant_accumulate(acc_h, peers_q[0].cpu().numpy(), peers_s[0].cpu().numpy(), 1024)
+    fp8.dequant_accumulate_bucket_many(abucket, peers_q, peers_s, indexed=indexed)
+    for pq, ps in zip(peers_q, peers_s):
+        oracle.fp8_dequant_accumulate(acc_h, pq.cpu().numpy(), ps.cpu().numpy(), 1024)
+    sync()
+    for i, (a, st, n) in enumerate(zip(accs, astore, sizes)):
+        assert np.array_equal(a.cpu().numpy().view(np.uint32), acc_h[offs[i]: offs[i + 1]].view(np.uint32)), (seed, i, sizes)
+        assert st[: i % 3].abs().sum() == 0 and st[i % 3 + n:].abs().sum() == 0  # neighbours untouched
+    for i, (st, n) in enumerate(zip(store, sizes)):                              # the quantiser only reads
+        assert st[: i % 4].abs().sum() == 0 and st[i % 4 + n:].abs().sum() == 0
+
+
 @pytest.mark.parametrize("ntensors", [1, 2, 64, 65, 66, 67, 130, 4225, 4226, 9000])
 def test_many_small_tensors_table_search(ntensors):
     # exercises the cooperative table search at its range boundaries (65-ary steps) with empty tensors mixed in
