@@ -189,37 +189,50 @@ __device__ __forceinline__ Rows<R> load_rows_of_two_tensors(const char* head, co
 }
 
 // The rare span that touches more than two tensors or holds the short last block: block by block, each block
-// narrowed to its own tensors by a wave-uniform walk over the table.  Returns the blocks (bit j: block b0 + j) that
-// are left for the careful path.
+// narrowed to its own tensors by a wave-uniform walk over the table; full blocks inside one tensor or shared by two
+// are loaded first, all of them, and quantised then.  Returns the blocks (bit j: block b0 + j) that are left for the
+// careful path.
 __device__ __forceinline__ uint32_t quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                               char* const* tensors, const uint64_t* offsets, uint64_t total,
                                                               uint64_t nblocks, uint32_t ntensors, uint32_t t_first, uint32_t t_last,
                                                               uint64_t b0, int lane) {
-    uint32_t redo = 0;
+    uint32_t redo = 0, loaded = 0;
     uint32_t tb = t_first;
+    uint4 row[2 * kBucketBlocks];
+#pragma unroll
     for (int j = 0; j < kBucketBlocks; ++j) {
         const uint64_t b = b0 + j;
-        if (b >= nblocks) break;
-        const uint64_t begin = b * kBlock;
-        const uint64_t end = begin + kBlock < total ? begin + kBlock : total;
-        while (tb < t_last && offsets[tb + 1] <= begin) ++tb;
-        if (end - begin == kBlock) {
-            const uint64_t next = offsets[tb + 1];
-            const char* src = tensors[tb] + (begin - offsets[tb]) * 2;
-            if (next >= end) {  // a full block inside one tensor
-                const uint4 lo = load16_unaligned(src + lane * 16);
-                const uint4 hi = load16_unaligned(src + 1024 + lane * 16);
-                if (quantize_loaded_block(q, scales, lo, hi, begin, b, lane)) continue;
-            } else if (tb + 2 <= ntensors && offsets[tb + 2] >= end) {  // a full block that two tensors share
-                const Rows<2> both = load_rows_of_two_tensors<2>(src, tensors[tb + 1], (uint32_t)(next - begin), lane);
-                if (quantize_loaded_block(q, scales, both.row[0], both.row[1], begin, b, lane)) continue;
+        if (b < nblocks) {
+            const uint64_t begin = b * kBlock;
+            const uint64_t end = begin + kBlock < total ? begin + kBlock : total;
+            while (tb < t_last && offsets[tb + 1] <= begin) ++tb;
+            bool ok = false;
+            if (end - begin == kBlock) {
+                const uint64_t next = offsets[tb + 1];
+                const char* src = tensors[tb] + (begin - offsets[tb]) * 2;
+                if (next >= end) {  // a full block inside one tensor
+                    row[2 * j] = load16_unaligned(src + lane * 16);
+                    row[2 * j + 1] = load16_unaligned(src + 1024 + lane * 16);
+                    ok = true;
+                } else if (tb + 2 <= ntensors && offsets[tb + 2] >= end) {  // a full block that two tensors share
+                    const Rows<2> both = load_rows_of_two_tensors<2>(src, tensors[tb + 1], (uint32_t)(next - begin), lane);
+                    row[2 * j] = both.row[0];
+                    row[2 * j + 1] = both.row[1];
+                    ok = true;
+                }
             }
+            if (ok) loaded |= 1u << j;
+            else redo |= 1u << j;
         }
-        redo |= 1u << j;
+    }
+#pragma unroll
+    for (int j = 0; j < kBucketBlocks; ++j) {
+        const uint64_t b = b0 + j;
+        if ((loaded >> j) & 1u)
+            if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane)) redo |= 1u << j;
     }
     return redo;
 }
-
 // The kBucketBlocks blocks of a span whose elements are in registers, row[2j] and row[2j + 1] holding block j.
 // Returns the blocks (bit j: block b0 + j) that hold Inf or NaN and are left for the careful path.
 __device__ __forceinline__ uint32_t quantize_loaded_span(uint8_t* __restrict__ q, float* __restrict__ scales,
