@@ -262,7 +262,15 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_kernel(ReduceArgs a) {
         const uint64_t i = nvec * V + threadIdx.x;
         if (threadIdx.x < V && i < a.numel) {
             acc_t acc = VT::widen1(a.in[0], i);
-            for (uint32_t r = 1; r < a.n; ++r) acc = combine<MODE>(acc, VT::widen1(a.in[r], i), a.op);
+            uint32_t r = 1;
+            for (; r + 8 <= a.n; r += 8) {  // eight loads in flight, as in the body
+                acc_t x[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) x[j] = VT::widen1(a.in[r + j], i);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc = combine<MODE>(acc, x[j], a.op);
+            }
+            for (; r < a.n; ++r) acc = combine<MODE>(acc, VT::widen1(a.in[r], i), a.op);
             VT::narrow1(a.out, i, finish(acc, MODE == kAvg, a.scale, a.divisor));
         }
     }
@@ -374,7 +382,7 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
 
     for (uint64_t c = tile0 * kReduceThreads + threadIdx.x; c < nchunks; c += stride) {
         const uint64_t first = c * V;
-        if (first + V > a.total) {
+        if (a.total < (uint64_t)V) {  // an output shorter than one vector
             for (uint64_t t = first; t < a.total; ++t) one_element(t);
             continue;
         }
@@ -384,11 +392,13 @@ __global__ __launch_bounds__(kReduceThreads) void reduce_scatter_ragged_kernel(S
         uint64_t ta = first, ra = r0, tb = 0, rb = 0;
         bool do_b = false;
         if (rem < (uint64_t)V) {
+            // the last chunk of the output ends its last row: vector A alone, ending where the output ends (one lane
+            // summing the last elements one by one, input after input, cost a small launch 2-3 us)
             ta = first + rem - V;
             ra = r0 + rem - V;
             tb = first + rem;
-            rb = a.out_offset[k] + decode<WIDE, D>(a.out_dims, tb, &col);
-            do_b = true;
+            do_b = tb < a.total;
+            if (do_b) rb = a.out_offset[k] + decode<WIDE, D>(a.out_dims, tb, &col);
         }
         uint64_t ca, cb;
         const uint64_t la = a.in_offset + decode<WIDE, D>(a.in_dims, ra, &ca);
