@@ -209,12 +209,25 @@ __global__ __launch_bounds__(THREADS) void fp8_dequant_accumulate_many_kernel(De
                                                    __float_as_uint(v[2]), __float_as_uint(v[3])));
             continue;
         }
-        // last tile: element by element
+        // last tile: element by element, eight peers' codes in flight at a time
         for (uint64_t e = i0; e < a.numel && e < i0 + 4; ++e) {
             float x = a.overwrite ? 0.0f : acc[e];
-            for (uint32_t r = 0; r < n; ++r) {
-                const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)a.q[r][e], false);
-                x = x + p[0] * a.scales[r][e / kBlock];
+            for (uint32_t r0 = 0; r0 < n; r0 += 8) {
+                uint8_t c[8];
+                float s[8];
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    const uint32_t r = r0 + g < n ? r0 + g : n - 1;  // clamped: surplus loads are unused
+                    c[g] = a.q[r][e];
+                    s[g] = a.scales[r][e / kBlock];
+                }
+#pragma unroll
+                for (int g = 0; g < 8; ++g) {
+                    if (r0 + g < n) {
+                        const auto p = __builtin_amdgcn_cvt_pk_f32_fp8((int)c[g], false);
+                        x = x + p[0] * s[g];
+                    }
+                }
             }
             acc[e] = x;
         }
