@@ -992,6 +992,98 @@ def sweep_strided_views(dtypes, launches=20):
         torch.cuda.empty_cache()
 
 
+BUCKET_SIZES_HEADER = """\
+# The stages of configuration 5 on buckets of a few to a hundred million elements (MI355X)
+
+Command (repository root, one GPU; under a minute):
+
+    python bench.py --sweep bucket_sizes > profiles/fp8_bucket_sizes.md
+
+Buckets of bf16 tensors with `round(exp(U(ln 2^10, ln 2^21)))` elements each (numpy `default_rng(total in M)`), drawn
+until the bucket holds the stated number of elements, every tensor an allocation of its own; the flat buffers, codes,
+scales and fp32 accumulators beside them.  Every cell is the time of one launch in microseconds and, in brackets, the
+fraction of the 8 TB/s HBM peak its algorithmic bytes make of it (flat pack 4 T, quantise 3 T + 4 B, dequantise and
+accumulate 9 T + 4 B, flat unpack of fp32 8 T; T elements, B blocks of 1024): median of 3 runs of {launches} launches,
+3 rotating bucket sets, all forms with the bucket's block index.  A launch of a few MB is bound by its longest
+wavefront, not by bandwidth: the rows show what the rare paths of the fused kernels (tensor boundaries inside a span,
+the short last block) cost there.
+"""
+
+
+def sweep_bucket_sizes(launches=30):
+    """Time per launch of the flat-bucket and fp8 stages against the bucket's size (--sweep bucket_sizes)."""
+    import numpy as np
+    torch, lib, _ = _load()
+    from monarch_amd import fp8
+    torch.cuda.set_device(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    stages = ("flat_pack", "quantize", "quantize_bucket", "dequant", "dequant_bucket", "flat_unpack")
+    print(BUCKET_SIZES_HEADER.format(launches=launches))
+    print("| elements | tensors | " + " | ".join(stages) + " |")
+    print("|---:|---:|" + "---:|" * len(stages))
+    for total_m in (4, 13, 32, 64, 128):
+        rng = np.random.default_rng(total_m)
+        sizes = []
+        while sum(sizes) < total_m << 20:
+            sizes.append(int(round(np.exp(rng.uniform(np.log(2 ** 10), np.log(2 ** 21))))))
+        total, n = sum(sizes), len(sizes)
+        nblk = (total + 1023) // 1024
+        sets = []
+        for _ in range(3):
+            tensors = [torch.empty(k, dtype=torch.bfloat16, device="cuda:0").normal_() for k in sizes]
+            bucket = fp8.FlatBucket(tensors)
+            flat = bucket.pack()
+            q, sc = fp8.quantize(flat)
+            accs = [torch.zeros(k, device="cuda:0") for k in sizes]
+            outs = [torch.empty(k, device="cuda:0") for k in sizes]
+            sets.append(dict(bucket=bucket, tensors=tensors, flat=flat, q=q, s=sc, acc=torch.zeros(total, device="cuda:0"), accs=accs,
+                             outs=outs, aptrs=bucket.pointer_table(accs), optrs=bucket.pointer_table(outs),
+                             index=bucket.block_index().data_ptr()))
+        torch.cuda.synchronize()
+        cells = []
+        for stage in stages:
+            calls = []
+            for d in sets:
+                b = d["bucket"]
+                tables = (b.d_offsets.data_ptr(), n, total)
+                if stage == "flat_pack":
+                    nbytes = 4 * total
+                    calls.append(prepared("mhip_flat_pack", d["flat"].data_ptr(), b.d_ptrs.data_ptr(), *tables, 2, d["index"], STREAM()))
+                elif stage == "quantize":
+                    nbytes = 3 * total + 4 * nblk
+                    calls.append(prepared("mhip_fp8_quantize", d["q"].data_ptr(), d["s"].data_ptr(), d["flat"].data_ptr(), total, 1024, STREAM()))
+                elif stage == "quantize_bucket":
+                    nbytes = 3 * total + 4 * nblk
+                    calls.append(prepared("mhip_fp8_quantize_bucket", d["q"].data_ptr(), d["s"].data_ptr(), b.d_ptrs.data_ptr(), *tables, 1024,
+                                          d["index"], STREAM()))
+                elif stage == "dequant":
+                    nbytes = 9 * total + 4 * nblk
+                    calls.append(prepared("mhip_fp8_dequant_accumulate", d["acc"].data_ptr(), d["q"].data_ptr(), d["s"].data_ptr(), total, 1024,
+                                          STREAM()))
+                elif stage == "dequant_bucket":
+                    nbytes = 9 * total + 4 * nblk
+                    calls.append(prepared("mhip_fp8_dequant_accumulate_bucket", d["aptrs"].data_ptr(), d["q"].data_ptr(), d["s"].data_ptr(),
+                                          *tables, 1024, d["index"], STREAM()))
+                else:
+                    nbytes = 8 * total
+                    calls.append(prepared("mhip_flat_unpack", d["optrs"].data_ptr(), d["acc"].data_ptr(), *tables, 4, d["index"], STREAM()))
+            res = []
+            for _ in range(3):
+                for c in calls:
+                    assert c() == 0
+                torch.cuda.synchronize()
+                ev = Events(lib, stream)
+                ev.start()
+                for i in range(launches):
+                    calls[i % 3]()
+                res.append(ev.stop_ms() / launches * 1e3)
+            us = sorted(res)[1]
+            cells.append(f"{us:.1f} ({nbytes / us / 1e3 / HBM_PEAK_GBS:.2f})")
+        print(f"| {total} | {n} | " + " | ".join(cells) + " |", flush=True)
+        del sets, calls
+        torch.cuda.empty_cache()
+
+
 # The default run reports these beside the headline workload, measured in the same process:
 # workload -> fraction of HBM peak that BASELINE.json's north star asks of its class (None: no target stated)
 SUMMARY = {
@@ -1094,11 +1186,14 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views"], help="print an A/B table instead of the bench line")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views", "bucket_sizes"], help="print a table instead of the bench line")
     ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep == "bucket_sizes":
+        sweep_bucket_sizes()
+        return
     if args.sweep == "strided_views":
         sweep_strided_views([d for d in args.dtypes.split(",") if d != "f64"])
         return
