@@ -38,6 +38,40 @@ pub struct mhip_rdma_buffer_t {
     pub size: usize,
 }
 
+/// `rdmaxcel_sys::wqe_params_t` (`rdmaxcel-sys/src/rdmaxcel.h:26-39`): same fields, order and widths.
+#[repr(C)]
+#[derive(Debug, Clone, Copy)]
+pub struct mhip_wqe_params_t {
+    pub laddr: usize,
+    pub lkey: u32,
+    pub length: usize,
+    pub wr_id: u64,
+    pub signaled: bool,
+    pub op_type: u32,
+    pub raddr: usize,
+    pub rkey: u32,
+    pub qp_num: u32,
+    pub buf: *mut u8,
+    pub dbrec: *mut u32,
+    pub wqe_cnt: u32,
+}
+
+/// `rdmaxcel_sys::cqe_poll_params_t` (`rdmaxcel.h:42-48`).
+#[repr(C)]
+#[derive(Debug, Clone, Copy)]
+pub struct mhip_cqe_poll_params_t {
+    pub cqe_buf: *mut u8,
+    pub cqe_size: u32,
+    pub consumer_index: u32,
+    pub cqe_cnt: u32,
+    pub dbrec: *mut u32,
+}
+
+/// `MLX5_OPCODE_*` as `RdmaQueuePair::send_wqe` uses them (`monarch_rdma/src/rdma_components.rs:1119-1124`).
+pub const MHIP_MLX5_OPCODE_RDMA_WRITE: u32 = 0x08;
+pub const MHIP_MLX5_OPCODE_RDMA_WRITE_IMM: u32 = 0x09;
+pub const MHIP_MLX5_OPCODE_RDMA_READ: u32 = 0x10;
+
 /// `Option::None` of `WorkerActor::send_tensor`'s `from_rank` / `to_rank`.
 pub const MHIP_NO_RANK: u64 = u64::MAX;
 
@@ -67,6 +101,7 @@ pub mod status {
     pub const UNSUPPORTED_BLOCK: i32 = 10204;
     pub const BUFFER_TOO_SMALL: i32 = 10205;
     pub const SCRATCH_TOO_SMALL: i32 = 10206;
+    pub const WQE_OVERFLOW: i32 = 10207;
     pub const MESH_DIM_LENGTH_MISMATCH: i32 = 10301;
     pub const MESH_DIM_MISSING: i32 = 10302;
 }
@@ -133,6 +168,16 @@ extern "C" {
     pub fn mhip_send_tensor_route(from_ranks: *const mhip_slice_t, to_ranks: *const mhip_slice_t, rank: u64, from_rank: *mut u64, to_rank: *mut u64) -> c_int;
     pub fn mhip_to_mesh_from_ranks(slicing_names: *const *const c_char, slicing: *const mhip_slice_t, mesh_names: *const *const c_char, mesh_sizes: *const u64, mesh_ndim: u32, out_sizes: *mut u64, out_strides: *mut u64, out_ndim: *mut u32, broadcast_dims: *mut u32, n_broadcast: *mut u32, culprit: *mut u32) -> c_int;
     pub fn mhip_send_tensor(result: *mut c_void, result_bytes: usize, src_base: *const c_void, src_view: *const mhip_slice_t, elem_size: u32, staging: *mut c_void, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_send_wqe(params: *const mhip_wqe_params_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_recv_wqe(params: *const mhip_wqe_params_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_db_ring(dst: *mut c_void, src: *const c_void, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_ring_doorbells(dst: *mut c_void, sq_buf: *const c_void, stride: u32, wqe_cnt: u32, first_db_idx: u32, count: u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_cqe_poll(d_result: *mut i32, params: *const mhip_cqe_poll_params_t, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_post_transfer(params: *const mhip_wqe_params_t, max_segment_bytes: usize, n_wqes: *mut u32, stream: mhip_stream_t) -> c_int;
+    pub fn mhip_rdmaxcel_send_wqe_host(params: *const mhip_wqe_params_t) -> c_int;
+    pub fn mhip_rdmaxcel_recv_wqe_host(params: *const mhip_wqe_params_t) -> c_int;
+    pub fn mhip_rdmaxcel_db_ring_host(dst: *mut c_void, src: *const c_void) -> c_int;
+    pub fn mhip_rdmaxcel_cqe_poll_host(result: *mut i32, params: *const mhip_cqe_poll_params_t) -> c_int;
     pub fn mhip_fp8_quantize(q: *mut u8, scales: *mut f32, x_bf16: *const c_void, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate(acc: *mut f32, q: *const u8, scales: *const f32, numel: u64, block: u32, stream: mhip_stream_t) -> c_int;
     pub fn mhip_fp8_dequant_accumulate_many(acc: *mut f32, q: *const *const u8, scales: *const *const f32, n: u32, numel: u64, block: u32, overwrite: c_int, stream: mhip_stream_t) -> c_int;

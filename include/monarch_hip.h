@@ -62,6 +62,7 @@ enum {
     MHIP_ERR_UNSUPPORTED_BLOCK = 10204,
     MHIP_ERR_BUFFER_TOO_SMALL = 10205,
     MHIP_ERR_SCRATCH_TOO_SMALL = 10206,
+    MHIP_ERR_WQE_OVERFLOW = 10207,
     /* Tensor.to_mesh checks, python/monarch/common/tensor.py:426-437 */
     MHIP_ERR_MESH_DIM_LENGTH_MISMATCH = 10301,
     MHIP_ERR_MESH_DIM_MISSING = 10302
@@ -302,6 +303,98 @@ int mhip_to_mesh_from_ranks(const char* const* slicing_names, const mhip_slice_t
 int mhip_send_tensor(void* result, size_t result_bytes, const void* src_base,
                      const mhip_slice_t* src_view, uint32_t elem_size, void* staging,
                      mhip_stream_t stream);
+
+/* ====================================================================== */
+/* Device-initiated RDMA: work-queue and completion-queue entries (mlx5)   */
+/* ====================================================================== */
+/* The NIC-free half of rdmaxcel-sys: the queue memory is whatever the caller passes (the mlx5dv_qp /
+ * mlx5dv_cq buffers once they are mapped for the GPU, ordinary device or host memory otherwise); the
+ * library only builds and reads the entries.  Byte layouts are rdma-core's <infiniband/mlx5dv.h>
+ * (control, remote-address and data segments of 16 bytes each, big-endian fields; see
+ * monarch_hip_rdmaxcel_device.h, which holds the same functions for callers' own kernels).
+ * Registering queue memory for the GPU (register_cuda_memory, rdmaxcel-sys/src/rdmaxcel.c:147-207)
+ * and creating queue pairs are not part of this library. */
+
+/* wqe_params_t, rdmaxcel-sys/src/rdmaxcel.h:26-39: same fields, order and widths, hence the same
+ * 80-byte layout (signaled is the reference's bool). */
+typedef struct {
+    uintptr_t laddr;
+    uint32_t lkey;
+    size_t length;
+    uint64_t wr_id;
+    uint8_t signaled;
+    uint32_t op_type; /* MLX5_OPCODE_* */
+    uintptr_t raddr;
+    uint32_t rkey;
+    uint32_t qp_num;
+    uint8_t* buf;    /* send: mlx5dv_qp.sq.buf; receive: the slot itself */
+    uint32_t* dbrec; /* mlx5dv_qp.dbrec: [0] receive, [1] send */
+    uint32_t wqe_cnt;
+} mhip_wqe_params_t;
+/* cqe_poll_params_t, rdmaxcel.h:42-48 (32 bytes). */
+typedef struct {
+    uint8_t* cqe_buf;
+    uint32_t cqe_size;
+    uint32_t consumer_index;
+    uint32_t cqe_cnt;
+    uint32_t* dbrec;
+} mhip_cqe_poll_params_t;
+/* MLX5_OPCODE_* values RdmaQueuePair::send_wqe maps RdmaOperation to
+ * (monarch_rdma/src/rdma_components.rs:1119-1124). */
+enum { MHIP_MLX5_OPCODE_RDMA_WRITE = 0x08, MHIP_MLX5_OPCODE_RDMA_WRITE_IMM = 0x09, MHIP_MLX5_OPCODE_RDMA_READ = 0x10 };
+
+/* launch_send_wqe (rdmaxcel.h:93, rdmaxcel.cu:269-275; caller monarch_rdma/src/test_utils.rs:131-160):
+ * send_wqe (rdmaxcel.cu:201-245) as a kernel on `stream`.  Writes the 48 bytes of control, remote-address
+ * and data segment into slot (uint32)wr_id & (wqe_cnt - 1) of buf (64-byte slots; bytes 48-63 untouched)
+ * and then dbrec[1] = big-endian ((uint32)wr_id + 1) & 0xFFFFFF.  length is cut to 32 bits as in the
+ * reference.  Unlike the reference's launcher it does not synchronise the device.
+ * Refused with INVALID_ARGUMENT: NULL params / buf / dbrec, buf not 16-byte aligned, dbrec not 4-byte
+ * aligned, wqe_cnt zero or not a power of two. */
+int mhip_rdmaxcel_send_wqe(const mhip_wqe_params_t* params, mhip_stream_t stream);
+/* launch_recv_wqe (rdmaxcel.h:94, rdmaxcel.cu:184-190; caller test_utils.rs:162-189): recv_wqe
+ * (rdmaxcel.cu:139-160) as a kernel: one data segment at buf itself, then dbrec[0] = big-endian
+ * (uint32)(wr_id + 1).  wqe_cnt is not used. */
+int mhip_rdmaxcel_recv_wqe(const mhip_wqe_params_t* params, mhip_stream_t stream);
+/* launch_db_ring (rdmaxcel.h:78, rdmaxcel.cu:122-124; caller test_utils.rs:191-209): db_ring
+ * (rdmaxcel.cu:82-93) as a kernel: 64 bytes from src to dst as eight 64-bit stores in address order.
+ * Both 8-byte aligned. */
+int mhip_rdmaxcel_db_ring(void* dst, const void* src, mhip_stream_t stream);
+/* RdmaQueuePair::ring_doorbell's loop (rdma_components.rs:868-885; test_utils.rs:191-209) in one launch: for
+ * k = first_db_idx .. first_db_idx + count - 1 in order, db_ring(dst, sq_buf + (k % wqe_cnt) * stride), with a
+ * system-scope fence between rings.  count > wqe_cnt -> MHIP_ERR_WQE_OVERFLOW ("Overflow of WQE, possible data
+ * loss", rdma_components.rs:874-876).  stride is mlx5dv_qp.sq.stride, a multiple of 8 and at least 64. */
+int mhip_rdmaxcel_ring_doorbells(void* dst, const void* sq_buf, uint32_t stride, uint32_t wqe_cnt,
+                                 uint32_t first_db_idx, uint32_t count, mhip_stream_t stream);
+/* launch_cqe_poll (rdmaxcel.h:82-84, rdmaxcel.cu:358-395; caller test_utils.rs:211-257): cqe_poll
+ * (rdmaxcel.cu:292-326) as a kernel, ONE look at entry consumer_index & (cqe_cnt - 1), no spin.  The result
+ * goes to the caller's device word d_result instead of a managed allocation made and freed per poll:
+ * the byte count (big-endian word at byte 44 of the entry) when software owns the entry and its opcode is
+ * below 4, -2 when it owns it with any other opcode, untouched otherwise; the two owned cases also store
+ * big-endian (consumer_index + 1) & 0xFFFFFF at dbrec[0].  The caller sets *d_result to -1 before the call
+ * (rdmaxcel.cu:293,368) and reads it after the stream has reached the kernel's end: CQE_POLL_TRUE is
+ * *d_result >= 0 (rdmaxcel.cu:392).  Refused with INVALID_ARGUMENT: NULL pointers, cqe_size other than 64 or
+ * 128, cqe_cnt zero or not a power of two, cqe_buf / dbrec / d_result not 4-byte aligned. */
+int mhip_rdmaxcel_cqe_poll(int32_t* d_result, const mhip_cqe_poll_params_t* params, mhip_stream_t stream);
+
+/* A transfer of params->length bytes as a chain of send WQEs in one launch: WQE i (i = 0 .. n-1, n =
+ * ceil(length / max_segment_bytes)) is what send_wqe writes for {laddr + i*seg, raddr + i*seg,
+ * length_i = min(seg, rest), wr_id + i} with the other fields unchanged, and the doorbell record ends at
+ * ((uint32)wr_id + n) & 0xFFFFFF: the bytes n calls of mhip_rdmaxcel_send_wqe leave.  The reference posts
+ * one work request per call and cuts its length to 32 bits (rdma_components.rs:1041,1063, rdmaxcel.cu:229),
+ * so it has no counterpart for this; it is mhip_buffer_transfer's request walk for the device-initiated
+ * path.  max_segment_bytes == 0, or anything above it, means 2^31 - 16 (bit 31 of a data segment's byte
+ * count marks inline data in the mlx5 format).  *n_wqes (may be NULL) receives n.  n > wqe_cnt ->
+ * MHIP_ERR_WQE_OVERFLOW; length == 0 posts one zero-length WQE, as send_wqe would. */
+int mhip_rdmaxcel_post_transfer(const mhip_wqe_params_t* params, size_t max_segment_bytes,
+                                uint32_t* n_wqes, mhip_stream_t stream);
+
+/* The same functions on the calling thread, for queue memory the host can address: the reference's
+ * functions are __host__ __device__ and RdmaQueuePair calls them from Rust directly
+ * (send_wqe / recv_wqe: rdma_components.rs:1159-1163; db_ring: :88,:880).  Same bytes, same argument checks. */
+int mhip_rdmaxcel_send_wqe_host(const mhip_wqe_params_t* params);
+int mhip_rdmaxcel_recv_wqe_host(const mhip_wqe_params_t* params);
+int mhip_rdmaxcel_db_ring_host(void* dst, const void* src);
+int mhip_rdmaxcel_cqe_poll_host(int32_t* result, const mhip_cqe_poll_params_t* params);
 
 /* ====================================================================== */
 /* Block-scaled fp8 (e4m3fn) transfer codec                                 */

@@ -41,6 +41,7 @@ ERR_TOO_MANY_INPUTS = 10203
 ERR_UNSUPPORTED_BLOCK = 10204
 ERR_BUFFER_TOO_SMALL = 10205
 ERR_SCRATCH_TOO_SMALL = 10206
+ERR_WQE_OVERFLOW = 10207
 ERR_MESH_DIM_LENGTH_MISMATCH = 10301
 ERR_MESH_DIM_MISSING = 10302
 NO_RANK = (1 << 64) - 1
@@ -57,7 +58,8 @@ STATUS_NAMES = {
     ERR_INPUT_SIZE_MISMATCH: "InputSizeMismatch", ERR_UNDEFINED_TENSOR: "UndefinedTensor",
     ERR_INVALID_ARGUMENT: "InvalidArgument", ERR_UNSUPPORTED_OP: "UnsupportedOp",
     ERR_TOO_MANY_INPUTS: "TooManyInputs", ERR_UNSUPPORTED_BLOCK: "UnsupportedBlock",
-    ERR_BUFFER_TOO_SMALL: "BufferTooSmall", ERR_SCRATCH_TOO_SMALL: "ScratchTooSmall", ERR_MESH_DIM_LENGTH_MISMATCH: "MeshDimLengthMismatch",
+    ERR_BUFFER_TOO_SMALL: "BufferTooSmall", ERR_SCRATCH_TOO_SMALL: "ScratchTooSmall", ERR_WQE_OVERFLOW: "WqeOverflow",
+    ERR_MESH_DIM_LENGTH_MISMATCH: "MeshDimLengthMismatch",
     ERR_MESH_DIM_MISSING: "MeshDimMissing",
 }
 
@@ -86,6 +88,19 @@ class RdmaBufferC(C.Structure):
     _fields_ = [("addr", C.c_void_p), ("size", C.c_size_t)]
 
 
+class WqeParamsC(C.Structure):
+    """``mhip_wqe_params_t`` == ``wqe_params_t`` (rdmaxcel-sys/src/rdmaxcel.h:26-39)."""
+    _fields_ = [("laddr", C.c_size_t), ("lkey", C.c_uint32), ("length", C.c_size_t), ("wr_id", C.c_uint64),
+                ("signaled", C.c_uint8), ("op_type", C.c_uint32), ("raddr", C.c_size_t), ("rkey", C.c_uint32),
+                ("qp_num", C.c_uint32), ("buf", C.c_void_p), ("dbrec", C.c_void_p), ("wqe_cnt", C.c_uint32)]
+
+
+class CqePollParamsC(C.Structure):
+    """``mhip_cqe_poll_params_t`` == ``cqe_poll_params_t`` (rdmaxcel.h:42-48)."""
+    _fields_ = [("cqe_buf", C.c_void_p), ("cqe_size", C.c_uint32), ("consumer_index", C.c_uint32),
+                ("cqe_cnt", C.c_uint32), ("dbrec", C.c_void_p)]
+
+
 class SliceC(C.Structure):
     _fields_ = [("offset", C.c_uint64), ("ndim", C.c_uint32),
                 ("sizes", C.POINTER(C.c_uint64)), ("strides", C.POINTER(C.c_uint64))]
@@ -98,6 +113,8 @@ _vp = C.c_void_p
 _vpp = C.POINTER(C.c_void_p)
 _bufp = C.POINTER(RdmaBufferC)
 _cpp = C.POINTER(C.c_char_p)
+_wqep = C.POINTER(WqeParamsC)
+_cqep = C.POINTER(CqePollParamsC)
 
 # name -> (restype, argtypes); mirrors include/monarch_hip.h declaration by declaration
 SIGNATURES = {
@@ -138,6 +155,16 @@ SIGNATURES = {
     "mhip_send_tensor_route": (C.c_int, [_slicep, _slicep, C.c_uint64, _u64p, _u64p]),
     "mhip_to_mesh_from_ranks": (C.c_int, [_cpp, _slicep, _cpp, _u64p, C.c_uint32, _u64p, _u64p, _u32p, _u32p, _u32p, _u32p]),
     "mhip_send_tensor": (C.c_int, [_vp, C.c_size_t, _vp, _slicep, C.c_uint32, _vp, _vp]),
+    "mhip_rdmaxcel_send_wqe": (C.c_int, [_wqep, _vp]),
+    "mhip_rdmaxcel_recv_wqe": (C.c_int, [_wqep, _vp]),
+    "mhip_rdmaxcel_db_ring": (C.c_int, [_vp, _vp, _vp]),
+    "mhip_rdmaxcel_ring_doorbells": (C.c_int, [_vp, _vp, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, _vp]),
+    "mhip_rdmaxcel_cqe_poll": (C.c_int, [_vp, _cqep, _vp]),
+    "mhip_rdmaxcel_post_transfer": (C.c_int, [_wqep, C.c_size_t, _u32p, _vp]),
+    "mhip_rdmaxcel_send_wqe_host": (C.c_int, [_wqep]),
+    "mhip_rdmaxcel_recv_wqe_host": (C.c_int, [_wqep]),
+    "mhip_rdmaxcel_db_ring_host": (C.c_int, [_vp, _vp]),
+    "mhip_rdmaxcel_cqe_poll_host": (C.c_int, [C.POINTER(C.c_int32), _cqep]),
     "mhip_fp8_quantize": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate": (C.c_int, [_vp, _vp, _vp, C.c_uint64, C.c_uint32, _vp]),
     "mhip_fp8_dequant_accumulate_many": (C.c_int, [_vp, _vpp, _vpp, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int, _vp]),

@@ -59,6 +59,7 @@ const char* mhip_error_string(int status) {
         case MHIP_ERR_UNSUPPORTED_BLOCK: return "unsupported fp8 scale block (must be 1024)";
         case MHIP_ERR_BUFFER_TOO_SMALL: return "remote buffer is smaller than the transfer";
         case MHIP_ERR_SCRATCH_TOO_SMALL: return "input exceeds what the library's static scratch holds (2^20 - 1 blocks of 1024 elements)";
+        case MHIP_ERR_WQE_OVERFLOW: return "Overflow of WQE, possible data loss: more work requests than the queue has slots";
         case MHIP_ERR_MESH_DIM_LENGTH_MISMATCH: return "dimension of destination device_mesh has a different length than the source tensor";
         case MHIP_ERR_MESH_DIM_MISSING: return "destination mesh does not have a dimension of the source tensor";
         default: break;

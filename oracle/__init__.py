@@ -421,3 +421,49 @@ def flat_unpack(flat: np.ndarray, offsets: Sequence[int]) -> List[np.ndarray]:
     ptrs = (C.c_void_p * len(outs))(*[t.ctypes.data for t in outs])
     lib().o_flat_unpack(ptrs, _ptr(flat), _u64(offsets), C.c_uint32(len(outs)), C.c_uint32(flat.itemsize))
     return outs
+
+
+# ---- device-initiated RDMA: WQE / CQE byte images (rdmaxcel-sys/src/rdmaxcel.cu) ----
+class _CWqeParams(C.Structure):  # o_wqe_params_t
+    _fields_ = [("laddr", C.c_uint64), ("lkey", C.c_uint32), ("length", C.c_uint64), ("wr_id", C.c_uint64),
+                ("signaled", C.c_uint8), ("op_type", C.c_uint32), ("raddr", C.c_uint64), ("rkey", C.c_uint32),
+                ("qp_num", C.c_uint32), ("buf", C.c_void_p), ("dbrec", C.c_void_p), ("wqe_cnt", C.c_uint32)]
+
+
+class _CCqePollParams(C.Structure):  # o_cqe_poll_params_t
+    _fields_ = [("cqe_buf", C.c_void_p), ("cqe_size", C.c_uint32), ("consumer_index", C.c_uint32),
+                ("cqe_cnt", C.c_uint32), ("dbrec", C.c_void_p)]
+
+
+def _wqe_params(buf: np.ndarray, dbrec: np.ndarray, wqe_cnt: int, *, laddr=0, lkey=0, length=0, wr_id=0, signaled=True,
+                op_type=0, raddr=0, rkey=0, qp_num=0, buf_offset=0) -> _CWqeParams:
+    assert buf.dtype == np.uint8 and dbrec.dtype == np.uint32 and buf.flags.c_contiguous
+    return _CWqeParams(laddr, lkey, length, wr_id, 1 if signaled else 0, op_type, raddr, rkey, qp_num,
+                       buf.ctypes.data + buf_offset, dbrec.ctypes.data, wqe_cnt)
+
+
+def send_wqe(sq: np.ndarray, dbrec: np.ndarray, wqe_cnt: int, **fields) -> None:
+    """rdmaxcel.cu:201-245 on host arrays: ``sq`` (uint8, wqe_cnt * 64 bytes) and ``dbrec`` (2 x uint32)."""
+    p = _wqe_params(sq, dbrec, wqe_cnt, **fields)
+    lib().o_send_wqe(C.byref(p))
+
+
+def recv_wqe(rq_slot: np.ndarray, dbrec: np.ndarray, wqe_cnt: int, **fields) -> None:
+    """rdmaxcel.cu:139-160: the data segment goes to the first 16 bytes of ``rq_slot`` (+ ``buf_offset``)."""
+    p = _wqe_params(rq_slot, dbrec, wqe_cnt, **fields)
+    lib().o_recv_wqe(C.byref(p))
+
+
+def db_ring(dst: np.ndarray, src: np.ndarray) -> None:
+    """rdmaxcel.cu:82-93: 64 bytes from ``src`` to ``dst``."""
+    assert dst.dtype == np.uint8 and src.dtype == np.uint8 and dst.size >= 64 and src.size >= 64
+    lib().o_db_ring(C.c_void_p(dst.ctypes.data), C.c_void_p(src.ctypes.data))
+
+
+def cqe_poll(cq: np.ndarray, dbrec: np.ndarray, cqe_size: int, cqe_cnt: int, consumer_index: int, result: int = -1) -> int:
+    """rdmaxcel.cu:292-326: one look at the CQ; returns the byte count, -2 (bad opcode) or ``result`` untouched."""
+    assert cq.dtype == np.uint8 and dbrec.dtype == np.uint32
+    p = _CCqePollParams(cq.ctypes.data, cqe_size, consumer_index, cqe_cnt, dbrec.ctypes.data)
+    out = C.c_int32(result)
+    lib().o_cqe_poll(C.byref(out), C.byref(p))
+    return out.value

@@ -858,3 +858,124 @@ int o_num_threads(void) {
     return 1;
 #endif
 }
+
+/* ====================================================================================
+ * Device-initiated RDMA: work-queue and completion-queue entries (mlx5 wire format).
+ *
+ * Restates rdmaxcel-sys/src/rdmaxcel.cu:82-93 (db_ring), :139-160 (recv_wqe), :201-245
+ * (send_wqe) and :292-326 (cqe_poll) over ordinary host memory.  The segment layouts
+ * come from rdma-core's <infiniband/mlx5dv.h> (system package rdma-core-devel, no
+ * version pinned, README.md:83; absent from the reference tree and from this image),
+ * whose published layout is, in bytes, every multi-byte field big-endian:
+ *
+ *   mlx5_wqe_ctrl_seg  (16): 0-3 opmod_idx_opcode, 4-7 qpn_ds, 8 signature, 9-10 reserved
+ *                            (dci_stream_channel_id), 11 fm_ce_se, 12-15 imm
+ *                            (the reference repeats it at rdmaxcel-sys/src/lib.rs:22-31)
+ *   mlx5_wqe_raddr_seg (16): 0-7 raddr, 8-11 rkey, 12-15 reserved
+ *   mlx5_wqe_data_seg  (16): 0-3 byte_count, 4-7 lkey, 8-15 addr
+ *   MLX5_SEND_WQE_SHIFT 6 (64-byte send WQE slots), MLX5_RCV_DBR 0, MLX5_SND_DBR 1,
+ *   MLX5_WQE_CTRL_CQ_UPDATE 8 (2 << 2), MLX5_WQE_CTRL_SOLICITED 2 (1 << 1)
+ *   mlx5_cqe64: byte_cnt big-endian at byte 44, op_own in the last byte
+ *               (opcode in the upper 4 bits, ownership in bit 0)
+ *
+ * Pinning: the reference holds no byte vector of a WQE or CQE (its tests need two NICs,
+ * monarch_rdma/src/rdma_manager_actor_tests.rs:396-600): PARITY UNPINNED in the reference.
+ * Pinned here by known-answer bytes derived by hand from the layout above
+ * (tests/test_oracle_rdmaxcel.py).
+ *
+ * The functions below assemble every field byte by byte, most significant byte first, rather
+ * than swapping words, so that they share no code shape with the product's kernels.
+ * ==================================================================================== */
+typedef struct { /* wqe_params_t, rdmaxcel-sys/src/rdmaxcel.h:26-39 */
+    uint64_t laddr;
+    uint32_t lkey;
+    uint64_t length;
+    uint64_t wr_id;
+    uint8_t signaled;
+    uint32_t op_type;
+    uint64_t raddr;
+    uint32_t rkey;
+    uint32_t qp_num;
+    uint8_t* buf;
+    uint32_t* dbrec;
+    uint32_t wqe_cnt;
+} o_wqe_params_t;
+
+typedef struct { /* cqe_poll_params_t, rdmaxcel-sys/src/rdmaxcel.h:42-48 */
+    uint8_t* cqe_buf;
+    uint32_t cqe_size;
+    uint32_t consumer_index;
+    uint32_t cqe_cnt;
+    uint32_t* dbrec;
+} o_cqe_poll_params_t;
+
+static void put_be32(uint8_t* p, uint32_t v) {
+    p[0] = (uint8_t)(v >> 24);
+    p[1] = (uint8_t)(v >> 16);
+    p[2] = (uint8_t)(v >> 8);
+    p[3] = (uint8_t)v;
+}
+static void put_be64(uint8_t* p, uint64_t v) {
+    put_be32(p, (uint32_t)(v >> 32));
+    put_be32(p + 4, (uint32_t)v);
+}
+
+/* rdmaxcel.cu:82-93: eight 64-bit words, lowest address first. */
+void o_db_ring(void* dst, const void* src) {
+    for (int i = 0; i < 8; i++) memcpy((uint8_t*)dst + 8 * i, (const uint8_t*)src + 8 * i, 8);
+}
+
+/* rdmaxcel.cu:139-160: one data segment at params.buf itself (the caller addresses the slot);
+ * length and wr_id + 1 are cut to 32 bits by the 32-bit swap they are passed to (:148,:159). */
+void o_recv_wqe(const o_wqe_params_t* p) {
+    uint8_t seg[16];
+    put_be32(seg + 0, (uint32_t)p->length);
+    put_be32(seg + 4, p->lkey);
+    put_be64(seg + 8, p->laddr);
+    memcpy(p->buf, seg, 16);
+    put_be32((uint8_t*)&p->dbrec[0], (uint32_t)(p->wr_id + 1));
+}
+
+/* rdmaxcel.cu:201-245.  idx is wr_id cut to 32 bits (:206); the slot is idx & (wqe_cnt - 1)
+ * (:207) at 64 bytes per slot (:234); opmod_idx_opcode = (idx << 8) | op_type in 32 bits, so
+ * idx bits 24-31 fall off and bits 16-23 land in the opmod byte (:214); qpn_ds = qp_num << 8 | 3
+ * (:220); the three segments are zero-initialised (:202-204), so signature, the reserved bytes,
+ * imm and the raddr segment's last word are written as zeros; the send doorbell record takes
+ * (idx + 1) & 0xFFFFFF (:244). */
+void o_send_wqe(const o_wqe_params_t* p) {
+    const uint32_t idx = (uint32_t)p->wr_id;
+    const uint32_t slot = idx & (p->wqe_cnt - 1u);
+    uint8_t wqe[48];
+    memset(wqe, 0, sizeof wqe);
+    put_be32(wqe + 0, (idx << 8) | p->op_type);
+    put_be32(wqe + 4, (p->qp_num << 8) | 3u);
+    wqe[11] = p->signaled ? (uint8_t)(8 | 2) : 0;
+    put_be64(wqe + 16, p->raddr);
+    put_be32(wqe + 24, p->rkey);
+    put_be32(wqe + 32, (uint32_t)p->length);
+    put_be32(wqe + 36, p->lkey);
+    put_be64(wqe + 40, p->laddr);
+    memcpy(p->buf + ((uint64_t)slot << 6), wqe, 48);
+    put_be32((uint8_t*)&p->dbrec[1], (idx + 1u) & 0xFFFFFFu);
+}
+
+/* rdmaxcel.cu:292-326: one look at the entry consumer_index & (cqe_cnt - 1).  Software owns it
+ * when bit 0 of op_own equals the lap parity (consumer_index / cqe_cnt) & 1 and the opcode is not
+ * 0xF (:310-311); an owned entry whose opcode has either of its two upper bits set is an error
+ * (:314-315, -2), otherwise *byte_cnt receives the big-endian word at byte 44 as a signed 32-bit
+ * value (:318); both owned cases store (consumer_index + 1) & 0xFFFFFF big-endian at dbrec[0]
+ * (:319-324).  An entry that is not owned leaves *byte_cnt and the record alone. */
+void o_cqe_poll(int32_t* byte_cnt, const o_cqe_poll_params_t* p) {
+    const uint32_t idx = p->consumer_index;
+    const uint8_t* cqe = p->cqe_buf + (uint64_t)(idx & (p->cqe_cnt - 1u)) * p->cqe_size;
+    const uint8_t op_own = cqe[p->cqe_size - 1];
+    const uint8_t opcode = (uint8_t)(op_own >> 4);
+    const int owned = ((op_own & 1u) == ((idx / p->cqe_cnt) & 1u)) && opcode != 0xF;
+    if (!owned) return;
+    if ((opcode & 0xC) == 0) {
+        *byte_cnt = (int32_t)(((uint32_t)cqe[44] << 24) | ((uint32_t)cqe[45] << 16) | ((uint32_t)cqe[46] << 8) | cqe[47]);
+    } else {
+        *byte_cnt = -2;
+    }
+    put_be32((uint8_t*)&p->dbrec[0], (idx + 1u) & 0xFFFFFFu);
+}

@@ -124,6 +124,8 @@ _RUST_TYPE = {
     "uint8_t*": "*mut u8", "void*": "*mut c_void", "void* const*": "*const *mut c_void", "void**": "*mut *mut c_void",
     "const char*": "*const c_char", "const char* const*": "*const *const c_char", "uint32_t*": "*mut u32",
     "const mhip_rdma_buffer_t*": "*const mhip_rdma_buffer_t", "const size_t*": "*const usize",
+    "const mhip_wqe_params_t*": "*const mhip_wqe_params_t", "const mhip_cqe_poll_params_t*": "*const mhip_cqe_poll_params_t",
+    "int32_t*": "*mut i32",
 }
 
 

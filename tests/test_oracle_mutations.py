@@ -12,6 +12,7 @@ import pytest
 import oracle
 import test_oracle_collectives as K
 import test_oracle_numeric as T
+import test_oracle_rdmaxcel as R
 
 SRC = os.path.join(os.path.dirname(oracle.__file__), "monarch_oracle.c")
 
@@ -54,6 +55,43 @@ MUTATIONS = [
      K.test_stack_scatter_matches_reference_all_to_all_vector),
     ("send_route_swaps_the_sides", "o_send_tensor_route", "        *to_rank = peer;", "        *from_rank = peer;",
      K.test_send_tensor_result_is_the_contiguous_view),
+    # work-queue / completion-queue entries against the hand-derived bytes
+    ("send_wqe_slot_of_48_bytes", "o_send_wqe", "(uint64_t)slot << 6", "(uint64_t)slot * 48",
+     lambda: R.test_send_wqe_known_bytes_signaled_write(R.OracleImpl)),
+    ("send_wqe_flags_in_the_signature_byte", "o_send_wqe", "wqe[11] = p->signaled", "wqe[8] = p->signaled",
+     lambda: R.test_send_wqe_known_bytes_signaled_write(R.OracleImpl)),
+    ("send_wqe_lkey_before_byte_count", "o_send_wqe", "put_be32(wqe + 32, (uint32_t)p->length);\n    put_be32(wqe + 36, p->lkey);",
+     "put_be32(wqe + 36, (uint32_t)p->length);\n    put_be32(wqe + 32, p->lkey);",
+     lambda: R.test_send_wqe_known_bytes_signaled_write(R.OracleImpl)),
+    ("send_wqe_data_before_remote_address", "o_send_wqe", "put_be64(wqe + 16, p->raddr);\n    put_be32(wqe + 24, p->rkey);",
+     "put_be64(wqe + 40, p->raddr);\n    put_be32(wqe + 24, p->rkey);",
+     lambda: R.test_send_wqe_known_bytes_signaled_write(R.OracleImpl)),
+    ("send_wqe_record_without_24_bit_mask", "o_send_wqe", "(idx + 1u) & 0xFFFFFFu", "(idx + 1u)",
+     lambda: R.test_send_wqe_known_bytes_truncations_and_24_bit_record(R.OracleImpl)),
+    ("send_wqe_record_in_the_receive_word", "o_send_wqe", "&p->dbrec[1]", "&p->dbrec[0]",
+     lambda: R.test_send_wqe_known_bytes_signaled_write(R.OracleImpl)),
+    ("send_wqe_index_not_cut_to_24_bits_by_the_shift", "o_send_wqe", "put_be32(wqe + 0, (idx << 8) | p->op_type);",
+     "put_be32(wqe + 0, ((idx & 0xFFFFu) << 8) | p->op_type);",
+     lambda: R.test_send_wqe_known_bytes_truncations_and_24_bit_record(R.OracleImpl)),
+    ("little_endian_words", "put_be32", "p[0] = (uint8_t)(v >> 24);\n    p[1] = (uint8_t)(v >> 16);\n    p[2] = (uint8_t)(v >> 8);\n    p[3] = (uint8_t)v;",
+     "p[3] = (uint8_t)(v >> 24);\n    p[2] = (uint8_t)(v >> 16);\n    p[1] = (uint8_t)(v >> 8);\n    p[0] = (uint8_t)v;",
+     lambda: R.test_recv_wqe_known_bytes(R.OracleImpl)),
+    ("recv_wqe_record_masked_to_24_bits", "o_recv_wqe", "(uint32_t)(p->wr_id + 1)", "(uint32_t)(p->wr_id + 1) & 0xFFFFFFu",
+     lambda: R.test_recv_wqe_known_bytes(R.OracleImpl)),
+    ("recv_wqe_record_is_wr_id", "o_recv_wqe", "(uint32_t)(p->wr_id + 1)", "(uint32_t)(p->wr_id)",
+     lambda: R.test_recv_wqe_known_bytes(R.OracleImpl)),
+    ("cqe_poll_ignores_the_lap", "o_cqe_poll", "((idx / p->cqe_cnt) & 1u)", "0u",
+     lambda: R.test_cqe_poll_second_lap_large_entries_and_record_wrap(R.OracleImpl)),
+    ("cqe_poll_owns_opcode_15", "o_cqe_poll", " && opcode != 0xF", "",
+     lambda: R.test_cqe_poll_known_answers(R.OracleImpl)),
+    ("cqe_poll_accepts_opcodes_up_to_7", "o_cqe_poll", "(opcode & 0xC) == 0", "(opcode & 0x8) == 0",
+     lambda: R.test_cqe_poll_known_answers(R.OracleImpl)),
+    ("cqe_poll_op_own_at_byte_63_of_large_entries", "o_cqe_poll", "cqe[p->cqe_size - 1]", "cqe[63]",
+     lambda: R.test_cqe_poll_second_lap_large_entries_and_record_wrap(R.OracleImpl)),
+    ("cqe_poll_error_leaves_the_record", "o_cqe_poll", "        *byte_cnt = -2;\n    }", "        *byte_cnt = -2;\n        return;\n    }",
+     lambda: R.test_cqe_poll_known_answers(R.OracleImpl)),
+    ("db_ring_copies_56_bytes", "o_db_ring", "i < 8", "i < 7",
+     lambda: R.test_db_ring_copies_exactly_64_bytes(R.OracleImpl)),
 ]
 
 
