@@ -817,7 +817,8 @@ WORKLOADS = {
 
 
 SWEEPS = {
-    # name -> (environment variable the library reads at every call, {column: value or None for the library's choice})
+    # name -> (environment variable the library reads at every call when MONARCH_HIP_TUNING=1 was set at load time,
+    #          {column: value or None for the library's choice})
     "transpose_walks": ("MONARCH_HIP_TRANSPOSE_WALK",
                         {"library": None, "blocked 4": "0,1,4,0", "blocked 4 rot": "0,1,4,1", "blocked 8": "0,1,8,0",
                          "blocked 8 rot": "0,1,8,1", "blocked 16": "0,1,16,0", "packed fastest": "1,0", "memory fastest": "2,0",
@@ -866,6 +867,7 @@ def sweep_transpose(which, dtypes, reps=5, launches=30):
     library reads at every call, medians of `reps` alternations of `launches` launches, three rotating buffer sets.
     Prints one Markdown table per element size: fraction of HBM peak per variant."""
     envvar, variants = SWEEPS[which]
+    os.environ["MONARCH_HIP_TUNING"] = "1"  # the library looks at its tuning variables only when this is set while it loads
     torch, lib, _ = _load()
     from monarch_amd import Slice
     torch.cuda.set_device(0)

@@ -44,9 +44,14 @@ __global__ __launch_bounds__(kThreads) void bucket_index_kernel(uint32_t* __rest
 // All 64 lanes call it with the same arguments.
 __device__ __forceinline__ void span_tensors(const BucketArgs& a, uint64_t begin, uint64_t end, uint32_t* t_lo, uint32_t* t_hi) {
     if (a.index != nullptr) {
-        const uint32_t lo = a.index[begin / kBlock];
+        // clamped: an index that was built for another bucket, or that another call on this GPU is rewriting (the
+        // library's static index is shared), must not send the table reads out of bounds
+        const uint32_t last = a.ntensors - 1;
+        uint32_t lo = a.index[begin / kBlock];
+        lo = lo < last ? lo : last;
+        uint32_t hi = a.offsets[lo + 1] >= end ? lo : a.index[(end + kBlock - 1) / kBlock];
         *t_lo = lo;
-        *t_hi = a.offsets[lo + 1] >= end ? lo : a.index[(end + kBlock - 1) / kBlock];
+        *t_hi = hi < last ? hi : last;
     } else {
         wave_find_tensor_pair(a.offsets, 1, 0, a.ntensors, begin, end - 1, t_lo, t_hi);
     }
@@ -619,21 +624,28 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static uint32_t* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until looked up
 
-// Address of the current device's copy of `scratch`; the caller has made the launch device current.
-static int static_index_for_current_device(uint32_t** out) {
+// Address of the current device's copy of `scratch`; the caller has made the launch device current.  The look-up
+// happens once per device: from mhip_set_device / mhip_stream_create (the set-up calls of a process that uses this
+// library), or else from the first call of the entry point on that device.  `capturing`: the look-up is not a stream
+// operation and loads the device's code object the first time, so it must not fall inside a stream capture; a first
+// call under capture is refused instead.
+static int static_index_for_current_device(uint32_t** out, bool capturing) {
     int dev = -1;
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= kMaxDevices) return MHIP_ERR_INVALID_DEVICE;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        if (capturing) return (int)hipErrorStreamCaptureUnsupported;
         uint32_t* ptr = nullptr;
         if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
         if (ptr == nullptr) return MHIP_ERR_INVALID_DEVICE;
         g_scratch_ptr[dev] = ptr;
     }
-    *out = g_scratch_ptr[dev];
+    if (out) *out = g_scratch_ptr[dev];
     return MHIP_SUCCESS;
 }
+
+int prepare_static_scratch() { return static_index_for_current_device(nullptr, false); }
 
 }  // namespace mhip
 
@@ -681,7 +693,9 @@ int mhip_fp8_quantize_bucket_static(uint8_t* q, float* scales, const void* const
     hipStream_t hs = static_cast<hipStream_t>(stream);
     DeviceGuard guard(hs);
     uint32_t* index = nullptr;
-    if (int rc = static_index_for_current_device(&index)) return rc;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hs != nullptr && hipStreamIsCapturing(hs, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
+    if (int rc = static_index_for_current_device(&index, capture != hipStreamCaptureStatusNone)) return rc;
     // every entry the quantiser reads is rewritten by this build, so nothing of an earlier call has to be cleared
     if (int rc = build_bucket_index(index, d_offsets, ntensors, total, hs)) return rc;
     return quantize_bucket(q, scales, d_tensors, d_offsets, ntensors, total, index, hs);

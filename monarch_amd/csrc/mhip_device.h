@@ -243,23 +243,21 @@ private:
     bool restore_ = false;
 };
 
+// The library reads the process environment exactly once, while it is being loaded (runtime.cpp), never from an
+// entry point: getenv races with a setenv of the host application on another thread, and a stray variable must not
+// change which kernel a production process runs.  MONARCH_HIP_TUNING=1 at load time switches the tuning aids on: only
+// then does tuning_env() look a variable up, at every call, so that an A/B sweep can switch variants inside one process.
+extern const bool g_tuning;
+extern const uint64_t g_max_launch_lanes;
+inline const char* tuning_env(const char* name) { return g_tuning ? std::getenv(name) : nullptr; }
+
 // The runtime forms the global size of a launch (workgroups x lanes) in 32 bits.  A launch of exactly
 // 2^32 lanes is refused, and a larger one wraps silently: (2^26 + 1) workgroups of 64 lanes ran as ONE
 // workgroup and reported success.  Every host launch therefore keeps its grid at or below this bound;
 // grid-stride kernels clamp to it, one-shot kernels are launched in several pieces.
-// MONARCH_HIP_MAX_LAUNCH_LANES lowers the bound (a test aid: it drives small inputs through the
-// clamped and multi-piece paths).
-inline uint64_t max_launch_lanes() {
-    static const uint64_t limit = [] {
-        uint64_t v = 0xffffffffull;
-        if (const char* e = std::getenv("MONARCH_HIP_MAX_LAUNCH_LANES")) {
-            const unsigned long long x = std::strtoull(e, nullptr, 10);
-            if (x >= 8192 && x < v) v = x;
-        }
-        return v;
-    }();
-    return limit;
-}
+// With the tuning aids on, MONARCH_HIP_MAX_LAUNCH_LANES (read at load) lowers the bound: a test aid that drives
+// small inputs through the clamped and multi-piece paths.
+inline uint64_t max_launch_lanes() { return g_max_launch_lanes; }
 inline uint64_t max_workgroups(uint32_t lanes) { return max_launch_lanes() / lanes; }
 
 // Every kernel of the library is launched through MHIP_LAUNCH, which keeps the launch's own return value in a
@@ -284,7 +282,7 @@ inline void launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size
     static_assert(sizeof...(Params) == sizeof...(Args) && sizeof...(Params) > 0, "argument count");
     const hipError_t e = launch_kernel_impl(kernel, grid, block, lds_bytes, stream, std::index_sequence_for<Params...>{},
                                             std::forward<Args>(args)...);
-    if (e != hipSuccess) last_launch_error() = e;  // the first failure of a multi-piece launch stays visible
+    if (e != hipSuccess && last_launch_error() == hipSuccess) last_launch_error() = e;  // the first failure of several launches stays
 }
 #define MHIP_LAUNCH(kernel, grid, block, lds_bytes, stream, ...) \
     ::mhip::launch_kernel(kernel, grid, block, lds_bytes, stream, __VA_ARGS__)

@@ -49,4 +49,8 @@ bool same_shape(const CanonSlice& a, const CanonSlice& b);
 constexpr int kCopyManyMax = 64;
 int copy_many(void* const* dst, const void* const* src, const uint64_t* nbytes, uint32_t n, void* stream);
 
+// Looks up, once per device, the address of the library's static scratch array on the CURRENT device (the block index
+// of mhip_fp8_quantize_bucket_static).  Called from the set-up entry points so that the data path never does it.
+int prepare_static_scratch();
+
 }  // namespace mhip

@@ -561,6 +561,7 @@ __global__ __launch_bounds__(THREADS) void flat_copy_kernel(FlatArgs a) {
         if (u_last >= a.total) u_last = a.total - 1;
         // index[b] holds the tensor of element b * 1024, which is at or before the tensor of this tile's first unit
         uint32_t lo = a.index[(u_first / a.units_per_elem) >> 10];
+        if (lo >= a.ntensors) lo = a.ntensors - 1;  // an index built for another bucket must not send loads out of the tables
         while (lo + 1 < a.ntensors && a.offsets[lo + 1] * a.units_per_elem <= u_first) ++lo;
         uint32_t hi = lo;
         if (lo + 1 < a.ntensors && a.offsets[lo + 1] * a.units_per_elem <= u_last)
@@ -1014,6 +1015,7 @@ static int flat_copy_entry(char* flat, char* const* d_tensors, const uint64_t* d
     if (elem_size == 0) return MHIP_ERR_INVALID_ARGUMENT;
     if (ntensors == 0 || total == 0) return MHIP_SUCCESS;
     if (!flat || !d_tensors || !d_offsets) return MHIP_ERR_UNDEFINED_TENSOR;
+    if ((uintptr_t)d_index & 3u) return MHIP_ERR_INVALID_ARGUMENT;
     // unit: the power-of-two part of the element size, limited by the flat buffer's alignment
     uint32_t unit = 16;
     while (unit > 1 && ((elem_size | (uintptr_t)flat) & (unit - 1))) unit >>= 1;

@@ -1,13 +1,31 @@
 // Runtime pass-through and error text: the small part of the HIP runtime that the
 // data path's callers reach through this library instead of through cuda-sys/nccl-sys.
 #include <cstdint>
+#include <cstdlib>
 #include <hip/hip_runtime.h>
 
 #include "mhip_device.h"
+#include "mhip_internal.h"
 
 #define MHIP_VERSION 100
 
 namespace mhip {
+
+// The only two reads of the environment in the library; both run while the library is loaded.
+const bool g_tuning = [] {
+    const char* e = std::getenv("MONARCH_HIP_TUNING");
+    return e != nullptr && e[0] == '1' && e[1] == '\0';
+}();
+const uint64_t g_max_launch_lanes = [] {
+    uint64_t v = 0xffffffffull;
+    if (const char* e = std::getenv("MONARCH_HIP_TUNING"); e != nullptr && e[0] == '1' && e[1] == '\0') {
+        if (const char* m = std::getenv("MONARCH_HIP_MAX_LAUNCH_LANES")) {
+            const unsigned long long x = std::strtoull(m, nullptr, 10);
+            if (x >= 8192 && x < v) v = x;
+        }
+    }
+    return v;
+}();
 
 // Byte fill as a kernel rather than hipMemsetAsync: memset nodes recorded into a HIP graph have produced wrong
 // results on replays after the first on this platform, kernel nodes have not, and callers may capture this call
@@ -71,7 +89,10 @@ const char* mhip_error_string(int status) {
 int mhip_version(void) { return MHIP_VERSION; }
 
 int mhip_device_count(int* count) { return count ? (int)hipGetDeviceCount(count) : MHIP_ERR_INVALID_ARGUMENT; }
-int mhip_set_device(int device) { return (int)hipSetDevice(device); }
+int mhip_set_device(int device) {
+    if (hipError_t e = hipSetDevice(device); e != hipSuccess) return (int)e;
+    return prepare_static_scratch();  // so that no data-path call, possibly under stream capture, has to look it up
+}
 int mhip_device_synchronize(void) { return (int)hipDeviceSynchronize(); }
 
 int mhip_stream_create(mhip_stream_t* stream) {
@@ -79,7 +100,8 @@ int mhip_stream_create(mhip_stream_t* stream) {
     hipStream_t s = nullptr;
     hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);  // default priority
     *stream = s;
-    return (int)e;
+    if (e != hipSuccess) return (int)e;
+    return prepare_static_scratch();  // the stream's device is the current one
 }
 int mhip_stream_destroy(mhip_stream_t stream) { return (int)hipStreamDestroy(static_cast<hipStream_t>(stream)); }
 int mhip_stream_synchronize(mhip_stream_t stream) { return (int)hipStreamSynchronize(static_cast<hipStream_t>(stream)); }

@@ -586,12 +586,12 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
 // Streaming stores of rows that are not 16-byte aligned write partial lines (u8 5000 x 7000: 0.57 -> 0.42), so rows like
 // that keep going through the cache, which combines what neighbouring tiles share; streaming loads need both sides
 // aligned for the same reason.
-// MONARCH_HIP_TRANSPOSE_POLICY overrides the choice (tuning aid, read at every call): 0 cached loads + write-through /
+// With the tuning aids on (MONARCH_HIP_TUNING=1 when the library was loaded), MONARCH_HIP_TRANSPOSE_POLICY overrides the choice at every call: 0 cached loads + write-through /
 // cached stores, 1 streaming loads + streaming stores, 2 streaming loads only, 3 streaming stores only.
 static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint64_t packed_bytes, bool stores_aligned, bool both_sides_aligned) {
     if (stores_aligned) a->aligned_stores = kStoreStreaming;
     if (both_sides_aligned && packed_bytes >= (120ull << 20)) *stream_loads = true;
-    if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_POLICY")) {
+    if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_POLICY")) {
         const int p = std::atoi(e);
         *stream_loads = p == 1 || p == 2;
         a->aligned_stores = (p == 1 || p == 3) ? kStoreStreaming : stores_aligned ? kStoreWriteThrough : kStoreCached;
@@ -608,7 +608,7 @@ static void choose_cache_policy(TransArgs* a, bool* stream_loads, uint64_t packe
 //     0.03 with it and keep the blocked walk;
 //   * at every other pitch the rows of a tile spread by themselves, neighbouring tiles share partial cache lines, and
 //     the blocked XCD-contiguous walk wins (the diagonal one loses 0.02 to 0.10 there).
-// MONARCH_HIP_TRANSPOSE_WALK overrides the choice (a tuning aid, read at every call so that variants can be
+// With the tuning aids on, MONARCH_HIP_TRANSPOSE_WALK overrides the choice at every call (so that variants can be
 // switched in turn inside one process): "<walk>[,<xcd_ranges>[,<group>[,<rotate>]]]" with walk 0 blocked,
 // 1 packed side fastest, 2 memory side fastest, 3 diagonal.
 static void choose_walk(TransArgs* a, uint32_t unit, uint64_t nbatch) {
@@ -620,7 +620,7 @@ static void choose_walk(TransArgs* a, uint32_t unit, uint64_t nbatch) {
         a->xcd_ranges = 0;
         a->rotate = 0;
     }
-    if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_WALK")) {
+    if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_WALK")) {
         unsigned walk = 0, ranges = 1, group = a->group, rotate = 0;
         const int n = std::sscanf(e, "%u,%u,%u,%u", &walk, &ranges, &group, &rotate);
         if (n >= 1 && walk <= kWalkDiagonal) {
@@ -706,7 +706,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     const uint32_t tile = vec ? (big ? 512 : 256) / unit : 32;
     // Written rows that do not start on cache lines take the kernel whose windows do (slice_transpose_lines_kernel):
     // the extent along the written rows grows by the most a window can start early.
-    // MONARCH_HIP_TRANSPOSE_LINES=0 / 1 overrides the choice (a tuning aid, read at every call).
+    // With the tuning aids on, MONARCH_HIP_TRANSPOSE_LINES=0 / 1 overrides the choice at every call.
     bool lines = false;
     if (vec && !big && unit >= 2 && (PACK ? Sc : Q) >= tile) {  // 1-byte elements lose with it (8200^2 0.475 -> 0.36: 96 KiB of LDS, byte-wise LDS reads)
         uint64_t written = PACK ? ((uint64_t)(uintptr_t)packed | Q * unit) : ((uint64_t)(uintptr_t)base + c.offset * unit);
@@ -714,7 +714,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
             for (int k = 0; k < c.ndim; ++k)
                 if (k != cd) written |= c.dims[k].stride * unit;
         lines = (written & 127u) != 0;
-        if (const char* e = std::getenv("MONARCH_HIP_TRANSPOSE_LINES")) lines = std::atoi(e) != 0;
+        if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_LINES")) lines = std::atoi(e) != 0;
     }
     const uint32_t early = lines ? 128 / unit - 1 : 0;
     a.base = base;

@@ -645,13 +645,11 @@ def test_transposing_views_interior_and_edge_tiles(dtype):
         assert torch.equal(back.cpu(), ref), (shape, dtype)
 
 
-@pytest.mark.parametrize("lines", ["0", "1"])
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
-def test_transposes_with_line_aligned_windows_and_without(dtype, lines, monkeypatch):
-    # written rows that start anywhere in a cache line, through the kernel whose windows start on lines and through
-    # the fixed-position tiles: extents of exactly one tile, of a tile and a bit, shorter than the early start of a
+def test_transposes_whose_written_rows_start_inside_cache_lines(dtype):
+    # written rows that start anywhere in a cache line, with the kernel the library picks for them (both kernels, forced
+    # in turn, run in tests/tuning_variants.py): extents of exactly one tile, of a tile and a bit, shorter than the early start of a
     # window, batches, offsets, a packed side spanning two dimensions
-    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_LINES", lines)
     g = torch.Generator().manual_seed(18)
     info = torch.iinfo(dtype)
     t = 256 // torch.empty(0, dtype=dtype).element_size()
@@ -801,56 +799,3 @@ def test_stream_send_tensor_semantics():
         stream_send_tensor(world, 0, None, None, f)
     fr, to = Slice(offset=0, sizes=[2], strides=[1]), Slice(offset=2, sizes=[2], strides=[1])
     assert route(fr, to, 3) == (1, None)
-
-
-@pytest.mark.parametrize("walk", ["0,1,4,0", "0,1,4,1", "0,1,16,1", "0,0,8,0", "1,0", "1,1", "2,0", "2,1", "3,0", "3,1"])
-def test_every_tile_walk_of_the_transposing_kernel_moves_the_same_bytes(walk, monkeypatch):
-    # the library picks one walk per shape; every walk it can pick (and the variants the A/B sweep forces) must give the
-    # same bytes: whole and partial tiles, batches, a tile count that is no multiple of 8, pitches that are and are not
-    # multiples of 4 KiB
-    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_WALK", walk)
-    g = torch.Generator().manual_seed(sum(walk.encode()))
-    cases = [(torch.int16, (1, 256, 384, 384)), (torch.int16, (3, 200, 333, 340)), (torch.int32, (1, 192, 64, 64)),
-             (torch.int32, (2, 130, 257, 300)), (torch.uint8, (1, 512, 768, 768)), (torch.uint8, (2, 300, 515, 600)),
-             (torch.int64, (1, 96, 160, 160)), (torch.int32, (1, 1024, 2048, 2048)), (torch.int16, (1, 2048, 1024, 2048))]
-    for dtype, (b, r, c, pitch) in cases:
-        info = torch.iinfo(dtype)
-        host = torch.randint(info.min, info.max, (b, r, pitch), dtype=dtype, generator=g)
-        dev = host.to(DEV)
-        view, hview = dev[:, :, :c].transpose(1, 2), host[:, :, :c].transpose(1, 2)
-        s = Slice.of_tensor(view)
-        out = staging.pack(view, s)
-        sync()
-        assert torch.equal(out.cpu(), hview.contiguous().flatten()), (walk, dtype, b, r, c, pitch)
-        back = torch.zeros_like(dev)
-        staging.unpack(back, s, out)
-        sync()
-        ref = torch.zeros_like(host)
-        ref[:, :, :c] = host[:, :, :c]
-        assert torch.equal(back.cpu(), ref), (walk, dtype, b, r, c, pitch)
-
-
-@pytest.mark.parametrize("policy", ["0", "1", "2", "3"])
-def test_every_cache_policy_of_the_transposing_kernel_moves_the_same_bytes(policy, monkeypatch):
-    # cached / write-through / streaming loads and stores, forced on aligned and unaligned rows alike (the library only
-    # streams aligned rows; correctness must not depend on that)
-    monkeypatch.setenv("MONARCH_HIP_TRANSPOSE_POLICY", policy)
-    g = torch.Generator().manual_seed(40 + int(policy))
-    cases = [(torch.int32, (1, 523, 772, 777)), (torch.int16, (2, 300, 515, 600)), (torch.uint8, (1, 512, 768, 768)),
-             (torch.int64, (1, 96, 160, 160)), (torch.int32, (1, 1024, 2048, 2048)), (torch.int16, (1, 515, 260, 261))]
-    for dtype, (b, r, c, pitch) in cases:
-        info = torch.iinfo(dtype)
-        host = torch.randint(info.min, info.max, (b, r, pitch), dtype=dtype, generator=g)
-        dev = host.to(DEV)
-        view, hview = dev[:, :, :c].transpose(1, 2), host[:, :, :c].transpose(1, 2)
-        s = Slice.of_tensor(view)
-        for rep in range(3):
-            out = staging.pack(view, s)
-            sync()
-            assert torch.equal(out.cpu(), hview.contiguous().flatten()), (policy, dtype, b, r, c, pitch, rep)
-        back = torch.zeros_like(dev)
-        staging.unpack(back, s, out)
-        sync()
-        ref = torch.zeros_like(host)
-        ref[:, :, :c] = host[:, :, :c]
-        assert torch.equal(back.cpu(), ref), (policy, dtype, b, r, c, pitch)

@@ -173,7 +173,7 @@ def test_cqe_poll_result_word_is_left_alone_when_not_owned():
 def test_post_transfer_equals_sequential_send_wqes():
     L = lib()
     rng = np.random.default_rng(5)
-    for cnt, length, seg, wr_id in [(8, 5 * 4096 + 17, 4096, 0), (8, 8 * 4096, 4096, 6), (4, 0, 0, 3), (2, 1 << 33, 0, 0xFFFFFF),
+    for cnt, length, seg, wr_id in [(8, 5 * 4096 + 17, 4096, 0), (8, 8 * 4096, 4096, 6), (4, 0, 0, 3), (8, 1 << 33, 0, 0xFFFFFF),
                                     (2048, 1500 * 8192 - 5, 8192, 0x00FFFFF0), (16, 3 << 30, 1 << 30, 14), (4, 100, 1 << 40, 1)]:
         f = random_fields(rng)
         f.update(length=length, wr_id=wr_id)

@@ -71,3 +71,37 @@ def test_static_index_entry_point_refuses_what_does_not_fit():
     assert lib.mhip_fp8_quantize_bucket_static(16, 16, 16, 16, 1, 100, 512, None) == _lib.ERR_UNSUPPORTED_BLOCK
     assert lib.mhip_fp8_quantize_bucket_static(None, 16, 16, 16, 1, 100, 1024, None) == _lib.ERR_UNDEFINED_TENSOR
     assert lib.mhip_fp8_quantize_bucket_static(None, None, None, None, 0, 0, 1024, None) == 0
+
+
+def test_static_index_entry_point_records_into_a_graph_and_allocates_nothing():
+    # the callers it exists for: code under stream capture.  The scratch address is resolved at set-up
+    # (mhip_set_device / mhip_stream_create, or an earlier call), so the captured call only launches kernels; every
+    # replay, with new tensor contents and eager work in between, equals the eager mhip_fp8_quantize_bucket.
+    lib = _lib.lib()
+    assert lib.mhip_set_device(0) == 0
+    sizes = [5000, 1, 1024, 777, 30000, 2049]
+    tensors, d_ptrs, d_offs, total = _bucket(sizes, 11)
+    nblk = (total + 1023) // 1024
+    q = torch.zeros(total, dtype=torch.uint8, device=DEV)
+    s = torch.zeros(nblk, dtype=torch.float32, device=DEV)
+    q_ref, s_ref = torch.zeros_like(q), torch.zeros_like(s)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        rc = lib.mhip_fp8_quantize_bucket_static(q.data_ptr(), s.data_ptr(), d_ptrs.data_ptr(), d_offs.data_ptr(), len(sizes), total,
+                                                 1024, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.cuda.mem_get_info()[0] >= free_before - (2 << 20)   # the call took no device memory (the graph itself: a little)
+    for rep in range(3):
+        g = torch.Generator().manual_seed(100 + rep)
+        for t in tensors:
+            t.copy_(torch.randn(t.numel(), generator=g).bfloat16())
+        other = torch.randn(1 << 18, device=DEV).sum()                # unrelated eager work between replays
+        graph.replay()
+        assert lib.mhip_fp8_quantize_bucket(q_ref.data_ptr(), s_ref.data_ptr(), d_ptrs.data_ptr(), d_offs.data_ptr(), len(sizes), total,
+                                            1024, None, torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32)), rep
+        assert torch.isfinite(other)
