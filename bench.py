@@ -1102,8 +1102,26 @@ SUMMARY = {
 }
 
 
+def sig(x, digits=4):
+    """x rounded to `digits` significant digits (the bench line has to stay short enough for the driver's tail)."""
+    if x is None or x == 0 or x != x:
+        return x
+    from math import floor, log10
+    return round(x, digits - 1 - floor(log10(abs(x))))
+
+
+INFINITY_CACHE_BYTES = 256 << 20
+# workloads that are pipelines of launches in which a kernel reads what the one before it has just written
+PIPELINES = ("c3_reshard_e2e", "c3_reshard_e2e_one_by_one", "c1_pipeline", "c1_pipeline_fused")
+
+
 def measure(torch, lib, workload: str, steps: int, warmup: int):
+    torch.cuda.synchronize()
+    held_before = torch.cuda.memory_allocated()
     name, nbytes, launch, cpu, kernel, dtype = WORKLOADS[workload](torch)
+    # device memory of the workload's rotating buffer sets: what one rotation walks through.  (The C5 stages share one
+    # set of buffers made by the first of them; each of their launches alone moves 3 GB and more.)
+    rotation = max(torch.cuda.memory_allocated() - held_before, nbytes)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = 0
     for i in range(warmup):
@@ -1119,8 +1137,21 @@ def measure(torch, lib, workload: str, steps: int, warmup: int):
         sys.exit(f"a launch of {workload} returned status {rc}")
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # a figure quoted against the HBM peak is cache-assisted when a rotation is short enough for a good part of it to stay
+    # in the 256 MB Infinity Cache, or when a kernel of the step reads what the previous one wrote
+    assisted = rotation < 2 * INFINITY_CACHE_BYTES or workload in PIPELINES
     return dict(name=name, nbytes=nbytes, cpu=cpu, kernel=kernel, dtype=dtype, kernel_ms=kernel_ms, wall_ms=wall_ms,
-                keep=launch)
+                keep=launch, rotation=rotation, cache_assisted=assisted)
+
+
+def short_cpu(cpu: dict) -> dict:
+    """A workload's CPU legs as GB/s figures only: 1-core port of the reference loop, the same on all cores, torch CPU."""
+    out = {"port": sig(cpu["value"], 3)}
+    if "all_cores" in cpu:
+        out["all_cores"] = sig(cpu["all_cores"]["value"], 3)
+    if "torch_cpu" in cpu:
+        out["torch"] = sig(cpu["torch_cpu"]["value"], 3)
+    return out
 
 
 def run(workload: str, steps: int, warmup: int, cpu_baseline: bool, summary: bool = False):
@@ -1131,32 +1162,38 @@ def run(workload: str, steps: int, warmup: int, cpu_baseline: bool, summary: boo
     nbytes = m["nbytes"]
     achieved = nbytes / (m["kernel_ms"] * 1e-3) / 1e9
     rec = {
-        "metric": METRIC, "value": nbytes / (m["wall_ms"] * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1,
-        "steps": steps, "warmup": warmup, "ms_per_step": m["wall_ms"], "higher_is_better": True,
+        "metric": METRIC, "value": sig(nbytes / (m["wall_ms"] * 1e-3) / 1e9, 6), "unit": "GB/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": sig(m["wall_ms"], 6), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": m["dtype"], "data": "synthetic",
         "config": {"workload": m["name"], "algorithmic_bytes_per_step": nbytes, "kernel": m["kernel"],
                    **({"layout": LAYOUT[workload]} if workload in LAYOUT else {})},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic.get(workload, {}).get("traffic"),
-                     "traffic_source": TRAFFIC_SOURCE},
+        "roofline": {"bound": "hbm", "achieved": sig(achieved, 6), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": sig(achieved, 6) / HBM_PEAK_GBS, "traffic": traffic.get(workload, {}).get("traffic"),
+                     "traffic_source": TRAFFIC_SOURCE,
+                     # what one rotation of the buffer sets walks through; under 2 x 256 MB part of it stays in the
+                     # Infinity Cache.  frac_cold: the same kernel rotating over 8 sets (3.6 GB), filled in by the default run
+                     "rotation_bytes": m["rotation"], "cache_assisted": m["cache_assisted"], "frac_cold": None},
     }
     if cpu_baseline:
         rec["cpu_baseline"] = m["cpu"]()
         rec["cpu_baseline"]["host_cpus"] = os.cpu_count()
     if summary:
         # every other class of the path, same process, same method (HIP events on the launch stream, rotating buffer
-        # sets), fewer launches; the CPU legs here are the short ones (the headline's own leg runs above)
+        # sets), fewer launches; short entries (`--all` prints every workload's full record); the CPU legs here are the
+        # short ones (the headline's own leg runs above)
         import gc
         k_steps, k_warm = max(5, min(steps, 60)), max(2, min(warmup, 10))
         cpu_legs = ("c2p_pack", "c3_pack", "c3_reshard_e2e", "c4", "c5_quantize", "c5_dequant", "stack8", "c1_pack", "c1_reduce")
 
         def entry(w, mm, with_cpu):
-            ach = mm["nbytes"] / (mm["kernel_ms"] * 1e-3) / 1e9
-            e = {"workload": mm["name"], "kernel": mm["kernel"], "ms": mm["kernel_ms"], "achieved": ach,
-                 "frac": ach / HBM_PEAK_GBS, "target": SUMMARY[w], "algorithmic_bytes": mm["nbytes"],
-                 "traffic": traffic.get(w, {}).get("traffic")}
+            frac = mm["nbytes"] / (mm["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+            t = traffic.get(w, {}).get("traffic")
+            e = {"ms": sig(mm["kernel_ms"]), "frac": sig(frac), "target": SUMMARY[w], "bytes": mm["nbytes"],
+                 "traffic_x": sig(t / mm["nbytes"]) if t else None, "rot_mb": int(mm["rotation"] >> 20)}
+            if mm["cache_assisted"]:
+                e["cache_assisted"] = True
             if with_cpu:
-                e["cpu_baseline"] = mm["cpu"]()
+                e["cpu"] = short_cpu(mm["cpu"]())
             return e
 
         out = {}
@@ -1171,10 +1208,14 @@ def run(workload: str, steps: int, warmup: int, cpu_baseline: bool, summary: boo
             mm = measure(torch, lib, w, k_steps, k_warm)
             out[w] = entry(w, mm, cpu_baseline and w in cpu_legs)
             mm = None
-        out = {w: out[w] for w in SUMMARY}
-        rec["workloads"] = out
-        rec["config"]["workloads_note"] = (f"each entry of `workloads`: {k_steps} launches after {k_warm} warm-up launches, HIP events "
-                                           "on the launch stream; target = fraction of HBM peak asked of the class")
+        # rows without a target first, rows that carry one last: a reader that keeps only the end of the line keeps those
+        order = [w for w in SUMMARY if SUMMARY[w] is None] + [w for w in SUMMARY if SUMMARY[w] is not None]
+        rec["workloads"] = {w: out[w] for w in order}
+        if workload == "c2" and "c2_cold" in out:
+            rec["roofline"]["frac_cold"] = out["c2_cold"]["frac"]
+        rec["config"]["workloads_note"] = (f"{k_steps} launches after {k_warm}, HIP events; frac = bytes / ms / 8 TB/s; traffic_x = counter "
+                                           "bytes / bytes; rot_mb = MiB one buffer rotation walks; cache_assisted: rotation < 512 MiB, or "
+                                           "a kernel reads what the one before wrote; cpu: GB/s")
     release_shared()
     return rec
 

@@ -55,17 +55,27 @@ def test_default_bench_line():
     assert cpu["sample"] and cpu["all_cores"]["cores"] >= 1
     # wall-clock throughput cannot exceed the kernel-time throughput by more than timer noise
     assert rec["value"] <= roof["achieved"] * 1.10
-    # every class of the path is reported in the same line, measured in the same process
+    # the headline says how long its buffer rotation is, whether the Infinity Cache helps it, and what the same kernel does cold
+    assert roof["rotation_bytes"] >= 3 * 9 * 25_165_824 * 2 and roof["cache_assisted"] is False
+    assert 0.3 < roof["frac_cold"] <= roof["frac"] * 1.03
+    # every class of the path is reported in the same line, measured in the same process, short enough for a reader
+    # that keeps only the last 8 KB of output, rows that carry a target last
+    assert len(lines[0]) < 7000, len(lines[0])
     sys.path.insert(0, ROOT)
     import bench
     wl = rec["workloads"]
-    assert list(wl) == list(bench.SUMMARY)
+    assert sorted(wl) == sorted(bench.SUMMARY)
+    names = list(wl)
+    first_target = min(i for i, w in enumerate(names) if bench.SUMMARY[w] is not None)
+    assert all(bench.SUMMARY[w] is not None for w in names[first_target:])
     for w, e in wl.items():
         floor = 0.0 if w.startswith("c1_") else 0.2    # configuration 1 moves 1 MiB per call: launch-bound
-        assert e["ms"] > 0 and abs(e["frac"] - e["achieved"] / 8000.0) < 1e-9 and floor < e["frac"] < 1.0, (w, e)
-        assert e["target"] == bench.SUMMARY[w] and e["algorithmic_bytes"] > 0
-        if e["traffic"] is not None:
-            assert 0.9 < e["traffic"] / e["algorithmic_bytes"] < 1.1, (w, e)
-    assert wl["c2"]["frac"] == roof["frac"]
+        assert e["ms"] > 0 and abs(e["frac"] - e["bytes"] / (e["ms"] * 1e-3) / 8e12) < 2e-3 * e["frac"] and floor < e["frac"] < 1.0, (w, e)
+        assert e["target"] == bench.SUMMARY[w] and e["bytes"] > 0 and e["rot_mb"] > 0
+        if e["traffic_x"] is not None:
+            assert 0.9 < e["traffic_x"] < 1.1, (w, e)
+        assert e.get("cache_assisted", False) == (e["rot_mb"] < 512 or w in bench.PIPELINES), (w, e)
+    assert abs(wl["c2"]["frac"] - roof["frac"]) < 1e-3 and wl["c2_cold"]["frac"] == roof["frac_cold"]
+    assert wl["c3_reshard_e2e"]["cache_assisted"] is True and "cache_assisted" not in wl["c2_cold"]
     for w in ("c4", "c5_quantize"):
-        assert wl[w]["cpu_baseline"]["torch_cpu"]["value"] > 0
+        assert wl[w]["cpu"]["torch"] > 0 and wl[w]["cpu"]["port"] > 0
