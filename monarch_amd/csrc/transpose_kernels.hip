@@ -34,6 +34,7 @@ struct TransArgs {
     uint32_t qgroups;   // ceil(qtiles / group)
     uint64_t rows_per_eighth;  // ceil(nbatch * qgroups / 8)
     uint32_t aligned_stores;  // kStore*: how tile rows are written (write-through / streaming need 16-byte aligned rows)
+    uint32_t seg_len, nseg, nstrips;  // strip kernel: positions of a written row per workgroup, segments per row, strips of written rows
     uint32_t group;    // tiles are walked in group x group blocks so that concurrently running workgroups
     uint32_t cgroups;  // touch neighbouring segments on BOTH sides (DRAM row locality); cgroups = ceil(ctiles/group)
     int n_inner;       // dimensions after c (decode q -> memory offset), outermost first
@@ -574,6 +575,152 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
     }
 }
 
+// ---- written rows that do not start on cache lines, narrow elements: a workgroup walks ALONG the written rows ----
+// The windows of the kernel above start up to a line early, so a tile reads D = 128 / sizeof(T) more rows of the other side
+// than it writes positions; for 1-byte elements that is 384 rows of 256 bytes per tile (96 KiB of LDS, half again the
+// reads), and the kernel loses to the fixed tiles.  Here a workgroup owns a strip of TW written rows and a segment
+// [xs, xe) of their positions and moves along it in chunks of CH = D positions: chunk k (CH rows of the read side, 256
+// bytes of each) goes into one half of a two-chunk ring in LDS while the other half still holds chunk k - 1, and
+// written row w takes positions xs + k CH - d_w .. + CH - 1 of it, one whole 128-byte line, d_w < D being what its
+// address needs to start on a line.  The rows a window starts early by are the tail of the chunk before, which the
+// ring still holds: the read side crosses L2 once per segment (plus D rows where a segment starts), every line of
+// the written side is stored whole by one instruction, and the ring is 64 KiB for 1-byte elements.  The next chunk's
+// loads are issued before the current chunk's windows are stored.  u8 8200^2, pack: 0.47 (fixed tiles) -> 0.56 of
+// peak.  2-byte elements gain 0.02 over the kernel above, 4- and 8-byte elements lose 0.03 to 0.05, so only 1-byte
+// elements take it.  (What bounds all of these is the access pattern itself: with rows that are not whole lines,
+// bare 256-byte reads run at 4.9 TB/s and line-by-line writes of rows a pitch apart at 5.4 TB/s, against 6.4 and 5.6
+// for aligned rows.)
+// W is the index of a written row (c when packing, q when unpacking), X the position along it.
+template <typename T, int THREADS, bool PACK>
+__global__ __launch_bounds__(THREADS) void slice_transpose_strip_kernel(TransArgs a) {
+    constexpr int ES = sizeof(T), E = 16 / ES;
+    constexpr int TW = 256 / ES, CH = 128 / ES, RING = 2 * CH;
+    constexpr int LP = CH * 16 / THREADS;  // load passes: CH rows x 16 vectors
+    constexpr int SP = TW * 8 / THREADS;   // store passes: TW rows x 8 vectors (one line of each row)
+    static_assert(LP >= 1 && SP >= 1 && (CH * 16) % THREADS == 0 && (TW * 8) % THREADS == 0, "whole passes");
+    constexpr int LROWS = THREADS / 16, SROWS = THREADS / 8;
+    __shared__ __attribute__((aligned(16))) T tile[RING * TW];  // [read row, modulo the ring][written row]
+    union Vec {
+        u32x4 v;
+        T e[E];
+    };
+
+    // workgroup i runs on XCD i % 8: each XCD takes a contiguous eighth of the (batch, segment, strip) list, strips
+    // fastest, so that the strips that read neighbouring pieces of the same rows run side by side in one L2
+    const uint64_t wg = a.wg0 + blockIdx.x;
+    const uint64_t id = (wg % 8) * ((a.ntiles + 7) / 8) + wg / 8;
+    if (id >= a.ntiles) return;
+    const uint64_t per_batch = (uint64_t)a.nseg * a.nstrips;
+    const uint64_t b = id / per_batch;
+    const uint32_t in_batch = (uint32_t)(id - b * per_batch);
+    const uint32_t seg = in_batch / a.nstrips, sw = in_batch - seg * a.nstrips;
+    const uint32_t Wn = PACK ? a.Sc : a.Q, Xn = PACK ? a.Q : a.Sc;
+    uint32_t w0 = sw * TW;
+    if (w0 + TW > Wn) w0 = Wn - TW;  // the host sends extents of at least a strip; the overlap is written twice, same bytes
+    const uint32_t xs = seg * a.seg_len;
+    const uint32_t xe = xs + a.seg_len < Xn ? xs + a.seg_len : Xn;
+    const int K = (int)((xe - xs + CH - 1) / CH);
+    // the last segment of a row also stores what lies behind its last whole window: the row's last d_w positions
+    const int iters = K + (seg + 1 == a.nseg ? 1 : 0);
+
+    T* __restrict__ mem = reinterpret_cast<T*>(a.base) + a.offset;
+    T* __restrict__ packed = reinterpret_cast<T*>(a.packed);
+    uint64_t batch_off = 0;
+    {
+        uint64_t rem = b;
+        for (int k = a.n_outer - 1; k >= 0; --k) {
+            const uint64_t qd = rem / a.outer_size[k];
+            batch_off += (rem - qd * a.outer_size[k]) * a.outer_stride[k];
+            rem = qd;
+        }
+    }
+    auto q_offset = [&](uint32_t q) {  // memory offset of row q of the batch
+        uint64_t off = 0;
+        for (int k = a.n_inner - 1; k > 0; --k) {
+            uint32_t qd, r;
+            a.inner_div[k].divmod(q, qd, r);
+            off += (uint64_t)r * a.inner_stride[k];
+            q = qd;
+        }
+        return off + (uint64_t)q * a.inner_stride[0];
+    };
+
+    const int v16 = threadIdx.x % 16, r16 = threadIdx.x / 16;
+    const int v8 = threadIdx.x % 8, r8 = threadIdx.x / 8;
+    // chunk c = read rows xs + c CH .. + CH - 1, clamped into the extent (what a clamped row holds is never stored)
+    auto load_chunk = [&](int c, Vec* d) {
+#pragma unroll
+        for (int p = 0; p < LP; ++p) {
+            int64_t x = (int64_t)xs + (int64_t)c * CH + r16 + LROWS * p;
+            x = x < 0 ? 0 : (x > (int64_t)Xn - 1 ? (int64_t)Xn - 1 : x);
+            const T* src;
+            if constexpr (PACK) src = mem + batch_off + q_offset((uint32_t)x) + w0 + v16 * E;
+            else src = packed + (b * a.Sc + (uint64_t)x) * (uint64_t)a.Q + w0 + v16 * E;
+            d[p].v = tload<false>(src);
+        }
+    };
+    auto put_chunk = [&](int c, const Vec* d) {
+#pragma unroll
+        for (int p = 0; p < LP; ++p) {
+            const int rr = ((c + 1) * CH + r16 + LROWS * p) & (RING - 1);
+            *reinterpret_cast<u32x4*>(&tile[rr * TW + E * (v16 ^ ((rr / E) % 16))]) = d[p].v;
+        }
+    };
+
+    // The written rows of this lane.  The eight rows of a wavefront take elements that sit in eight different 32-bit words:
+    // each row reads its own LDS rows (its window starts at its own place), so rows whose elements share a word would meet
+    // in one bank at different addresses.
+    constexpr int S = ES >= 4 ? 1 : 4 / ES;
+    int wr[SP], dws[SP];
+    T* rowp[SP];
+#pragma unroll
+    for (int p = 0; p < SP; ++p) {
+        const int logical = r8 + SROWS * p;
+        const int in_block = logical % (8 * S);
+        wr[p] = logical - in_block + (in_block % 8) * S + in_block / 8;
+        if constexpr (PACK) rowp[p] = packed + (b * a.Sc + w0 + wr[p]) * (uint64_t)a.Q;
+        else rowp[p] = mem + batch_off + q_offset(w0 + wr[p]);
+        dws[p] = (int)(((uintptr_t)rowp[p] & 127u) / ES);  // xs is a multiple of CH, i.e. of a line
+    }
+
+    Vec d[LP];
+    if (xs > 0) {
+        load_chunk(-1, d);
+        put_chunk(-1, d);
+    }
+    load_chunk(0, d);
+    put_chunk(0, d);
+    __syncthreads();
+    for (int k = 0; k < iters; ++k) {
+        const bool more = k + 1 < K;
+        if (more) load_chunk(k + 1, d);
+#pragma unroll
+        for (int p = 0; p < SP; ++p) {
+            const int t0 = (k + 1) * CH - dws[p] + v8 * E;  // the vector's first element, counted from the first row of chunk -1
+            const int64_t xw = (int64_t)xs + (int64_t)k * CH - dws[p] + v8 * E;
+            // its E rows lie in at most two groups of E ring rows, i.e. see two XOR permutations
+            const int r0 = t0 & (RING - 1);
+            const int g0 = r0 / E, g1 = (g0 + 1) % (RING / E);
+            const int first = E - r0 % E;
+            const T* __restrict__ p0 = tile + r0 * TW + (wr[p] ^ (E * (g0 % 16)));
+            const T* __restrict__ p1 = tile + (g1 * E - first) * TW + (wr[p] ^ (E * (g1 % 16)));
+            Vec o;
+#pragma unroll
+            for (int j = 0; j < E; ++j) o.e[j] = (j < first ? p0 : p1)[j * TW];
+            if (xw >= 0 && xw + E <= (int64_t)Xn) {
+                tstore(rowp[p] + xw, o.v, kStoreStreaming);
+            } else {
+#pragma unroll
+                for (int j = 0; j < E; ++j)
+                    if (xw + j >= 0 && xw + j < (int64_t)Xn) rowp[p][xw + j] = o.e[j];
+            }
+        }
+        __syncthreads();  // every window of this step has been read: the older half of the ring is free
+        if (more) put_chunk(k + 1, d);
+        __syncthreads();
+    }
+}
+
 // Cache policy of a launch, from an A/B over sixteen shapes, both directions and four element sizes (fractions of the
 // HBM peak; "cached" = plain loads, write-through stores on aligned rows; the table is
 // profiles/transpose_cache_policy_ab.md):
@@ -704,17 +851,51 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         }
     }
     const uint32_t tile = vec ? (big ? 512 : 256) / unit : 32;
-    // Written rows that do not start on cache lines take the kernel whose windows do (slice_transpose_lines_kernel):
-    // the extent along the written rows grows by the most a window can start early.
-    // With the tuning aids on, MONARCH_HIP_TRANSPOSE_LINES=0 / 1 overrides the choice at every call.
-    bool lines = false;
-    if (vec && !big && unit >= 2 && (PACK ? Sc : Q) >= tile) {  // 1-byte elements lose with it (8200^2 0.475 -> 0.36: 96 KiB of LDS, byte-wise LDS reads)
+    // Written rows that do not start on cache lines take a kernel whose windows do: 2-, 4- and 8-byte elements the one
+    // with a window per row of a tile (slice_transpose_lines_kernel; the extent along the written rows grows by the
+    // most a window can start early), 1-byte elements the one that walks along the written rows
+    // (slice_transpose_strip_kernel; with per-tile windows they lose, 8200^2 0.475 -> 0.36: 96 KiB of LDS, byte-wise LDS reads).
+    // With the tuning aids on, MONARCH_HIP_TRANSPOSE_LINES overrides the choice at every call: 0 fixed tiles, 1 windows per
+    // tile, 2 strips (1- and 2-byte elements).
+    bool lines = false, strips = false;
+    if (vec && !big && (PACK ? Sc : Q) >= tile) {
         uint64_t written = PACK ? ((uint64_t)(uintptr_t)packed | Q * unit) : ((uint64_t)(uintptr_t)base + c.offset * unit);
         if (!PACK)
             for (int k = 0; k < c.ndim; ++k)
                 if (k != cd) written |= c.dims[k].stride * unit;
-        lines = (written & 127u) != 0;
-        if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_LINES")) lines = std::atoi(e) != 0;
+        const bool inside_lines = (written & 127u) != 0;
+        lines = inside_lines && unit >= 2;
+        // strips need enough of them to fill the part: 512 workgroups of segments of 4 chunks (u8 7000 x 5000, 280
+        // workgroups: 0.43 of peak against 0.57 with the fixed tiles)
+        const uint64_t Wn = PACK ? Sc : Q, Xn = PACK ? Q : Sc;
+        strips = inside_lines && unit == 1 && nbatch * ((Wn + 255) / 256) * ((Xn + 511) / 512) >= 512;
+        if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_LINES")) {
+            const int v = std::atoi(e);
+            lines = v == 1;
+            strips = v == 2 && unit <= 2;
+        }
+    }
+    if (strips) {
+        // Segments of 4 chunks (512 bytes of every written row): 1-byte elements 8200^2 0.56 of peak with 4, 0.53 with 8,
+        // 0.34 with 16 (too few workgroups); short rows get one segment.
+        const uint32_t chunk = 128 / unit, rows_per_strip = 256 / unit;
+        const uint64_t Wn = PACK ? Sc : Q, Xn = PACK ? Q : Sc;
+        a.base = base;
+        a.packed = packed;
+        a.offset = c.offset;
+        a.Sc = (uint32_t)Sc;
+        a.Q = (uint32_t)Q;
+        a.seg_len = 4 * chunk;
+        a.nseg = (uint32_t)((Xn + a.seg_len - 1) / a.seg_len);
+        a.nstrips = (uint32_t)((Wn + rows_per_strip - 1) / rows_per_strip);
+        a.ntiles = nbatch * a.nseg * a.nstrips;
+        const uint64_t nblocks = 8 * ((a.ntiles + 7) / 8);
+        *rc = launch_in_pieces(nblocks, 512, 8, [&](uint64_t wg0, uint32_t count) {
+            a.wg0 = wg0;
+            if (unit == 1) MHIP_LAUNCH((slice_transpose_strip_kernel<uint8_t, 512, PACK>), dim3(count), dim3(512), 0, stream, a);
+            else MHIP_LAUNCH((slice_transpose_strip_kernel<uint16_t, 512, PACK>), dim3(count), dim3(512), 0, stream, a);
+        });
+        return true;
     }
     const uint32_t early = lines ? 128 / unit - 1 : 0;
     a.base = base;

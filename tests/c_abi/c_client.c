@@ -272,6 +272,59 @@ int main(void) {
         free(stacked);
     }
 
+    /* 6. device-initiated RDMA: a send WQE, the doorbell ring and one completion-queue poll on ordinary device
+     * memory, against bytes written out by hand (mlx5 layouts: control, remote-address and data segment) */
+    {
+        enum { CNT = 4 };
+        void *dsq, *ddb, *dreg, *dcq, *dres;
+        CHECK(mhip_malloc(&dsq, CNT * 64)); CHECK(mhip_malloc(&ddb, 8)); CHECK(mhip_malloc(&dreg, 64));
+        CHECK(mhip_malloc(&dcq, CNT * 64)); CHECK(mhip_malloc(&dres, 4));
+        CHECK(mhip_memset(dsq, 0xEE, CNT * 64, stream)); CHECK(mhip_memset(ddb, 0, 8, stream));
+        CHECK(mhip_memset(dcq, 0, CNT * 64, stream)); CHECK(mhip_memset(dres, 0xFF, 4, stream));   /* -1 */
+        mhip_wqe_params_t w;
+        memset(&w, 0, sizeof w);
+        w.laddr = 0x00007F1234567890ull; w.lkey = 0xAABBCCDDu; w.length = 0x00100000; w.wr_id = 5; w.signaled = 1;
+        w.op_type = MHIP_MLX5_OPCODE_RDMA_WRITE; w.raddr = 0x00007E00DEADBEE0ull; w.rkey = 0x11223344u; w.qp_num = 0x001234;
+        w.buf = dsq; w.dbrec = ddb; w.wqe_cnt = CNT;
+        CHECK(mhip_rdmaxcel_send_wqe(&w, stream));
+        CHECK(mhip_rdmaxcel_ring_doorbells(dreg, dsq, 64, CNT, 5, 1, stream));
+        /* the NIC's completion for consumer index 5: entry 1, second lap (owner bit 1), opcode 0, 1 MiB */
+        unsigned char cqe[64];
+        memset(cqe, 0, sizeof cqe);
+        cqe[44] = 0x00; cqe[45] = 0x10; cqe[46] = 0x00; cqe[47] = 0x00; cqe[63] = 0x01;
+        CHECK(mhip_memcpy_htod((char*)dcq + 64, cqe, 64, stream));
+        mhip_cqe_poll_params_t c;
+        c.cqe_buf = dcq; c.cqe_size = 64; c.consumer_index = 5; c.cqe_cnt = CNT; c.dbrec = (uint32_t*)ddb;
+        CHECK(mhip_rdmaxcel_cqe_poll(dres, &c, stream));
+        unsigned char sq[CNT * 64], reg[64], db[8];
+        int32_t res = 0;
+        CHECK(mhip_memcpy_dtoh(sq, dsq, sizeof sq, stream)); CHECK(mhip_memcpy_dtoh(reg, dreg, 64, stream));
+        CHECK(mhip_memcpy_dtoh(db, ddb, 8, stream)); CHECK(mhip_memcpy_dtoh(&res, dres, 4, stream));
+        CHECK(mhip_stream_synchronize(stream));
+        static const unsigned char want[48] = {
+            0x00, 0x00, 0x05, 0x08, 0x00, 0x12, 0x34, 0x03, 0x00, 0x00, 0x00, 0x0A, 0x00, 0x00, 0x00, 0x00,
+            0x00, 0x00, 0x7E, 0x00, 0xDE, 0xAD, 0xBE, 0xE0, 0x11, 0x22, 0x33, 0x44, 0x00, 0x00, 0x00, 0x00,
+            0x00, 0x10, 0x00, 0x00, 0xAA, 0xBB, 0xCC, 0xDD, 0x00, 0x00, 0x7F, 0x12, 0x34, 0x56, 0x78, 0x90};
+        static const unsigned char want_db[8] = {0, 0, 0, 6, 0, 0, 0, 6};   /* CQ consumer 6 | send counter 6 */
+        int ok = memcmp(sq + 64, want, 48) == 0 && memcmp(reg, sq + 64, 64) == 0 && memcmp(db, want_db, 8) == 0 && res == 0x00100000;
+        for (int i = 0; i < CNT * 64; ++i)
+            if ((i < 64 || i >= 112) && sq[i] != 0xEE) ok = 0;
+        if (!ok) {
+            fprintf(stderr, "rdmaxcel: WQE / doorbell / poll bytes differ (poll result %d)\n", (int)res);
+            return 1;
+        }
+        /* the same WQE through the host function, into host memory */
+        _Alignas(64) unsigned char hsq[CNT * 64];
+        uint32_t hdb[2] = {0, 0};
+        w.buf = hsq; w.dbrec = hdb;
+        CHECK(mhip_rdmaxcel_send_wqe_host(&w));
+        if (memcmp(hsq + 64, want, 48) != 0 || memcmp(&hdb[1], want_db + 4, 4) != 0) {
+            fprintf(stderr, "rdmaxcel: host WQE bytes differ\n");
+            return 1;
+        }
+        CHECK(mhip_free(dsq)); CHECK(mhip_free(ddb)); CHECK(mhip_free(dreg)); CHECK(mhip_free(dcq)); CHECK(mhip_free(dres));
+    }
+
     for (int g = 0; g < G; ++g) CHECK(mhip_free(d[g]));
     CHECK(mhip_free(dx)); CHECK(mhip_free(dp)); CHECK(mhip_free(db)); CHECK(mhip_free(dout));
     CHECK(mhip_free(dt)); CHECK(mhip_free(dq)); CHECK(mhip_free(dsc)); CHECK(mhip_free(dacc));

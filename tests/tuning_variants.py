@@ -20,7 +20,7 @@ def test_the_switch_is_on():
     assert os.environ.get("MONARCH_HIP_TUNING") == "1", "run through tests/test_gpu_tuning_variants.py"
 
 
-@pytest.mark.parametrize("lines", ["0", "1"])
+@pytest.mark.parametrize("lines", ["0", "1", "2"])
 @pytest.mark.parametrize("dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
 def test_transposes_with_line_aligned_windows_and_without(dtype, lines, monkeypatch):
     # written rows that start anywhere in a cache line, through the kernel whose windows start on lines and through
