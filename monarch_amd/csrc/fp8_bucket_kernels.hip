@@ -254,7 +254,14 @@ __device__ __forceinline__ uint32_t quantize_loaded_span(uint8_t* __restrict__ q
 __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(4))) void fp8_quantize_bucket_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                        BucketArgs a) {
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (threadIdx.x >> 6);
+    // The wavefront's number goes through a scalar register: what is derived from it (span, block index entry, offsets and
+    // pointers of the span's tensors) is then wave-uniform for the compiler too.  In the quantiser, whose only stores go to
+    // its restrict-qualified outputs, the table reads on the way to the first data load become scalar loads (fused
+    // quantiser on the 756 M-element bucket 0.73 -> 0.79 of peak; 0.87 -> 0.94 of the flat quantiser on the same GPU).
+    // The dequantisers store through pointers they loaded from a table, so the compiler keeps vector loads for their table
+    // reads; forcing scalar loads there (reads through the constant address space) was measured and loses: single-peer
+    // 0.746 -> 0.703, eight peers 0.716 -> 0.703, although buckets of a few MB gain 0.8 us.
+    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint64_t nwaves = (uint64_t)gridDim.x * (kBucketThreads / 64);
     for (uint64_t b0 = wave * kBucketBlocks; b0 < a.nblocks; b0 += nwaves * kBucketBlocks) {
         const uint64_t span_begin = b0 * kBlock;
@@ -469,7 +476,7 @@ __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(
                                                                                  const float* __restrict__ scales,
                                                                                  BucketArgs a) {
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // see fp8_quantize_bucket_kernel
     const uint64_t nwaves = (uint64_t)gridDim.x * (kBucketThreads / 64);
     for (uint64_t b = wave; b < a.nblocks; b += nwaves) {
         const uint64_t begin = b * kBlock;
@@ -552,7 +559,7 @@ __device__ __forceinline__ void dequant_accumulate_block_peers(const BucketPeers
 __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(7))) void fp8_dequant_accumulate_bucket_many_kernel(BucketPeersArgs p) {
     const BucketArgs& a = p.b;
     const int lane = threadIdx.x & 63;
-    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (threadIdx.x >> 6);
+    const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // see fp8_quantize_bucket_kernel
     const uint64_t nwaves = (uint64_t)gridDim.x * (kBucketThreads / 64);
     for (uint64_t b = wave; b < a.nblocks; b += nwaves) {
         const uint64_t begin = b * kBlock;

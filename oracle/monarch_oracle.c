@@ -30,6 +30,10 @@
  *   fp8 e4m3fn block-scaled codec                  no counterpart in the reference (fp8 reductions are
  *     refused, torch-sys-cuda/src/nccl.rs:474-476): PARITY UNPINNED in the reference; the encode/decode
  *     tables are pinned against the OCP format via torch's CPU cast over all 65536 bf16 patterns.
+ *   work-queue / completion-queue entries (send_wqe, recv_wqe, cqe_poll, db_ring; rdmaxcel-sys/src/rdmaxcel.cu)
+ *                                                  the reference holds no byte vector (its tests need two NICs):
+ *     PARITY UNPINNED in the reference; pinned by bytes written out by hand from rdma-core's published mlx5 segment
+ *     layouts (tests/test_oracle_rdmaxcel.py), sixteen source mutations of these functions each fail one of them.
  */
 #ifdef _OPENMP
 #include <omp.h>
