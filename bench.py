@@ -524,11 +524,16 @@ def wl_stack(torch, scatter=False, sets=None):
 def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3, n=None):
     from monarch_amd import Slice, staging
     n = n or int(os.environ.get("MONARCH_BENCH_TRANSPOSE_N", "8192"))
-    dt = {"f32": torch.float32, "bf16": torch.bfloat16}[dtype_name]
+    dt = {"f32": torch.float32, "bf16": torch.bfloat16, "u8": torch.uint8}[dtype_name]
     g = torch.Generator(device="cuda:0").manual_seed(6000)
     s = Slice(offset=0, sizes=[n, n], strides=[1, n])  # iterate columns first: packs x.T
-    bufs = [(torch.randn(n, n, generator=g, device="cuda:0").to(dt), torch.empty(n * n, dtype=dt, device="cuda:0"))
-            for _ in range(sets)]
+
+    def values():
+        if dt == torch.uint8:
+            return torch.randint(0, 256, (n, n), generator=g, device="cuda:0", dtype=torch.uint8)
+        return torch.randn(n, n, generator=g, device="cuda:0").to(dt)
+
+    bufs = [(values(), torch.empty(n * n, dtype=dt, device="cuda:0")) for _ in range(sets)]
     es = bufs[0][0].element_size()
     nbytes = 2 * n * n * es
     for x, st in bufs:
@@ -544,7 +549,7 @@ def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3, n=None):
     def cpu():
         import oracle
         m = 2048
-        h = bufs[0][0][:m, :m].contiguous().cpu().view(torch.uint16 if es == 2 else torch.int32).numpy().reshape(-1)
+        h = bufs[0][0][:m, :m].contiguous().cpu().view({1: torch.uint8, 2: torch.uint16, 4: torch.int32}[es]).numpy().reshape(-1)
         t0 = time.perf_counter()
         oracle.pack(h, oracle.OSlice(0, [m, m], [1, m]))
         dt_ = (time.perf_counter() - t0) * (n * n / (m * m))
@@ -552,7 +557,8 @@ def wl_transpose(torch, dtype_name="f32", unpack=False, sets=3, n=None):
                 "sample": f"{m}x{m} corner through the per-element Slice::get walk, scaled to {n}x{n}"}
 
     name = f"transpose_{dtype_name}_{n}x{n}_" + ("unpack" if unpack else "pack")
-    kernel = "slice_transpose_vec_kernel" if n * es % 128 == 0 else "slice_transpose_lines_kernel"
+    kernel = ("slice_transpose_vec_kernel" if n * es % 128 == 0 else
+              "slice_transpose_strip_kernel" if es == 1 else "slice_transpose_lines_kernel")
     return name, nbytes, launch, cpu, kernel, "u8"
 
 
@@ -800,6 +806,8 @@ WORKLOADS = {
     # rows of 16400 bytes: no written row starts on a cache line
     "tr_bf16_8200_pack": lambda t: wl_transpose(t, "bf16", False, n=8200),
     "tr_bf16_8200_unpack": lambda t: wl_transpose(t, "bf16", True, n=8200),
+    "tr_u8_8200_pack": lambda t: wl_transpose(t, "u8", False, n=8200, sets=6),
+    "tr_u8_8200_unpack": lambda t: wl_transpose(t, "u8", True, n=8200, sets=6),
     "c5_flat_pack": lambda t: wl_c5(t, "flat_pack"),
     "c5_quantize": lambda t: wl_c5(t, "quantize"),
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
@@ -1096,7 +1104,7 @@ SUMMARY = {
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
     "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
-    "tr_bf16_8200_pack": None, "tr_bf16_8200_unpack": None,
+    "tr_bf16_8200_pack": None, "tr_bf16_8200_unpack": None, "tr_u8_8200_pack": None, "tr_u8_8200_unpack": None,
     # configuration 1 (1 MiB views): launch-bound, reported as time per call
     "c1_pack": None, "c1_unpack": None, "c1_reduce": None, "c1_pipeline": None, "c1_pipeline_fused": None,
 }
@@ -1117,11 +1125,13 @@ PIPELINES = ("c3_reshard_e2e", "c3_reshard_e2e_one_by_one", "c1_pipeline", "c1_p
 
 def measure(torch, lib, workload: str, steps: int, warmup: int):
     torch.cuda.synchronize()
-    held_before = torch.cuda.memory_allocated()
+    held_before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     name, nbytes, launch, cpu, kernel, dtype = WORKLOADS[workload](torch)
-    # device memory of the workload's rotating buffer sets: what one rotation walks through.  (The C5 stages share one
+    torch.cuda.synchronize()
+    # device memory of the workload's rotating buffer sets: what one rotation walks through.  Staging areas are mapped
+    # by the library, not by torch, hence the device's own free-memory figure beside torch's.  (The C5 stages share one
     # set of buffers made by the first of them; each of their launches alone moves 3 GB and more.)
-    rotation = max(torch.cuda.memory_allocated() - held_before, nbytes)
+    rotation = max(torch.cuda.memory_allocated() - held_before, free_before - torch.cuda.mem_get_info()[0], nbytes)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     rc = 0
     for i in range(warmup):
