@@ -585,8 +585,11 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
 // address needs to start on a line.  The rows a window starts early by are the tail of the chunk before, which the
 // ring still holds: the read side crosses L2 once per segment (plus D rows where a segment starts), every line of
 // the written side is stored whole by one instruction, and the ring is 64 KiB for 1-byte elements.  The next chunk's
-// loads are issued before the current chunk's windows are stored.  u8 8200^2, pack: 0.47 (fixed tiles) -> 0.56 of
-// peak.  2-byte elements gain 0.02 over the kernel above, 4- and 8-byte elements lose 0.03 to 0.05, so only 1-byte
+// loads are issued before the current chunk's windows are stored.  u8 8200^2, pack / unpack, both kernels in turn on one
+// GPU: 0.465 / 0.47 (fixed tiles) -> 0.555 / 0.545 of peak while source and destination rotate over 400 MB of buffers,
+// i.e. partly out of the 256 MB Infinity Cache, as they do when the neighbouring stage of a pipeline has just written or
+// is about to read them; rotating over 800 MB both kernels read 0.45.  Never slower than the fixed tiles on nine
+// shapes.  2-byte elements gain 0.02 over the kernel above, 4- and 8-byte elements lose 0.03 to 0.05, so only 1-byte
 // elements take it.  (What bounds all of these is the access pattern itself: with rows that are not whole lines,
 // bare 256-byte reads run at 4.9 TB/s and line-by-line writes of rows a pitch apart at 5.4 TB/s, against 6.4 and 5.6
 // for aligned rows.)
@@ -876,8 +879,8 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         }
     }
     if (strips) {
-        // Segments of 4 chunks (512 bytes of every written row): 1-byte elements 8200^2 0.56 of peak with 4, 0.53 with 8,
-        // 0.34 with 16 (too few workgroups); short rows get one segment.
+        // Segments of 4 chunks (512 bytes of every written row): 1-byte elements 8200^2 over 400 MB of buffers 0.56 of peak
+        // with 4, 0.53 with 8, 0.34 with 16 (too few workgroups); short rows get one segment.
         const uint32_t chunk = 128 / unit, rows_per_strip = 256 / unit;
         const uint64_t Wn = PACK ? Sc : Q, Xn = PACK ? Q : Sc;
         a.base = base;
