@@ -284,3 +284,42 @@ def test_host_mode_queue_pair_on_host_memory_gives_the_same_bytes():
     assert int(host(result)[0]) == 256 and cqdb_h.numpy().view(np.uint8)[:4].tobytes() == bytes.fromhex("00000001")
     host_qp.launch_cqe_poll(PollTarget.Send)
     assert res[0] == 256
+
+
+def test_posting_ringing_and_polling_record_into_a_graph():
+    # the entry points only enqueue kernels (no synchronisation, no allocation: the reference's launchers synchronise
+    # the device per entry and allocate managed memory per poll), so a caller can record a post -> ring -> poll sequence
+    # once and replay it; every replay, with a new completion written in between, must give the eager result
+    L = lib()
+    cnt = 4
+    sq, dbrec, reg = dev_bytes(cnt * 64, 0), torch.zeros(2, dtype=torch.int32, device="cuda"), dev_bytes(64, 0)
+    cq = torch.zeros(64 * cnt, dtype=torch.uint8, device="cuda")
+    cq[63::64] = 0xF0
+    cqdb = torch.zeros(2, dtype=torch.int32, device="cuda")
+    result = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+    f = dict(laddr=0x7000_0000_1000, lkey=3, length=1 << 16, wr_id=2, signaled=True, op_type=MLX5_OPCODE_RDMA_WRITE_IMM,
+             raddr=0x7100_0000_2000, rkey=4, qp_num=0x99)
+    p = wqe(sq, dbrec, cnt, **f)
+    c = CqePollParamsC(cq.data_ptr(), 64, 2, cnt, cqdb.data_ptr())
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        s = stream()
+        check(L.mhip_memset(result.data_ptr(), 0xFF, 4, s))
+        check(L.mhip_rdmaxcel_send_wqe(C.byref(p), s))
+        check(L.mhip_rdmaxcel_ring_doorbells(reg.data_ptr(), sq.data_ptr(), 64, cnt, 2, 1, s))
+        check(L.mhip_rdmaxcel_cqe_poll(result.data_ptr(), C.byref(c), s))
+    want_sq, want_db = np.zeros(cnt * 64, dtype=np.uint8), np.zeros(2, dtype=np.uint32)
+    oracle.send_wqe(want_sq, want_db, cnt, **f)
+    for rep, (op_own, count, want) in enumerate([(0xF0, 0, -1), (0x00, 4096, 4096), (0xD0, 0, -2), (0x01, 7, -1)]):
+        sq.zero_(); dbrec.zero_(); reg.zero_(); cqdb.zero_()
+        cq[2 * 64 + 44:2 * 64 + 48] = torch.tensor(list(int(count).to_bytes(4, "big")), dtype=torch.uint8, device="cuda")
+        cq[2 * 64 + 63] = op_own
+        other = torch.randn(1 << 16, device="cuda").sum()   # unrelated eager work between replays
+        graph.replay()
+        assert int(host(result)[0]) == want, rep
+        assert host(sq).tobytes() == want_sq.tobytes() and host(dbrec).view(np.uint32).tobytes() == want_db.tobytes(), rep
+        assert host(reg).tobytes() == want_sq[128:192].tobytes(), rep
+        assert int(host(cqdb)[0]) == (int.from_bytes((3).to_bytes(4, "big"), "little") if want != -1 else 0), rep
+        assert torch.isfinite(other)

@@ -340,13 +340,28 @@ int main() {
   mhip_rdmaxcel::send_wqe(p);
   for (int i = 64; i < 112; ++i) std::printf("%02x", sq[i]);
   std::printf(" %08x\n", dbrec[1]);
+  // the other three functions once each, on the same memory
+  mhip_rdmaxcel::recv_wqe(p);
+  alignas(8) unsigned char reg[64];
+  mhip_rdmaxcel::db_ring(reg, sq + 64);
+  alignas(4) unsigned char cq[128]; std::memset(cq, 0, sizeof cq); cq[44] = 0x12; cq[63] = 0x00;
+  uint32_t cqdb[1] = {0};
+  mhip_cqe_poll_params_t q{cq, 64, 0, 2, cqdb};
+  int32_t res = -1;
+  mhip_rdmaxcel::cqe_poll(&res, q);
+  std::printf("%02x%02x %08x %08x\n", sq[3], reg[3], (unsigned)res, cqdb[0]);
 }
 '''
     exe = tmp_path / "t"
-    r = subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-Werror", "-I", os.path.join(root, "include"), "-x", "c++", "-", "-o", str(exe)],
-                       input=src, text=True, capture_output=True)
+    # under the host sanitizers: the 16-byte segment stores, the doorbell record and the byte swaps have no undefined behaviour
+    r = subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-Wall", "-Werror", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                        "-I", os.path.join(root, "include"), "-x", "c++", "-", "-o", str(exe)], input=src, text=True, capture_output=True)
     assert r.returncode == 0, r.stderr
-    out = subprocess.run([str(exe)], capture_output=True, text=True).stdout.split()
+    run = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert run.returncode == 0, run.stderr[-2000:]
+    out = run.stdout.split()
     assert out[0] == ("00000108" "00000903" "0000000a" "00000000" "0000000000002000" "00000003" "00000000"
                       "00000040" "00000002" "0000000000001000")
     assert out[1] == "02000000"   # big-endian 2 read back as a little-endian word
+    # recv_wqe put byte_count 0x40 big-endian at the queue's start; the ring copied the posted slot; the poll read 0x12000000
+    assert out[2:] == ["4008", "12000000", "01000000"]
