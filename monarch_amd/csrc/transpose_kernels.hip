@@ -586,13 +586,12 @@ __global__ __launch_bounds__(THREADS) void slice_transpose_lines_kernel(TransArg
 // ring still holds: the read side crosses L2 once per segment (plus D rows where a segment starts), every line of
 // the written side is stored whole by one instruction, and the ring is 64 KiB for 1-byte elements.  The next chunk's
 // loads are issued before the current chunk's windows are stored.  u8 8200^2, pack / unpack, both kernels in turn on one
-// GPU: 0.465 / 0.47 (fixed tiles) -> 0.555 / 0.545 of peak while source and destination rotate over 400 MB of buffers,
-// i.e. partly out of the 256 MB Infinity Cache, as they do when the neighbouring stage of a pipeline has just written or
-// is about to read them; rotating over 800 MB both kernels read 0.45.  Never slower than the fixed tiles on nine
-// shapes.  2-byte elements gain 0.02 over the kernel above, 4- and 8-byte elements lose 0.03 to 0.05, so only 1-byte
-// elements take it.  (What bounds all of these is the access pattern itself: with rows that are not whole lines,
-// bare 256-byte reads run at 4.9 TB/s and line-by-line writes of rows a pitch apart at 5.4 TB/s, against 6.4 and 5.6
-// for aligned rows.)
+// GPU: 0.44 / 0.46 of peak (fixed tiles) -> 0.50 / 0.50 rotating over 800 MB of buffers, 0.464 / 0.472 -> 0.589 / 0.566
+// rotating over 400 MB (partly out of the 256 MB Infinity Cache, as when the neighbouring stage of a pipeline has just
+// written or is about to read them).  2-byte elements gain 0.02 over the kernel above, 4- and 8-byte elements lose 0.03 to
+// 0.05, so only 1-byte elements take it.  (What bounds all of these is the access pattern itself: with rows that are not
+// whole lines, bare 256-byte reads run at 4.9 TB/s and line-by-line writes of rows a pitch apart at 5.4 TB/s, against
+// 6.4 and 5.6 for aligned rows.)
 // W is the index of a written row (c when packing, q when unpacking), X the position along it.
 template <typename T, int THREADS, bool PACK>
 __global__ __launch_bounds__(THREADS) void slice_transpose_strip_kernel(TransArgs a) {
@@ -861,6 +860,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
     // With the tuning aids on, MONARCH_HIP_TRANSPOSE_LINES overrides the choice at every call: 0 fixed tiles, 1 windows per
     // tile, 2 strips (1- and 2-byte elements).
     bool lines = false, strips = false;
+    uint32_t seg_chunks = 2;
     if (vec && !big && (PACK ? Sc : Q) >= tile) {
         uint64_t written = PACK ? ((uint64_t)(uintptr_t)packed | Q * unit) : ((uint64_t)(uintptr_t)base + c.offset * unit);
         if (!PACK)
@@ -868,19 +868,25 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
                 if (k != cd) written |= c.dims[k].stride * unit;
         const bool inside_lines = (written & 127u) != 0;
         lines = inside_lines && unit >= 2;
-        // strips need enough of them to fill the part: 512 workgroups of segments of 4 chunks (u8 7000 x 5000, 280
-        // workgroups: 0.43 of peak against 0.57 with the fixed tiles)
+        // strips need enough of them to fill the part: 1024 workgroups of segments of 2 chunks (u8 7000 x 5000, 560
+        // workgroups: 0.44 / 0.40 of peak against 0.57 / 0.58 with the fixed tiles; 8200^2, 1089 workgroups, wins)
         const uint64_t Wn = PACK ? Sc : Q, Xn = PACK ? Q : Sc;
-        strips = inside_lines && unit == 1 && nbatch * ((Wn + 255) / 256) * ((Xn + 511) / 512) >= 512;
+        strips = inside_lines && unit == 1 && nbatch * ((Wn + 255) / 256) * ((Xn + 255) / 256) >= 1024;
         if (const char* e = tuning_env("MONARCH_HIP_TRANSPOSE_LINES")) {
-            const int v = std::atoi(e);
-            lines = v == 1;
-            strips = v == 2 && unit <= 2;
+            int v = 0, chunks = 0;
+            const int n = std::sscanf(e, "%d,%d", &v, &chunks);
+            lines = n >= 1 && v == 1;
+            strips = n >= 1 && v == 2 && unit <= 2;
+            if (n >= 2 && chunks >= 1 && chunks <= 64) seg_chunks = (uint32_t)chunks;  // "2,<chunks per segment>"
         }
     }
     if (strips) {
-        // Segments of 4 chunks (512 bytes of every written row): 1-byte elements 8200^2 over 400 MB of buffers 0.56 of peak
-        // with 4, 0.53 with 8, 0.34 with 16 (too few workgroups); short rows get one segment.
+        // Segments of 2 chunks (256 bytes of every written row).  1-byte elements 8200^2, pack, chunks per segment 1 / 2 / 3 / 4 /
+        // 8 / 16: rotating over 800 MB of buffers 0.456 / 0.504 / 0.484 / 0.456 / 0.414 / 0.380 of peak (fixed tiles 0.44), over
+        // 400 MB (partly out of the Infinity Cache) 0.545 / 0.589 / 0.609 / 0.552 (fixed tiles 0.464).  A segment re-reads the
+        // D rows before its start, but the segment before it runs at the same time on the same XCD, so most of them come out
+        // of L2: FETCH_SIZE reads 1.12 x the bytes read with 2 chunks, 1.25 x with 4; the fixed tiles read 1.08 x and write
+        // 1.09 x (partial lines stored twice), the strips write 1.03 x (the two ends of every row).
         const uint32_t chunk = 128 / unit, rows_per_strip = 256 / unit;
         const uint64_t Wn = PACK ? Sc : Q, Xn = PACK ? Q : Sc;
         a.base = base;
@@ -888,7 +894,7 @@ bool try_transpose_copy(char* base, char* packed, const CanonSlice& c, uint32_t 
         a.offset = c.offset;
         a.Sc = (uint32_t)Sc;
         a.Q = (uint32_t)Q;
-        a.seg_len = 4 * chunk;
+        a.seg_len = seg_chunks * chunk;
         a.nseg = (uint32_t)((Xn + a.seg_len - 1) / a.seg_len);
         a.nstrips = (uint32_t)((Wn + rows_per_strip - 1) / rows_per_strip);
         a.ntiles = nbatch * a.nseg * a.nstrips;

@@ -27,7 +27,10 @@ def test_traffic_figures_come_from_the_committed_profile_summary():
     for w, row in table.items():
         assert w in bench.WORKLOADS, w
         assert f"| {row['traffic']} |" in text                      # the very figure the summary states
-        assert 0.9 < row["traffic"] / row["algorithmic"] < 1.1, (w, row)   # no wasted re-reads anywhere
+        # no wasted re-reads: within 2 % of the algorithmic bytes, except the flat unpack (a counter artefact the summary
+        # explains) and the transposing copies of rows that start inside cache lines, which re-read by design
+        limit = 1.1 if w.startswith("tr_") and "8200" in w else 1.02
+        assert (0.95 if w.startswith("c5_flat_unpack") else 0.999) < row["traffic"] / row["algorithmic"] < limit, (w, row)
     assert table["c2"]["algorithmic"] == 9 * 25_165_824 * 2 and table["c3_pack"]["algorithmic"] == 2 * 4096 * 14336 * 2
 
 
