@@ -847,7 +847,8 @@ view (`x[:, :, :cols].transpose(1, 2)` of a `[batch, rows, pitch]` tensor; algor
 size) with one variant forced through `{{envvar}}`; `library` is what the host code picks by itself.  All variants of a
 row are switched in turn inside one process on one GPU: medians of {{reps}} alternations of {{launches}} launches, 3 rotating
 buffer sets.  Matrices of 4096 x 4096 and smaller partly live in the 256 MB Infinity Cache across the three buffer sets.  Shapes whose written rows do not start on cache lines (8200 x 8200, 5000 x 7000) run the kernel with
-line-aligned windows for 2-, 4- and 8-byte elements, under every variant of this table.
+line-aligned windows for 2-, 4- and 8-byte elements under every variant of this table; 1-byte elements of such shapes with at least 1024 strip
+segments (8200 x 8200) run the strip kernel, which has one order of its own and ignores the walk: its columns differ by run-to-run noise only.
 """
 SWEEP_HEADERS = {
     "transpose_walks": "# Transposing pack / unpack: A/B of the tile walks (MI355X)\n\n"

@@ -116,7 +116,8 @@ __device__ __forceinline__ void quantize_bucket_block_careful(uint8_t* __restric
 // cooperative search pair locates the tensors of the first and the last element of the
 // whole span; when they coincide (the common case) all 2 * kBucketBlocks loads of a lane
 // are issued back to back from one base pointer.
-constexpr int kBucketBlocks = 4;
+constexpr uint64_t kSmallBucketBlocks = 32768;  // buckets of up to 33.5 M elements take one block per wavefront step (see quantize_bucket)
+constexpr int kBucketBlocks = 4;       // blocks per wavefront step of the quantiser on large buckets (template parameter NB)
 // Lanes per workgroup.  Unlike the plain copy and the tensor-less quantiser, which stream best as single
 // wavefronts, the bucket kernels want 4 wavefronts: quantise / dequantise / dequantise 8 peers reach
 // 0.75 / 0.735 / 0.72 of peak with 256 lanes, 0.74 / 0.66 / 0.68 with 64 and 0.72 / 0.715 / 0.71 with 512.
@@ -197,15 +198,16 @@ __device__ __forceinline__ Rows<R> load_rows_of_two_tensors(const char* head, co
 // narrowed to its own tensors by a wave-uniform walk over the table; full blocks inside one tensor or shared by two
 // are loaded first, all of them, and quantised then.  Returns the blocks (bit j: block b0 + j) that are left for the
 // careful path.
+template <int NB>
 __device__ __forceinline__ uint32_t quantize_bucket_span_slow(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                               char* const* tensors, const uint64_t* offsets, uint64_t total,
                                                               uint64_t nblocks, uint32_t ntensors, uint32_t t_first, uint32_t t_last,
                                                               uint64_t b0, int lane) {
     uint32_t redo = 0, loaded = 0;
     uint32_t tb = t_first;
-    uint4 row[2 * kBucketBlocks];
+    uint4 row[2 * NB];
 #pragma unroll
-    for (int j = 0; j < kBucketBlocks; ++j) {
+    for (int j = 0; j < NB; ++j) {
         const uint64_t b = b0 + j;
         if (b < nblocks) {
             const uint64_t begin = b * kBlock;
@@ -231,26 +233,28 @@ __device__ __forceinline__ uint32_t quantize_bucket_span_slow(uint8_t* __restric
         }
     }
 #pragma unroll
-    for (int j = 0; j < kBucketBlocks; ++j) {
+    for (int j = 0; j < NB; ++j) {
         const uint64_t b = b0 + j;
         if ((loaded >> j) & 1u)
             if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane)) redo |= 1u << j;
     }
     return redo;
 }
-// The kBucketBlocks blocks of a span whose elements are in registers, row[2j] and row[2j + 1] holding block j.
+// The NB blocks of a span whose elements are in registers, row[2j] and row[2j + 1] holding block j.
 // Returns the blocks (bit j: block b0 + j) that hold Inf or NaN and are left for the careful path.
+template <int NB>
 __device__ __forceinline__ uint32_t quantize_loaded_span(uint8_t* __restrict__ q, float* __restrict__ scales,
-                                                         const uint4 (&row)[2 * kBucketBlocks], uint64_t b0, int lane) {
+                                                         const uint4 (&row)[2 * NB], uint64_t b0, int lane) {
     uint32_t redo = 0;
 #pragma unroll
-    for (int j = 0; j < kBucketBlocks; ++j) {
+    for (int j = 0; j < NB; ++j) {
         const uint64_t b = b0 + j;
         if (!quantize_loaded_block(q, scales, row[2 * j], row[2 * j + 1], b * kBlock, b, lane)) redo |= 1u << j;
     }
     return redo;
 }
 
+template <int NB>
 __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(4))) void fp8_quantize_bucket_kernel(uint8_t* __restrict__ q, float* __restrict__ scales,
                                                                        BucketArgs a) {
     const int lane = threadIdx.x & 63;
@@ -263,20 +267,20 @@ __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(
     // 0.746 -> 0.703, eight peers 0.716 -> 0.703, although buckets of a few MB gain 0.8 us.
     const uint64_t wave = (uint64_t)blockIdx.x * (kBucketThreads / 64) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint64_t nwaves = (uint64_t)gridDim.x * (kBucketThreads / 64);
-    for (uint64_t b0 = wave * kBucketBlocks; b0 < a.nblocks; b0 += nwaves * kBucketBlocks) {
+    for (uint64_t b0 = wave * NB; b0 < a.nblocks; b0 += nwaves * NB) {
         const uint64_t span_begin = b0 * kBlock;
-        const uint64_t span_end = span_begin + (uint64_t)kBucketBlocks * kBlock < a.total
-                                      ? span_begin + (uint64_t)kBucketBlocks * kBlock : a.total;
+        const uint64_t span_end = span_begin + (uint64_t)NB * kBlock < a.total
+                                      ? span_begin + (uint64_t)NB * kBlock : a.total;
         uint32_t t_first, t_last;
         span_tensors(a, span_begin, span_end, &t_first, &t_last);
-        const bool full = span_end - span_begin == (uint64_t)kBucketBlocks * kBlock;
+        const bool full = span_end - span_begin == (uint64_t)NB * kBlock;
         // Blocks that need the careful path are only noted (bit j: block b0 + j; wave-uniform) and worked off in one
         // place at the end of the step, where the span's registers are free: inlined where the rows are live, that
         // path costs the whole kernel a quarter of its wavefronts; as a function that is not inlined, its table reads
         // become vector loads with a round trip each (6 us for one short block).
         uint32_t redo = 0;
         uint32_t t_redo = t_first;     // last tensor those blocks can touch
-        uint4 row[2 * kBucketBlocks];  // row[2j] = first, row[2j + 1] = second 1 KiB of block j
+        uint4 row[2 * NB];  // row[2j] = first, row[2j + 1] = second 1 KiB of block j
         if (t_first == t_last && full) {
             // the whole span lies in one tensor (the common case): all loads of the lane back to back from one base pointer
             const uint64_t t_begin = a.offsets[t_first], t_end = a.offsets[t_first + 1];
@@ -285,14 +289,14 @@ __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(
             if (shift != 0 && (span_begin - t_begin) * 2 >= shift && (t_end - span_end) * 2 >= 16 - shift) {
                 const char* base = src - shift;  // 16-byte aligned, and [base, base + 8 KiB + 16) lies inside the tensor
 #pragma unroll
-                for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_aligned(base + k * 1024 + lane * 16);
-                const uint4 tail = load16_aligned(base + 2 * kBucketBlocks * 1024);
-                shift_rows_into_place<2 * kBucketBlocks>(row, tail, shift);
+                for (int k = 0; k < 2 * NB; ++k) row[k] = load16_aligned(base + k * 1024 + lane * 16);
+                const uint4 tail = load16_aligned(base + 2 * NB * 1024);
+                shift_rows_into_place<2 * NB>(row, tail, shift);
             } else {
 #pragma unroll
-                for (int k = 0; k < 2 * kBucketBlocks; ++k) row[k] = load16_unaligned(src + k * 1024 + lane * 16);
+                for (int k = 0; k < 2 * NB; ++k) row[k] = load16_unaligned(src + k * 1024 + lane * 16);
             }
-            redo = quantize_loaded_span(q, scales, row, b0, lane);
+            redo = quantize_loaded_span<NB>(q, scales, row, b0, lane);
         } else if (full && t_first + 2 <= a.ntensors && a.offsets[t_first + 2] >= span_end) {
             // one tensor ends inside the span and the next one holds the rest (every span that straddles tensors of
             // 4096 elements and more)
@@ -301,7 +305,7 @@ __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(
             const char* rest = reinterpret_cast<const char*>(reinterpret_cast<uintptr_t>(a.tensors[t_first + 1]) - (uintptr_t)cut * 2);
             // as in load_rows_of_two_tensors, on the span's own registers
 #pragma unroll
-            for (int k = 0; k < 2 * kBucketBlocks; ++k) {
+            for (int k = 0; k < 2 * NB; ++k) {
                 uint32_t v0 = k * 512 + lane * 8;
                 if (v0 < cut && v0 + 8 > cut) v0 = v0 >= 8 ? v0 - 8 : 8;
                 if (v0 < cut) row[k] = load16_unaligned(head + v0 * 2);
@@ -319,13 +323,13 @@ __global__ __launch_bounds__(kBucketThreads) __attribute__((amdgpu_waves_per_eu(
                     w[i / 2] = i % 2 ? w[i / 2] | (x << 16) : x;
                 }
 #pragma unroll
-                for (int k = 0; k < 2 * kBucketBlocks; ++k)
+                for (int k = 0; k < 2 * NB; ++k)
                     if (k == (int)cut_row) row[k] = make_uint4(w[0], w[1], w[2], w[3]);  // wave-uniform
             }
-            redo = quantize_loaded_span(q, scales, row, b0, lane);
+            redo = quantize_loaded_span<NB>(q, scales, row, b0, lane);
             t_redo = t_first + 1;
         } else {  // more than two tensors, or the short last span of the bucket
-            redo = quantize_bucket_span_slow(q, scales, a.tensors, a.offsets, a.total, a.nblocks, a.ntensors, t_first, t_last, b0, lane);
+            redo = quantize_bucket_span_slow<NB>(q, scales, a.tensors, a.offsets, a.total, a.nblocks, a.ntensors, t_first, t_last, b0, lane);
             t_redo = t_last;
         }
         for (uint64_t b = b0; redo != 0; ++b, redo >>= 1) {
@@ -594,11 +598,20 @@ static int quantize_bucket(uint8_t* q, float* scales, const void* const* d_tenso
     a.total = total;
     a.nblocks = (total + kBlock - 1) / kBlock;
     a.ntensors = ntensors;
-    const uint64_t per_wg = (kBucketThreads / 64) * kBucketBlocks;
+    // Buckets of up to kSmallBucketBlocks blocks run one block per wavefront step: a launch of a few MB is bound by how long its
+    // wavefronts live (three dependent table reads, then the data), not by bandwidth, and four times as many wavefronts hide
+    // that better; large buckets amortise the look-ups over four blocks.  One / four blocks per step, both in turn on one GPU:
+    // 4.5 M elements 6.0 / 7.9 us (the flat quantiser alone: 5.1), 14 M 10.6 / 12.3 (8.6), 34 M 21.5 / 21.7, 68 M 38.8 / 36.8,
+    // 134 M 73.3 / 66.0, 756 M 0.68 / 0.78 of peak.  With the tuning aids on, MONARCH_HIP_BUCKET_BLOCKS=1 / 4 overrides the
+    // choice at every call (the parity tests run both forms on the same buckets).
+    int nb = a.nblocks <= kSmallBucketBlocks ? 1 : kBucketBlocks;
+    if (const char* e = tuning_env("MONARCH_HIP_BUCKET_BLOCKS")) nb = std::atoi(e) == 1 ? 1 : kBucketBlocks;
+    const uint64_t per_wg = (uint64_t)(kBucketThreads / 64) * nb;
     const uint64_t wgs = (a.nblocks + per_wg - 1) / per_wg;
     const uint64_t cap = max_workgroups(kBucketThreads);
-    MHIP_LAUNCH(fp8_quantize_bucket_kernel, dim3((uint32_t)(wgs > cap ? cap : wgs)), dim3(kBucketThreads), 0, hs, q,
-                       scales, a);
+    const dim3 grid((uint32_t)(wgs > cap ? cap : wgs));
+    if (nb == 1) MHIP_LAUNCH(fp8_quantize_bucket_kernel<1>, grid, dim3(kBucketThreads), 0, hs, q, scales, a);
+    else MHIP_LAUNCH(fp8_quantize_bucket_kernel<kBucketBlocks>, grid, dim3(kBucketThreads), 0, hs, q, scales, a);
     return launch_status();
 }
 

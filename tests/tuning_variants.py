@@ -100,3 +100,24 @@ def test_every_cache_policy_of_the_transposing_kernel_moves_the_same_bytes(polic
         ref = torch.zeros_like(host)
         ref[:, :, :c] = host[:, :, :c]
         assert torch.equal(back.cpu(), ref), (policy, dtype, b, r, c, pitch)
+
+
+@pytest.mark.parametrize("blocks", ["1", "4"])
+def test_fused_quantiser_with_one_and_four_blocks_per_wavefront_step(blocks, monkeypatch):
+    # the library runs one block per step on buckets of up to 32768 blocks and four beyond; both forms, forced in turn
+    # on ragged buckets whose spans straddle one and several tensors, must equal flat pack + quantise bit for bit
+    import numpy as np
+    from monarch_amd import fp8
+    monkeypatch.setenv("MONARCH_HIP_BUCKET_BLOCKS", blocks)
+    g = torch.Generator().manual_seed(90 + int(blocks))
+    for sizes in ([5000, 1, 1024, 777, 30000, 2049, 0, 4096, 4097, 13], [200000], [3] * 700, [1023, 1025, 4095, 4097, 8191, 16385]):
+        tensors = [torch.randn(k, generator=g).bfloat16().to(DEV) for k in sizes]
+        if tensors[0].numel() > 10:
+            tensors[0][7] = float("inf")
+            tensors[0][9] = float("nan")
+        bucket = fp8.FlatBucket(tensors)
+        q_ref, s_ref = fp8.quantize(bucket.pack())
+        for indexed in (True, False):
+            q, s = fp8.quantize_bucket(bucket, indexed=indexed)
+            sync()
+            assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32)), (blocks, sizes[:4], indexed)
