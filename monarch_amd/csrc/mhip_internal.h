@@ -49,6 +49,12 @@ bool same_shape(const CanonSlice& a, const CanonSlice& b);
 constexpr int kCopyManyMax = 64;
 int copy_many(void* const* dst, const void* const* src, const uint64_t* nbytes, uint32_t n, void* stream);
 
+// Argument checks shared by the kernel-launching and the host forms of the mhip_rdmaxcel_* entry points
+// (rdmaxcel_host.cpp): null and misaligned queue memory, queue sizes that are not powers of two, entry sizes.
+int check_wqe(const mhip_wqe_params_t* p, bool send);
+int check_cqe(const int32_t* result, const mhip_cqe_poll_params_t* p);
+int check_ring(const void* dst, const void* src);
+
 // Looks up, once per device, the address of the library's static scratch array on the CURRENT device (the block index
 // of mhip_fp8_quantize_bucket_static).  Called from the set-up entry points so that the data path never does it.
 int prepare_static_scratch();

@@ -1,8 +1,8 @@
 // Device-initiated RDMA, the part that needs no NIC: building send / receive work-queue entries, ringing a
 // doorbell and the single-shot completion-queue poll of rdmaxcel-sys/src/rdmaxcel.cu:82-93,139-160,201-245,
 // 292-326, as kernels on the caller's stream (launch_* of rdmaxcel.cu:122-124,184-190,269-275,358-395) and as
-// host functions (the reference's functions are __host__ __device__, and monarch_rdma/src/rdma_components.rs:88,
-// 880,1159-1163 calls the host side).
+// host functions (rdmaxcel_host.cpp: the reference's functions are __host__ __device__, and
+// monarch_rdma/src/rdma_components.rs:88,880,1159-1163 calls the host side).
 //
 // Nothing here is bandwidth: an entry is 16 to 64 bytes and a call is one launch.  What the reference's launchers
 // cost is a device-wide synchronisation per posted entry and, per poll, a managed allocation, a synchronisation and
@@ -73,28 +73,6 @@ __global__ __launch_bounds__(kPostThreads) void post_transfer_kernel(mhip_wqe_pa
     }
 }
 
-static bool power_of_two(uint32_t v) { return v != 0 && (v & (v - 1)) == 0; }
-
-static int check_wqe(const mhip_wqe_params_t* p, bool send) {
-    if (!p || !p->buf || !p->dbrec) return MHIP_ERR_INVALID_ARGUMENT;
-    if (((uintptr_t)p->buf & 15u) || ((uintptr_t)p->dbrec & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
-    if (send && !power_of_two(p->wqe_cnt)) return MHIP_ERR_INVALID_ARGUMENT;
-    return MHIP_SUCCESS;
-}
-
-static int check_cqe(const int32_t* result, const mhip_cqe_poll_params_t* p) {
-    if (!result || !p || !p->cqe_buf || !p->dbrec) return MHIP_ERR_INVALID_ARGUMENT;
-    if (p->cqe_size != 64 && p->cqe_size != 128) return MHIP_ERR_INVALID_ARGUMENT;
-    if (!power_of_two(p->cqe_cnt)) return MHIP_ERR_INVALID_ARGUMENT;
-    if (((uintptr_t)p->cqe_buf & 3u) || ((uintptr_t)p->dbrec & 3u) || ((uintptr_t)result & 3u)) return MHIP_ERR_INVALID_ARGUMENT;
-    return MHIP_SUCCESS;
-}
-
-static int check_ring(const void* dst, const void* src) {
-    if (!dst || !src || ((uintptr_t)dst & 7u) || ((uintptr_t)src & 7u)) return MHIP_ERR_INVALID_ARGUMENT;
-    return MHIP_SUCCESS;
-}
-
 }  // namespace mhip
 
 using namespace mhip;
@@ -159,31 +137,6 @@ int mhip_rdmaxcel_post_transfer(const mhip_wqe_params_t* params, size_t max_segm
     DeviceGuard guard(hs);
     MHIP_LAUNCH(post_transfer_kernel, dim3(1), dim3(kPostThreads), 0, hs, *params, seg, (uint32_t)n);
     return launch_status();
-}
-
-int mhip_rdmaxcel_send_wqe_host(const mhip_wqe_params_t* params) {
-    if (int rc = check_wqe(params, true)) return rc;
-    mhip_rdmaxcel::send_wqe(*params);
-    return MHIP_SUCCESS;
-}
-
-int mhip_rdmaxcel_recv_wqe_host(const mhip_wqe_params_t* params) {
-    if (int rc = check_wqe(params, false)) return rc;
-    mhip_rdmaxcel::recv_wqe(*params);
-    return MHIP_SUCCESS;
-}
-
-int mhip_rdmaxcel_db_ring_host(void* dst, const void* src) {
-    if (int rc = check_ring(dst, src)) return rc;
-    mhip_rdmaxcel::db_ring(dst, src);
-    mhip_rdmaxcel::release_to_system();
-    return MHIP_SUCCESS;
-}
-
-int mhip_rdmaxcel_cqe_poll_host(int32_t* result, const mhip_cqe_poll_params_t* params) {
-    if (int rc = check_cqe(result, params)) return rc;
-    mhip_rdmaxcel::cqe_poll(result, *params);
-    return MHIP_SUCCESS;
 }
 
 }  // extern "C"

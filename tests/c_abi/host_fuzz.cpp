@@ -1,4 +1,5 @@
-// Host-only fuzz of the library's Slice code (slice_host.cpp) and copy planner (plan.cpp), meant to be
+// Host-only fuzz of the library's Slice code (slice_host.cpp), copy planner (plan.cpp) and host-side work-queue
+// entry builders (rdmaxcel_host.cpp), meant to be
 // built with -fsanitize=address,undefined: random valid and invalid Slices go through every host entry
 // point, and what comes back is checked against the definitions (iter == get, index(get(i)) == i,
 // the canonical form decodes to the same byte offsets as get).  No GPU, no HIP headers.
@@ -275,6 +276,139 @@ int main() {
         CHECK(rc == want);
         if (rc == MHIP_SUCCESS) CHECK(ond == kept && nbc == nb);
     }
+
+    // Work-queue and completion-queue entries built on the calling thread (rdmaxcel_host.cpp).  Queues are heap blocks
+    // of exactly the size the parameters describe, so a store outside a slot is an AddressSanitizer report; the bytes are
+    // compared with the wire format written out one byte at a time (rdmaxcel-sys/src/rdmaxcel.cu:139-160,201-245,292-326).
+    uint64_t n_entries = 0, n_refused = 0;
+    for (int round = 0; round < 20000; ++round) {
+        case_no = 2000000 + round;
+        const uint32_t cnt = below(8) == 0 ? (uint32_t)below(70) : 1u << below(7);   // mostly powers of two, some not
+        const bool pow2 = cnt != 0 && (cnt & (cnt - 1)) == 0;
+        const size_t slots = cnt ? cnt : 1;
+        uint8_t* sq = static_cast<uint8_t*>(std::aligned_alloc(64, slots * 64));
+        uint32_t* dbrec = static_cast<uint32_t*>(std::aligned_alloc(8, 8));
+        for (size_t i = 0; i < slots * 64; ++i) sq[i] = 0xA5;
+        dbrec[0] = dbrec[1] = 0xDEADBEEFu;
+        mhip_wqe_params_t p{};
+        p.laddr = rnd();
+        p.lkey = (uint32_t)rnd();
+        p.wr_id = below(4) == 0 ? rnd() : below(4 * slots + 1);
+        p.signaled = (uint8_t)below(2);
+        p.op_type = below(3) == 0 ? MHIP_MLX5_OPCODE_RDMA_READ : below(2) ? MHIP_MLX5_OPCODE_RDMA_WRITE : MHIP_MLX5_OPCODE_RDMA_WRITE_IMM;
+        p.raddr = rnd();
+        p.rkey = (uint32_t)rnd();
+        p.qp_num = (uint32_t)below(1u << 24);
+        p.length = below(3) == 0 ? rnd() : below(1u << 20);
+        p.buf = sq;
+        p.dbrec = dbrec;
+        p.wqe_cnt = cnt;
+        const unsigned spoil = (unsigned)below(12);     // 0..3 spoil one argument
+        if (spoil == 0) p.buf = nullptr;
+        if (spoil == 1) p.dbrec = nullptr;
+        if (spoil == 2) p.buf = sq + 4 * (1 + below(3));
+        if (spoil == 3) p.dbrec = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(dbrec) + 1 + below(3));
+        const bool bad = spoil < 4 || !pow2;
+        int rc = mhip_rdmaxcel_send_wqe_host(&p);
+        CHECK((rc == MHIP_SUCCESS) == !bad);
+        if (rc != MHIP_SUCCESS) {
+            CHECK(rc == MHIP_ERR_INVALID_ARGUMENT);
+            for (size_t i = 0; i < slots * 64; ++i) CHECK(sq[i] == 0xA5);
+            CHECK(dbrec[0] == 0xDEADBEEFu && dbrec[1] == 0xDEADBEEFu);
+            ++n_refused;
+        } else {
+            const uint32_t idx = (uint32_t)p.wr_id;
+            const size_t at = (size_t)(idx & (cnt - 1)) * 64;
+            uint8_t want[48] = {0};
+            const uint32_t w0 = (idx << 8) | p.op_type, w1 = (p.qp_num << 8) | 3u, len = (uint32_t)p.length;
+            for (int b = 0; b < 4; ++b) { want[b] = (uint8_t)(w0 >> (24 - 8 * b)); want[4 + b] = (uint8_t)(w1 >> (24 - 8 * b)); }
+            want[11] = p.signaled ? 0x0A : 0x00;
+            for (int b = 0; b < 8; ++b) { want[16 + b] = (uint8_t)(p.raddr >> (56 - 8 * b)); want[40 + b] = (uint8_t)(p.laddr >> (56 - 8 * b)); }
+            for (int b = 0; b < 4; ++b) { want[24 + b] = (uint8_t)(p.rkey >> (24 - 8 * b)); want[32 + b] = (uint8_t)(len >> (24 - 8 * b)); want[36 + b] = (uint8_t)(p.lkey >> (24 - 8 * b)); }
+            for (size_t i = 0; i < slots * 64; ++i) CHECK(sq[i] == (i >= at && i < at + 48 ? want[i - at] : 0xA5));
+            const uint32_t rec = (idx + 1u) & 0xFFFFFFu;
+            const uint8_t* d = reinterpret_cast<const uint8_t*>(dbrec + 1);
+            CHECK(d[0] == 0 && d[1] == (uint8_t)(rec >> 16) && d[2] == (uint8_t)(rec >> 8) && d[3] == (uint8_t)rec);
+            CHECK(dbrec[0] == 0xDEADBEEFu);
+            ++n_entries;
+        }
+
+        // the receive entry: 16 bytes at buf itself, any wqe_cnt
+        uint8_t* rq = static_cast<uint8_t*>(std::aligned_alloc(16, 16));
+        for (int i = 0; i < 16; ++i) rq[i] = 0x5A;
+        dbrec[0] = dbrec[1] = 0xDEADBEEFu;
+        p.buf = spoil == 0 ? nullptr : spoil == 2 ? rq + 8 : rq;
+        rc = mhip_rdmaxcel_recv_wqe_host(&p);
+        CHECK((rc == MHIP_SUCCESS) == (spoil >= 4));
+        if (rc == MHIP_SUCCESS) {
+            const uint32_t len = (uint32_t)p.length, rec = (uint32_t)(p.wr_id + 1);
+            for (int b = 0; b < 4; ++b) CHECK(rq[b] == (uint8_t)(len >> (24 - 8 * b)) && rq[4 + b] == (uint8_t)(p.lkey >> (24 - 8 * b)));
+            for (int b = 0; b < 8; ++b) CHECK(rq[8 + b] == (uint8_t)(p.laddr >> (56 - 8 * b)));
+            const uint8_t* d = reinterpret_cast<const uint8_t*>(dbrec);
+            for (int b = 0; b < 4; ++b) CHECK(d[b] == (uint8_t)(rec >> (24 - 8 * b)));
+            CHECK(dbrec[1] == 0xDEADBEEFu);
+            ++n_entries;
+        } else {
+            for (int i = 0; i < 16; ++i) CHECK(rq[i] == 0x5A);
+            ++n_refused;
+        }
+
+        // the doorbell ring: exactly 64 bytes, 8-byte aligned both sides
+        uint8_t* reg = static_cast<uint8_t*>(std::aligned_alloc(8, 64));
+        for (int i = 0; i < 64; ++i) reg[i] = 0;
+        const size_t from = (size_t)below(slots) * 64;
+        const unsigned skew = below(6) == 0 ? 1 + (unsigned)below(7) : 0;
+        rc = mhip_rdmaxcel_db_ring_host(skew && below(2) ? static_cast<void*>(reg + skew) : static_cast<void*>(reg),
+                                        skew ? static_cast<const void*>(sq + from + skew) : static_cast<const void*>(sq + from));
+        CHECK((rc == MHIP_SUCCESS) == (skew == 0));
+        if (rc == MHIP_SUCCESS) for (int i = 0; i < 64; ++i) CHECK(reg[i] == sq[from + i]);
+        else for (int i = 0; i < 64; ++i) CHECK(reg[i] == 0);
+        CHECK(mhip_rdmaxcel_db_ring_host(nullptr, sq) == MHIP_ERR_INVALID_ARGUMENT);
+        std::free(reg);
+        std::free(rq);
+
+        // one look at a completion queue of cqe_cnt entries of 64 or 128 bytes
+        const uint32_t csize = below(10) == 0 ? (uint32_t)(4 * below(40)) : below(2) ? 64u : 128u;
+        const bool cq_ok = pow2 && (csize == 64 || csize == 128);
+        const size_t cq_bytes = slots * (csize ? csize : 4);
+        uint8_t* cq = static_cast<uint8_t*>(std::aligned_alloc(64, (cq_bytes + 63) / 64 * 64));
+        for (size_t i = 0; i < cq_bytes; ++i) cq[i] = (uint8_t)rnd();
+        mhip_cqe_poll_params_t q{};
+        q.cqe_buf = cq;
+        q.cqe_size = csize;
+        q.consumer_index = below(3) == 0 ? (uint32_t)rnd() : (uint32_t)below(4 * slots + 1);
+        q.cqe_cnt = cnt;
+        q.dbrec = dbrec;
+        dbrec[0] = dbrec[1] = 0xDEADBEEFu;
+        int32_t result = -1;
+        rc = mhip_rdmaxcel_cqe_poll_host(&result, &q);
+        CHECK((rc == MHIP_SUCCESS) == cq_ok);
+        if (rc == MHIP_SUCCESS) {
+            const uint8_t* e = cq + (size_t)(q.consumer_index & (cnt - 1)) * csize;
+            const uint8_t op_own = e[csize - 1];
+            const bool owned = (uint32_t)(op_own & 1) == ((q.consumer_index / cnt) & 1u) && (op_own >> 4) != 0xF;
+            if (!owned) {
+                CHECK(result == -1 && dbrec[0] == 0xDEADBEEFu);
+            } else {
+                const uint32_t bc = (uint32_t)e[44] << 24 | (uint32_t)e[45] << 16 | (uint32_t)e[46] << 8 | e[47];
+                CHECK(result == ((op_own >> 4) < 4 ? (int32_t)bc : -2));
+                const uint32_t rec = (q.consumer_index + 1u) & 0xFFFFFFu;
+                const uint8_t* d = reinterpret_cast<const uint8_t*>(dbrec);
+                CHECK(d[0] == 0 && d[1] == (uint8_t)(rec >> 16) && d[2] == (uint8_t)(rec >> 8) && d[3] == (uint8_t)rec);
+            }
+            CHECK(dbrec[1] == 0xDEADBEEFu);
+            ++n_entries;
+        } else {
+            CHECK(rc == MHIP_ERR_INVALID_ARGUMENT && result == -1 && dbrec[0] == 0xDEADBEEFu);
+            ++n_refused;
+        }
+        CHECK(mhip_rdmaxcel_cqe_poll_host(nullptr, &q) == MHIP_ERR_INVALID_ARGUMENT);
+        std::free(cq);
+        std::free(dbrec);
+        std::free(sq);
+    }
+    CHECK(n_entries > 20000 && n_refused > 2000);
+    std::printf("ok: %" PRIu64 " queue entries built and %" PRIu64 " calls refused\n", n_entries, n_refused);
 
     std::printf("ok: %" PRIu64 " valid and %" PRIu64 " invalid slices\n", n_valid, n_invalid);
     return 0;
