@@ -2,7 +2,7 @@
 numpy indexing, reduces and fp8 buckets against the CPU oracle.  Shapes are drawn around the sizes at which the library
 switches kernels (tile, chunk, block and vector widths and their neighbours), buffers start at odd alignments, and guard
 zones either side of every buffer catch stray writes.  Each `*_case` function runs one case and raises AssertionError
-naming it; run as a program it repeats them for a number of seconds: python tests/fuzz_cases.py SECONDS SEED [pack|reduce|fp8]."""
+naming it; run as a program it repeats them for a number of seconds: python tests/fuzz_cases.py SECONDS SEED [pack|many|reduce|scatter|fp8 ...]."""
 import ctypes as C
 import os
 import random
@@ -16,7 +16,8 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 import oracle  # noqa: E402
 from monarch_amd import Slice, fp8  # noqa: E402
 from monarch_amd import reduce as R  # noqa: E402
-from monarch_amd._lib import check, lib  # noqa: E402
+from monarch_amd._lib import check, lib, ptr_array  # noqa: E402
+from monarch_amd.ndslice import slice_array  # noqa: E402
 
 DEV = "cuda:0"
 GUARD = 1 << 16
@@ -115,6 +116,61 @@ def pack_case(gen, tag, max_bytes=6 << 20, max_span_bytes=96 << 20):
     return total * es
 
 
+def many_case(gen, tag, max_bytes=2 << 20, max_span_bytes=24 << 20):
+    """Several views of one base through mhip_slice_pack_many / _unpack_many, staging buffers at staggered alignments."""
+    es = gen.choice([1, 2, 2, 4, 4, 8, 16, 6])
+    k = gen.choice([1, 2, 3, 5, 8, 8, 13])
+    views, span = [], 1
+    family = gen.random() < 0.5
+    if family:   # column blocks of one matrix, as a reshard makes them (unequal widths, the last one ragged)
+        rows, cols = gen.choice(EXTENTS[8:]), gen.choice(EXTENTS[10:])
+        pitch = cols + gen.choice([0, 0, 1, 3, 8])
+        cuts = sorted(gen.sample(range(1, cols), min(k - 1, cols - 1))) if cols > 1 else []
+        for lo, hi in zip([0] + cuts, cuts + [cols]):
+            views.append(Slice(offset=lo, sizes=[rows, hi - lo], strides=[pitch, 1]))
+        span = rows * pitch
+    else:
+        for _ in range(k):
+            v, sp, _ = random_slice(gen, max_bytes // es // k, max_span_bytes // es)
+            views.append(v)
+            span = max(span, sp)
+    if gen.random() < 0.3:
+        views.insert(gen.randrange(len(views) + 1), Slice(offset=0, sizes=[0], strides=[1]))   # an empty view among them
+    mis = gen.choice([0, 0, es, 16, 1, 64])
+    desc = f"{tag} many es={es} mis={mis} views={[(v.offset, list(v.sizes), list(v.strides)) for v in views]}"
+    stream = torch.cuda.current_stream().cuda_stream
+    nbytes = span * es
+    store = torch.randint(0, 256, (GUARD + mis + nbytes + GUARD,), dtype=torch.uint8, device=DEV)
+    host = store.cpu().numpy()
+    hb = host[GUARD + mis: GUARD + mis + nbytes].reshape(span, es)
+    base_ptr = store.data_ptr() + GUARD + mis
+    lens = [len(v) * es for v in views]
+    starts, pos = [], GUARD
+    for i, n in enumerate(lens):
+        pos += gen.choice([0, 1, es, 16, 3, 128])
+        starts.append(pos)
+        pos += n
+    out_store = torch.full((pos + GUARD,), 0xAB, dtype=torch.uint8, device=DEV)
+    outs = ptr_array([out_store.data_ptr() + st for st in starts])
+    arr = slice_array(views)
+    check(lib().mhip_slice_pack_many(outs, base_ptr, arr, len(views), es, stream))
+    torch.cuda.synchronize()
+    got = out_store.cpu().numpy()
+    want = np.full(got.size, 0xAB, dtype=np.uint8)
+    locs = [locations(v) for v in views]
+    for st, n, loc in zip(starts, lens, locs):
+        want[st: st + n] = hb[loc].reshape(-1)
+    assert np.array_equal(got, want), f"pack_many differs or wrote outside its outputs: {desc}"
+    canvas = torch.full_like(store, 0x5C)
+    check(lib().mhip_slice_unpack_many(canvas.data_ptr() + GUARD + mis, outs, arr, len(views), es, stream))
+    torch.cuda.synchronize()
+    hc = np.full(host.size, 0x5C, dtype=np.uint8)
+    for loc in locs:   # views may overlap: they carry the same bytes where they do
+        hc[GUARD + mis: GUARD + mis + nbytes].reshape(span, es)[loc] = hb[loc]
+    assert np.array_equal(canvas.cpu().numpy(), hc), f"unpack_many differs or wrote outside the views: {desc}"
+    return sum(lens)
+
+
 # ---- reduce ----
 
 def _rand_host(gen, dtype, n, seed, scale):
@@ -175,6 +231,63 @@ def reduce_case(gen, tag, max_numel=1 << 21):
     for r in range(n):
         assert r == alias or np.array_equal(_raw(views[r]), _raw(hosts[r])), f"reduce wrote input {r}: {desc}"
     return numel * n
+
+
+def scatter_case(gen, tag, max_len=1 << 18):
+    """mhip_reduce_scatter: members read through a random view (or contiguous), the reduced index space cut into contiguous
+    chunks (the dim-0 rule), column blocks (the fused last-dim form) or strided selections.  Checked against the oracle's
+    plain reduce of the gathered inputs, indexed with numpy."""
+    dtype = gen.choice([torch.float32, torch.float32, torch.bfloat16, torch.bfloat16, torch.float16, torch.float64, torch.int32])
+    G = gen.choice([1, 2, 3, 5, 8, 8, 16])
+    op, code = gen.choice(OPS)
+    if dtype == torch.int32 and op == R.ReduceOp.Avg:
+        op, code = OPS[0]
+    es = torch.empty(0, dtype=dtype).element_size()
+    if gen.random() < 0.5:
+        in_view, L = None, min(max_len, gen.choice(LENGTHS) if gen.random() < 0.5 else int(2 ** gen.uniform(3, 18)))
+        span, loc_in = L, None
+    else:
+        in_view, span, L = random_slice(gen, max_len, (16 << 20) // es)
+        loc_in = locations(in_view)
+    form = gen.choice(["chunks", "columns", "strided"]) if L >= 8 else "strided"
+    out_views = []
+    if form == "chunks":
+        parts = gen.choice([p for p in (1, 2, 4, 8) if L % p == 0])
+        c = L // parts
+        out_views = [Slice(offset=r * c, sizes=[c], strides=[1]) for r in gen.sample(range(parts), gen.randrange(1, parts + 1))]
+    elif form == "columns":
+        cols = gen.choice([d for d in (2, 3, 4, 8, 16, 24, 64, 100, 128, 512, 1000, 4096) if L % d == 0] or [1])
+        rows = L // cols
+        cuts = sorted(gen.sample(range(1, cols), min(gen.choice([0, 1, 3, 7]), cols - 1))) if cols > 1 else []
+        out_views = [Slice(offset=lo, sizes=[rows, hi - lo], strides=[cols, 1]) for lo, hi in zip([0] + cuts, cuts + [cols])]
+    else:
+        for _ in range(gen.choice([1, 2, 4])):
+            st = gen.choice([1, 1, 2, 3, 7])
+            n = gen.randrange(1, max(2, (L - 1) // st + 1))
+            out_views.append(Slice(offset=gen.randrange(0, L - (n - 1) * st), sizes=[n], strides=[st]))
+    desc = (f"{tag} scatter {dtype} G={G} op={op.name} L={L} in_view="
+            f"{None if in_view is None else (in_view.offset, list(in_view.sizes), list(in_view.strides))} "
+            f"outs={[(v.offset, list(v.sizes), list(v.strides)) for v in out_views[:8]]}")
+    scale = 1.0 if op == R.ReduceOp.Prod else gen.choice([0.02, 1.0])
+    hosts = [_rand_host(gen, dtype, span, gen.randrange(1 << 30), scale) for _ in range(G)]
+    group = [h.to(DEV) for h in hosts]
+    pads = [gen.choice([0, 0, 1, 3, 4]) for _ in out_views]
+    ostores = [torch.zeros(len(v) + p + 4, dtype=dtype, device=DEV) for v, p in zip(out_views, pads)]
+    outs = [st[p: p + len(v)] for st, p, v in zip(ostores, pads, out_views)]
+    R.reduce_scatter_views(outs, out_views, group, in_view, op)
+    torch.cuda.synchronize()
+    gathered = [_obits(h) if loc_in is None else _obits(h)[loc_in] for h in hosts]
+    if code in (oracle.SUM, oracle.AVG) and dtype in FLOATS:
+        red = oracle.reduce(gathered, code, half=dtype == torch.float16)
+    else:
+        red = oracle.reduce_op(gathered, code, kind="f16" if dtype == torch.float16 else None)
+    for k, (o, v, st, p) in enumerate(zip(outs, out_views, ostores, pads)):
+        assert _same(_obits(o), red[locations(v)], dtype), f"output {k} differs: {desc}"
+        full = _raw(st).reshape(-1, es)
+        assert not full[:p].any() and not full[p + len(v):].any(), f"wrote beside output {k}: {desc}"
+    for h, d in zip(hosts, group):
+        assert np.array_equal(_raw(d), _raw(h)), f"reduce_scatter wrote an input: {desc}"
+    return L * G
 
 
 # ---- fp8 buckets ----
@@ -263,7 +376,7 @@ def fp8_case(gen, tag, max_tensor=300000):
     return total
 
 
-CASES = {"pack": pack_case, "reduce": reduce_case, "fp8": fp8_case}
+CASES = {"pack": pack_case, "many": many_case, "reduce": reduce_case, "scatter": scatter_case, "fp8": fp8_case}
 
 
 def long_run(seconds, seed, kinds):

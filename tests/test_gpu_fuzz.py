@@ -28,3 +28,17 @@ def test_random_fp8_buckets_match_the_oracle(seed):
     gen = random.Random(seed)
     for i in range(80):
         fuzz_cases.fp8_case(gen, f"seed {seed} case {i}", max_tensor=60000)
+
+
+@pytest.mark.parametrize("seed", [401, 402])
+def test_random_groups_of_views_pack_and_unpack_in_one_call(seed):
+    gen = random.Random(seed)
+    for i in range(200):
+        fuzz_cases.many_case(gen, f"seed {seed} case {i}")
+
+
+@pytest.mark.parametrize("seed", [501, 502])
+def test_random_reduce_scatters_match_the_oracle(seed):
+    gen = random.Random(seed)
+    for i in range(200):
+        fuzz_cases.scatter_case(gen, f"seed {seed} case {i}", max_len=1 << 16)
