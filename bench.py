@@ -339,6 +339,44 @@ def wl_c2p(torch, unpack=False, sets=6):
     return ("c2p_contiguous_unpack" if unpack else "c2p_contiguous_pack"), nbytes, launch, cpu, "contiguous_copy_kernel", "u8"
 
 
+def wl_ref_copy(torch, how="hip", sets=6):
+    """Not this library: the platform's own device-to-device copy of the c2p buffers (48 MiB in, 48 MiB out, same rotation),
+    as context for the fractions the library's copies reach.  how = "hip": hipMemcpyAsync; "torch": Tensor.copy_."""
+    numel = 25_165_824
+    g = torch.Generator(device="cuda:0").manual_seed(2001)
+    bufs = [((torch.randn(numel, generator=g, device="cuda:0") * 0.02).bfloat16(),
+             torch.empty(numel, dtype=torch.bfloat16, device="cuda:0")) for _ in range(sets)]
+    nbytes = 2 * numel * 2
+    if how == "hip":
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        hip.hipMemcpyAsync.restype = C.c_int
+        stream = STREAM()
+        args = [(st.data_ptr(), x.data_ptr()) for x, st in bufs]
+
+        def launch(i):
+            d, s_ = args[i % sets]
+            return hip.hipMemcpyAsync(d, s_, numel * 2, 3, stream)  # 3 = hipMemcpyDeviceToDevice
+    else:
+        def launch(i):
+            x, st = bufs[i % sets]
+            st.copy_(x)
+            return 0
+
+    def cpu():
+        import numpy as np
+        h = bufs[0][0].cpu().view(torch.uint16).numpy()
+        out = np.empty_like(h)
+        t0 = time.perf_counter()
+        for _ in range(5):
+            np.copyto(out, h)
+        dt = (time.perf_counter() - t0) / 5
+        return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "sample": "5 passes of numpy.copyto (memcpy)"}
+
+    return (f"ref_copy_{how}_48mib", nbytes, launch, cpu,
+            "hipMemcpyAsync, device to device (the runtime's kernel)" if how == "hip" else "torch Tensor.copy_ (PyTorch's kernel)", "u8")
+
+
 def wl_c3(torch, unpack=False, sets=3):
     from monarch_amd import Slice, staging
     from monarch_amd._lib import ptr_array
@@ -790,6 +828,9 @@ WORKLOADS = {
     "c2_inplace_separate": lambda t: wl_c2(t, True, separate=True),
     "c2p_pack": lambda t: wl_c2p(t, False),
     "c2p_unpack": lambda t: wl_c2p(t, True),
+    # the platform's own copies of the same buffers, for context
+    "ref_copy_hip": lambda t: wl_ref_copy(t, "hip"),
+    "ref_copy_torch": lambda t: wl_ref_copy(t, "torch"),
     "ragged_pack": lambda t: wl_ragged(t, False), "ragged_unpack": lambda t: wl_ragged(t, True),
     "c3_pack": lambda t: wl_c3(t, False),
     "c3_unpack": lambda t: wl_c3(t, True),
@@ -1104,6 +1145,7 @@ SUMMARY = {
     "c5_flat_pack": 0.60, "c5_quantize": 0.60, "c5_dequant": 0.60, "c5_flat_unpack": 0.60,
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
+    "ref_copy_hip": None, "ref_copy_torch": None,   # not this library: hipMemcpyAsync and torch's copy_ on the c2p buffers
     "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
     "tr_bf16_8200_pack": None, "tr_bf16_8200_unpack": None, "tr_u8_8200_pack": None, "tr_u8_8200_unpack": None,
     # configuration 1 (1 MiB views): launch-bound, reported as time per call
