@@ -977,6 +977,155 @@ def sweep_transpose(which, dtypes, reps=5, launches=30):
             torch.cuda.empty_cache()
 
 
+PLATFORM_HEADER = """\
+# The library's kernels beside the platform's own on the same buffers (MI355X)
+
+Command (repository root, one GPU; under a minute):
+
+    python bench.py --sweep platform > profiles/platform_kernels_same_buffers.md
+
+Context, not a target: the reference holds no device kernel for this path (its data movement is NCCL's, ibverbs' and
+PyTorch's), so the nearest yardstick on this GPU is what the ROCm runtime and PyTorch do with the same bytes.  Every row
+times both sides on the same buffers in one process: HIP events on the launch stream, median of 3 runs of {launches} launches,
+rotating buffer sets; fraction of the 8 TB/s HBM peak over the same algorithmic bytes.  The PyTorch calls are the
+single-kernel forms that compute the same result (checked once per row before timing; `same result` says whether the bytes
+are identical: `torch.mean` adds the eight members in an order of its own, so an element here and there rounds the other way).
+"""
+
+
+def sweep_platform(launches=30):
+    """The library's kernels beside hipMemcpyAsync and PyTorch's own kernels on the same buffers (--sweep platform)."""
+    torch, lib, _ = _load()
+    from monarch_amd import Slice, _torch
+    from monarch_amd import reduce as R
+    torch.cuda.set_device(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpyAsync.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+    hip.hipMemcpyAsync.restype = C.c_int
+
+    def frac(fn, nbytes, nsets):
+        res = []
+        for _ in range(3):
+            for i in range(4):
+                fn(i % nsets)
+            torch.cuda.synchronize()
+            ev = Events(lib, stream)
+            ev.start()
+            for i in range(launches):
+                fn(i % nsets)
+            res.append(nbytes / (ev.stop_ms() / launches) / 1e6 / HBM_PEAK_GBS)
+        return sorted(res)[1]
+
+    torch.manual_seed(7)
+    print(PLATFORM_HEADER.format(launches=launches))
+    print("| operation | algorithmic bytes | this library | platform | platform call | same result |")
+    print("|---|---:|---:|---:|---|---|")
+
+    def row(what, nbytes, ours, theirs, call, same):
+        print(f"| {what} | {nbytes} | {ours:.3f} | {theirs:.3f} | {call} | {same} |", flush=True)
+
+    # contiguous copy, 48 MiB in and out (workload c2p)
+    numel, sets = 25_165_824, 6
+    bufs = [(torch.empty(numel, dtype=torch.bfloat16, device="cuda:0").normal_(), torch.empty(numel, dtype=torch.bfloat16, device="cuda:0"))
+            for _ in range(sets)]
+    s = Slice.new_row_major([numel])
+    calls = [prepared("mhip_slice_pack", st.data_ptr(), x.data_ptr(), C.byref(s.c), 2, STREAM()) for x, st in bufs]
+    ours = frac(lambda i: calls[i](), 4 * numel, sets)
+    ptrs = [(st.data_ptr(), x.data_ptr()) for x, st in bufs]
+    th = frac(lambda i: hip.hipMemcpyAsync(ptrs[i][0], ptrs[i][1], 2 * numel, 3, stream), 4 * numel, sets)
+    row("contiguous pack, 48 MiB", 4 * numel, ours, th, "`hipMemcpyAsync`, device to device", "yes")
+    tt = frac(lambda i: bufs[i][1].copy_(bufs[i][0]), 4 * numel, sets)
+    row("contiguous pack, 48 MiB", 4 * numel, ours, tt, "`dst.copy_(src)`", "yes")
+    del bufs, calls
+    torch.cuda.empty_cache()
+
+    # bf16 bucket reduce, avg over 8 members of 48 MiB (workload c2), members as the rows of one [8, N] tensor
+    sets = 3
+    stacks = [(torch.empty(8, numel, dtype=torch.bfloat16, device="cuda:0").normal_(0, 0.02), torch.empty(numel, dtype=torch.bfloat16, device="cuda:0"),
+               torch.empty(numel, dtype=torch.bfloat16, device="cuda:0")) for _ in range(sets)]
+    nbytes = 18 * numel
+
+    def ours_reduce(i):
+        x, o, _ = stacks[i]
+        R.all_reduce(o, [x[g] for g in range(8)], R.ReduceOp.Avg)
+
+    def torch_reduce(i):
+        x, _, o = stacks[i]
+        torch.mean(x, dim=0, out=o)
+
+    ours_reduce(0)
+    torch_reduce(0)
+    torch.cuda.synchronize()
+    same = "yes" if torch.equal(stacks[0][1].view(torch.int16), stacks[0][2].view(torch.int16)) else \
+        f"no ({(stacks[0][1].view(torch.int16) != stacks[0][2].view(torch.int16)).sum().item()} of {numel} elements differ)"
+    calls = []
+    for x, o, _ in stacks:
+        ptrs_in = (C.c_void_p * 8)(*[x[g].data_ptr() for g in range(8)])
+        calls.append(prepared("mhip_reduce", o.data_ptr(), ptrs_in, 8, numel, _torch.dtype_code(torch.bfloat16), int(R.ReduceOp.Avg), STREAM()))
+    ours = frac(lambda i: calls[i](), nbytes, sets)
+    tt = frac(torch_reduce, nbytes, sets)
+    row("bf16 reduce, avg of 8 x 48 MiB", nbytes, ours, tt, "`torch.mean(x[8, N], dim=0, out=o)`", same)
+    del stacks, calls
+    torch.cuda.empty_cache()
+
+    # column block of a [4096, 14336] bf16 matrix (one of workload c3's eight views), and all eight
+    rows_, cols_, w = 4096, 14336, 1792
+    sets = 3
+    mats = [(torch.empty(rows_, cols_, dtype=torch.bfloat16, device="cuda:0").normal_(), torch.empty(8, rows_, w, dtype=torch.bfloat16, device="cuda:0"),
+             torch.empty(8, rows_, w, dtype=torch.bfloat16, device="cuda:0")) for _ in range(sets)]
+    views = [Slice(offset=k * w, sizes=[rows_, w], strides=[cols_, 1]) for k in range(8)]
+
+    from monarch_amd._lib import ptr_array
+    from monarch_amd.ndslice import slice_array
+    varr = slice_array(views)
+    c3calls = [prepared("mhip_slice_pack_many", ptr_array([o[k].data_ptr() for k in range(8)]), x.data_ptr(), varr, 8, 2, STREAM())
+               for x, o, _ in mats]
+
+    def ours_c3(i):
+        return c3calls[i]()
+
+    def torch_c3(i):
+        x, _, o = mats[i]
+        o.copy_(x.view(rows_, 8, w).transpose(0, 1))
+
+    ours_c3(0)
+    torch_c3(0)
+    torch.cuda.synchronize()
+    same = "yes" if torch.equal(mats[0][1].view(torch.int16), mats[0][2].view(torch.int16)) else "no"
+    nbytes = 4 * rows_ * cols_
+    row("8 column blocks of [4096, 14336] bf16", nbytes, frac(ours_c3, nbytes, sets), frac(torch_c3, nbytes, sets),
+        "`o[8, R, w].copy_(x.view(R, 8, w).transpose(0, 1))`", same)
+    del mats
+    torch.cuda.empty_cache()
+
+    # transposing packs
+    for name, dt, es, n in (("bf16", torch.bfloat16, 2, 8192), ("f32", torch.float32, 4, 8192), ("u8", torch.uint8, 1, 8192),
+                            ("bf16", torch.bfloat16, 2, 8200), ("u8", torch.uint8, 1, 8200)):
+        sets = 3 if es > 1 else 6
+        tb = []
+        for _ in range(sets):
+            x = torch.empty(n, n, dtype=dt, device="cuda:0")
+            x.view(torch.uint8).random_(0, 255)
+            tb.append((x, torch.empty(n * n, dtype=dt, device="cuda:0"), torch.empty(n, n, dtype=dt, device="cuda:0")))
+        sl = Slice.of_tensor(tb[0][0].t())
+        calls = [prepared("mhip_slice_pack", o.data_ptr(), x.data_ptr(), C.byref(sl.c), es, STREAM()) for x, o, _ in tb]
+
+        def torch_tr(i):
+            x, _, o = tb[i]
+            o.copy_(x.t())
+
+        calls[0]()
+        torch_tr(0)
+        torch.cuda.synchronize()
+        same = "yes" if torch.equal(tb[0][1].view(torch.uint8), tb[0][2].view(-1).view(torch.uint8)) else "no"
+        nbytes = 2 * n * n * es
+        row(f"transposing pack {n} x {n} {name}", nbytes, frac(lambda i: calls[i](), nbytes, sets), frac(torch_tr, nbytes, sets),
+            "`o.copy_(x.t())`", same)
+        del tb, calls
+        torch.cuda.empty_cache()
+
+
 STRIDED_VIEWS_HEADER = """\
 # Strided pack / unpack of one column range: row length x alignment (MI355X)
 
@@ -1282,11 +1431,14 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views", "bucket_sizes"], help="print a table instead of the bench line")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views", "bucket_sizes", "platform"], help="print a table instead of the bench line")
     ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep == "platform":
+        sweep_platform()
+        return
     if args.sweep == "bucket_sizes":
         sweep_bucket_sizes()
         return
