@@ -715,9 +715,19 @@ def wl_c5(torch, stage="quantize"):
         nbytes, kern = 3 * total + 4 * nblk, "fp8_quantize_bucket_kernel"
         launch = prepared("mhip_fp8_quantize_bucket", q.data_ptr(), s.data_ptr(), bucket.d_ptrs.data_ptr(),
                           bucket.d_offsets.data_ptr(), len(sizes), total, 1024, index, STREAM())
-    elif stage == "dequant_bucket":
+    elif stage in ("dequant_bucket", "dequant_bucket_arena"):
         nbytes, kern = 9 * total + 4 * nblk, "fp8_dequant_accumulate_bucket_kernel"
-        accs = [torch.zeros(n, device="cuda:0") for n in sizes]
+        if stage.endswith("arena"):
+            # the same accumulators carved out of one allocation, each starting on a 256-byte boundary (so not the flat
+            # layout): what the kernel does when 1500 separate allocations are not in the way
+            starts, at = [], 0
+            for n in sizes:
+                starts.append(at)
+                at += (n + 63) // 64 * 64
+            arena = torch.zeros(at, device="cuda:0")
+            accs = [arena[st: st + n] for st, n in zip(starts, sizes)]
+        else:
+            accs = [torch.zeros(n, device="cuda:0") for n in sizes]
         aptrs = bucket.pointer_table(accs)
         launch = prepared("mhip_fp8_dequant_accumulate_bucket", aptrs.data_ptr(), q.data_ptr(), s.data_ptr(),
                           bucket.d_offsets.data_ptr(), len(sizes), total, 1024, index, STREAM())
@@ -854,6 +864,7 @@ WORKLOADS = {
     "c5_dequant": lambda t: wl_c5(t, "dequant_accumulate"),
     "c5_quantize_bucket": lambda t: wl_c5(t, "quantize_bucket"),
     "c5_dequant_bucket": lambda t: wl_c5(t, "dequant_bucket"),
+    "c5_dequant_bucket_arena": lambda t: wl_c5(t, "dequant_bucket_arena"),
     "c5_quantize_bucket_search": lambda t: wl_c5(t, "quantize_bucket_search"),
     "c5_dequant_bucket_search": lambda t: wl_c5(t, "dequant_bucket_search"),
     "c5_flat_unpack": lambda t: wl_c5(t, "flat_unpack"),
@@ -1294,6 +1305,7 @@ SUMMARY = {
     "c5_flat_pack": 0.60, "c5_quantize": 0.60, "c5_dequant": 0.60, "c5_flat_unpack": 0.60,
     "c5_quantize_bucket": 0.60, "c5_dequant_bucket": 0.60, "c5_dequant_many8": 0.60,
     "stack8": None, "stack_scatter8": None,
+    "c5_dequant_bucket_arena": None,   # c5_dequant_bucket with the 1500 accumulators inside one allocation
     "ref_copy_hip": None, "ref_copy_torch": None,   # not this library: hipMemcpyAsync and torch's copy_ on the c2p buffers
     "tr_f32_pack": None, "tr_f32_unpack": None, "tr_bf16_pack": None, "tr_bf16_unpack": None,
     "tr_bf16_8200_pack": None, "tr_bf16_8200_unpack": None, "tr_u8_8200_pack": None, "tr_u8_8200_unpack": None,
