@@ -238,7 +238,8 @@ int mhip_slice_subview(const mhip_slice_t* s, const uint64_t* starts, uint32_t n
 int mhip_slice_view(const mhip_slice_t* s, const uint64_t* new_sizes, uint32_t nnew, uint64_t* out_strides) {
     if (bad(s) || nnew > MHIP_MAX_DIMS || (nnew && (!new_sizes || !out_strides))) return MHIP_ERR_INVALID_ARGUMENT;
     uint64_t want = 1;
-    for (uint32_t k = 0; k < nnew; ++k) want *= new_sizes[k];
+    for (uint32_t k = 0; k < nnew; ++k)
+        if (__builtin_mul_overflow(want, new_sizes[k], &want)) return MHIP_ERR_INCOMPATIBLE_VIEW;  // no slice holds 2^64 elements
     if (want != slice_len(*s) || s->offset != 0) return MHIP_ERR_INCOMPATIBLE_VIEW;  // slice.rs:594-606
     uint64_t acc = 1;
     for (uint32_t k = nnew; k-- > 0;) {
@@ -307,7 +308,8 @@ int mhip_mesh_ranks_for_dims(const mhip_slice_t* ranks, uint64_t rank, const uin
         // a one-member dimension contributes stride 0 (device_mesh.rs:148-154)
         sub_strides[d] = sub_sizes[d] > 1 ? ranks->strides[dims[d]] : 0;
         origin -= sub_strides[d] * coord[dims[d]];
-        total *= sub_sizes[d];
+        // a dimension named twice can make the product wrap: such a group fits no buffer
+        if (__builtin_mul_overflow(total, sub_sizes[d], &total)) return MHIP_ERR_INVALID_ARGUMENT;
     }
     if (total > cap || (total && !out)) return MHIP_ERR_INVALID_ARGUMENT;
     const mhip_slice_t group{origin, ndims, sub_sizes, sub_strides};

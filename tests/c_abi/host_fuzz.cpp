@@ -158,6 +158,36 @@ int main() {
             CHECK(mhip_slice_at(&s, dim, sizes[dim], &aoff, asz.data(), ast.data()) != MHIP_SUCCESS);
         }
 
+        // view: a reshape of the same element count succeeds exactly when the slice starts at 0 and every offset of
+        // [0, len) is one of its locations (slice.rs:579-635); the strides that come back are row-major
+        if (len && len <= 4096) {
+            uint64_t ns[3] = {1, 1, 1};
+            uint64_t rest = len;
+            for (int k = 0; k < 2; ++k) {
+                uint64_t f = 1 + below(rest < 9 ? rest : 9);
+                while (rest % f) --f;
+                ns[k] = f;
+                rest /= f;
+            }
+            ns[2] = rest;
+            uint64_t vst[3] = {7, 7, 7};
+            const int vrc = mhip_slice_view(&s, ns, 3, vst);
+            std::vector<char> member(len, 0);
+            bool dense = offset == 0;
+            for (uint64_t i = 0; i < len && dense; ++i) {
+                if (locs[i] >= len) dense = false;
+                else member[locs[i]] = 1;
+            }
+            for (uint64_t i = 0; i < len && dense; ++i) dense = member[i] != 0;
+            CHECK((vrc == MHIP_SUCCESS) == dense);
+            if (vrc == MHIP_SUCCESS) CHECK(vst[2] == 1 && vst[1] == ns[2] && vst[0] == ns[1] * ns[2]);
+            else CHECK(vrc == MHIP_ERR_INCOMPATIBLE_VIEW);
+            ns[2] += 1;
+            CHECK(mhip_slice_view(&s, ns, 3, vst) == MHIP_ERR_INCOMPATIBLE_VIEW);   // another element count
+            const uint64_t wrap[2] = {1ull << 32, 1ull << 32};                     // a product that wraps to 0
+            CHECK(mhip_slice_view(&s, wrap, 2, vst) == MHIP_ERR_INCOMPATIBLE_VIEW);
+        }
+
         // the planner: every packed byte lands where the definition says, for several element sizes,
         // address alignments and unit limits
         for (int rep = 0; rep < 3; ++rep) {
@@ -198,6 +228,39 @@ int main() {
                 uint64_t dim_rank = ~0ull;
                 CHECK(mhip_mesh_dim_members(&s, rank, dim, members.data(), &dim_rank) == MHIP_SUCCESS);
                 CHECK(dim_rank < sizes[dim] && members[dim_rank] == rank && members[sizes[dim]] == ~0ull);
+            }
+            // the reduce group of a random list of dimensions, in the caller's order: row-major over those dimensions,
+            // the rank's own coordinates everywhere else (device_mesh.rs:120-177)
+            uint32_t dims[8];
+            uint32_t ndims = (uint32_t)below(nd + 1);
+            std::vector<uint32_t> pool(nd);
+            for (uint32_t k = 0; k < nd; ++k) pool[k] = k;
+            for (uint32_t k = nd; k > 1; --k) std::swap(pool[k - 1], pool[below(k)]);
+            uint64_t group = 1;
+            for (uint32_t d = 0; d < ndims; ++d) { dims[d] = pool[d]; group *= sizes[pool[d]]; }
+            std::vector<uint64_t> out(group + 1, ~0ull);
+            uint64_t count = ~0ull;
+            CHECK(mhip_mesh_ranks_for_dims(&s, rank, dims, ndims, out.data(), group, &count) == MHIP_SUCCESS);
+            if (ndims == 0) {
+                CHECK(count == 0);
+            } else {
+                CHECK(count == group && out[group] == ~0ull);
+                std::vector<uint64_t> own(nd), c(nd);
+                CHECK(mhip_slice_coordinates(&s, rank, own.data()) == MHIP_SUCCESS);
+                bool has_self = false;
+                for (uint64_t i = 0; i < group; ++i) {
+                    c = own;
+                    uint64_t rem = i;
+                    for (uint32_t d = ndims; d-- > 0;) { c[dims[d]] = rem % sizes[dims[d]]; rem /= sizes[dims[d]]; }
+                    uint64_t want = 0;
+                    CHECK(mhip_slice_location(&s, c.data(), nd, &want) == MHIP_SUCCESS);
+                    CHECK(out[i] == want);
+                    has_self |= out[i] == rank;
+                }
+                CHECK(has_self);
+                if (group > 1) CHECK(mhip_mesh_ranks_for_dims(&s, rank, dims, ndims, out.data(), group - 1, &count) == MHIP_ERR_INVALID_ARGUMENT);
+                dims[0] = nd;
+                CHECK(mhip_mesh_ranks_for_dims(&s, rank, dims, ndims, out.data(), group, &count) == MHIP_ERR_DIMENSION_OUT_OF_RANGE);
             }
         }
     }
