@@ -2,7 +2,7 @@
 kernels are launched in several pieces.  Inputs large enough to reach that bound (64 GiB per view) do
 not belong in a test suite, so the bound is lowered through MONARCH_HIP_MAX_LAUNCH_LANES (a tuning aid, honoured
 only with MONARCH_HIP_TUNING=1 at load time) and the
-pack, reduce, fp8 and graph-capture tests are run again in a child process: with 8192 lanes per launch nearly
+pack, reduce, fp8, graph-capture and random-case tests are run again in a child process: with 8192 lanes per launch nearly
 every case takes the clamped or the multi-piece path."""
 import os
 import subprocess
@@ -17,7 +17,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 @pytest.mark.timeout(900)
 def test_parity_suites_pass_with_a_tiny_launch_bound():
     env = dict(os.environ, MONARCH_HIP_TUNING="1", MONARCH_HIP_MAX_LAUNCH_LANES="8192")
-    files = ["tests/test_gpu_pack.py", "tests/test_gpu_reduce.py", "tests/test_gpu_fp8.py", "tests/test_gpu_graph_capture.py"]
+    files = ["tests/test_gpu_pack.py", "tests/test_gpu_reduce.py", "tests/test_gpu_fp8.py", "tests/test_gpu_graph_capture.py",
+             "tests/test_gpu_fuzz.py"]
     r = subprocess.run([sys.executable, "-u", "-m", "pytest", "-x", "-q", "-m", "gpu", "--timeout", "300",
                         "--timeout-method", "thread", "-p", "no:cacheprovider", *files],
                        cwd=ROOT, env=env, capture_output=True, text=True, timeout=850)
