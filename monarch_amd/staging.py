@@ -152,6 +152,10 @@ class RDMABuffer:
         return RdmaBufferC(self.addr + offset, self.size - offset)
 
     def read_into(self, dst: torch.Tensor, offset: int = 0, stream=None) -> int:
+        """Copies ``dst.numel()`` bytes of the buffer, from byte ``offset`` of it, into ``dst``.  (In the reference
+        ``offset`` is added to the local address and then checked against ``dst.numel()``
+        (python/monarch/_src/tensor_engine/rdma.py:160-165), which only ``offset == 0`` passes; every call that succeeds
+        there means the same here, and a non-zero offset addresses the registered range instead of raising.)"""
         _assert_tensor_is_1d_contiguous_uint8(dst)
         _torch.require_device(dst)
         size = dst.numel()
@@ -162,6 +166,7 @@ class RDMABuffer:
         return size
 
     def write_from(self, src: torch.Tensor, offset: int = 0, stream=None) -> None:
+        """Copies ``src`` into the buffer at byte ``offset`` of it (rdma.py:187-214; ``offset`` as in ``read_into``)."""
         _assert_tensor_is_1d_contiguous_uint8(src)
         _torch.require_device(src)
         size = src.numel()
