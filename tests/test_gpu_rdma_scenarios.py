@@ -80,3 +80,37 @@ def test_offsets_and_bounds_of_a_registered_buffer():
         buf.read_into(part, offset=241)
     with pytest.raises(ValueError, match="must be <="):
         buf.write_from(part, offset=241)
+
+
+@pytest.mark.parametrize("size", [8, (1 << 20) + 5])
+def test_parameter_server_example_sums_the_workers_gradient_chunks(size):
+    # monarch_rdma/examples/parameter_server/parameter_server.rs: BUFFER_SIZE = 8 bytes per buffer (:89), every worker
+    # computes gradient += weights + 1 (:337-343) and pushes it into its own chunk on the server (:368-370), the server adds
+    # every chunk to its weights with wrapping_add and wipes the chunks (:200-206), the workers pull the weights (:411-413).
+    # With N workers all bytes follow w <- w + N (w + 1) mod 256.  The server's sum is one mhip_reduce over
+    # [weights, chunk_0 .. chunk_N-1], in place on the weights.
+    from monarch_amd import reduce as R
+    n_workers, steps = 4, 5
+    ps_weights = torch.zeros(size, dtype=torch.uint8, device=DEV)
+    ps_chunks = [torch.zeros(size, dtype=torch.uint8, device=DEV) for _ in range(n_workers)]
+    weights_handle = RDMABuffer(ps_weights)
+    grad_handles = [RDMABuffer(c) for c in ps_chunks]
+    workers = [dict(weights=torch.zeros(size, dtype=torch.uint8, device=DEV), grads=torch.zeros(size, dtype=torch.uint8, device=DEV))
+               for _ in range(n_workers)]
+    w = 0
+    for _ in range(steps):
+        for rank, wk in enumerate(workers):                      # WorkerStep
+            wk["grads"] += wk["weights"] + 1
+            grad_handles[rank].write_from(wk["grads"])
+            wk["grads"].zero_()
+        R.all_reduce(ps_weights, [ps_weights] + ps_chunks, R.ReduceOp.Sum)   # PsUpdate
+        for c in ps_chunks:
+            c.zero_()
+        for wk in workers:                                       # WorkerUpdate
+            weights_handle.read_into(wk["weights"])
+        sync()
+        w = (w + n_workers * (w + 1)) % 256
+        assert ps_weights.unique().tolist() == [w]
+        for wk in workers:
+            assert torch.equal(wk["weights"], ps_weights)
+    assert w == (((((0 + 4) + 20) + 100) + 500) + 4 * 113) % 256    # 4, 24, 124, 112 (wrapped), 52 (wrapped)
