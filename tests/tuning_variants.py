@@ -121,3 +121,49 @@ def test_fused_quantiser_with_one_and_four_blocks_per_wavefront_step(blocks, mon
             q, s = fp8.quantize_bucket(bucket, indexed=indexed)
             sync()
             assert torch.equal(q, q_ref) and torch.equal(s.view(torch.int32), s_ref.view(torch.int32)), (blocks, sizes[:4], indexed)
+
+
+def test_random_transposing_views_through_every_form_of_the_kernels():
+    # seeded random shapes around the tile sizes (extents of a tile minus one, a tile, a tile and a bit, halves, tiny ones,
+    # batches, views that start inside the matrix, pitches that put no written row on a cache line), each through a
+    # form drawn at random: the library's choice, fixed tiles, per-tile windows, strips with segments of 1, 2 and 4 chunks
+    import ctypes as C
+    import random
+    libc = C.CDLL(None)
+    gen = random.Random(2718)
+    forms = [None, "0", "1", "2", "2,1", "2,4"]
+    try:
+        for n in range(600):
+            dtype = gen.choice([torch.uint8, torch.uint8, torch.int16, torch.int16, torch.int32, torch.int64])
+            t = 256 // torch.empty(0, dtype=dtype).element_size()
+
+            def extent():
+                if gen.random() < 0.4:
+                    return gen.choice([t - 1, t, t + 1, 2 * t - 1, 2 * t, 2 * t + 1, 3 * t + 5, t // 2, t // 2 + 1, 7, 1])
+                return int(2 ** gen.uniform(0, 10.5))
+            b, rows, cols = gen.choice([1, 1, 1, 2, 3]), extent(), extent()
+            pitch = cols + gen.choice([0, 0, 1, 3, 8, 64, 65])
+            r0, c0 = gen.choice([0, 0, 1, 5]), gen.choice([0, 0, 1, 2, 7])
+            if rows <= r0 or cols <= c0:
+                continue
+            form = gen.choice(forms)
+            if form is None:
+                libc.unsetenv(b"MONARCH_HIP_TRANSPOSE_LINES")
+            else:
+                libc.setenv(b"MONARCH_HIP_TRANSPOSE_LINES", form.encode(), 1)
+            info = torch.iinfo(dtype)
+            host = torch.randint(info.min, info.max, (b, rows, pitch), dtype=dtype)
+            dev = host.to(DEV)
+            view, hview = dev[:, r0:, c0:cols].transpose(1, 2), host[:, r0:, c0:cols].transpose(1, 2)
+            s = Slice.of_tensor(view)
+            out = staging.pack(view, s)
+            sync()
+            assert torch.equal(out.cpu(), hview.contiguous().flatten()), (n, dtype, b, rows, cols, pitch, r0, c0, form)
+            back = torch.full_like(dev, 7)
+            staging.unpack(back, s, out)
+            sync()
+            ref = torch.full_like(host, 7)
+            ref[:, r0:, c0:cols] = host[:, r0:, c0:cols]
+            assert torch.equal(back.cpu(), ref), (n, dtype, b, rows, cols, pitch, r0, c0, form)
+    finally:
+        libc.unsetenv(b"MONARCH_HIP_TRANSPOSE_LINES")
