@@ -8,8 +8,10 @@
  * >= 10000 = the library's own classes below).  Device entry points enqueue on the
  * caller's stream and never synchronise; completion is observed the way the
  * reference does it, by recording an event on that stream afterwards
- * (monarch_tensor_worker/src/comm.rs:156).  All device pointers are caller-owned;
- * the library allocates nothing.  Entry points may be called from any thread; the
+ * (monarch_tensor_worker/src/comm.rs:156).  All device pointers are caller-owned:
+ * no data-path entry point allocates or frees device memory (the only allocating
+ * calls are the explicit mhip_staging_alloc, mhip_stream_create and mhip_event_create
+ * near the end of this file).  Entry points may be called from any thread; the
  * device is taken from the stream (or is the current device for the NULL stream).
  *
  * Units: a Slice counts ELEMENTS (ndslice/src/slice.rs:85-90); pack/unpack take the
