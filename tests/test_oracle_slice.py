@@ -150,6 +150,9 @@ def test_len_contiguous_rowmajor():
     for x in range(2):
         for y in range(2):
             assert sub.location([x, y]) == s.location([x, 3, y])
+    # test_at_1d_to_0d, slice.rs:1031-1043
+    zero_d = OSlice.row_major([5]).at(0, 3)
+    assert (zero_d.offset, zero_d.sizes, zero_d.strides) == (3, [], []) and zero_d.location([]) == 3
 
 
 def test_subview_inclusion():
