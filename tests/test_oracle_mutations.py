@@ -104,6 +104,40 @@ MUTATIONS = [
      lambda: S.test_validation_rules()),
     ("location_adds_no_offset", "o_slice_location", "uint64_t v = s->offset;", "uint64_t v = 0;",
      lambda: S.test_len_contiguous_rowmajor()),     # the doc example slice.rs:72-80 and test_at_1d_to_0d, :1031-1043
+    ("iter_walks_column_major", "o_slice_iter", "for (uint32_t k = s->ndim; k-- > 0;) {\n            coord[k] = rest % s->sizes[k];",
+     "for (uint32_t k = 0; k < s->ndim; k++) {\n            coord[k] = rest % s->sizes[k];", lambda: S.test_iter_vectors(_vectors())),
+    ("coordinates_peels_small_strides_first", "o_slice_coordinates", "for (uint32_t r = n; r-- > 0;) {", "for (uint32_t r = 0; r < n; r++) {",
+     lambda: S.test_coordinates_index_vectors(_vectors())),
+    ("coordinates_accepts_a_remainder", "o_slice_coordinates", "if (pos != 0) return O_ERR_VALUE_NOT_IN_SLICE;", "",
+     lambda: S.test_named_and_fuzz_check(_vectors())),   # test_ndslice.py:127-131: no extra elements between the slice's own
+    ("index_is_column_major", "o_slice_index", "for (uint32_t k = s->ndim; k-- > 0;) {", "for (uint32_t k = 0; k < s->ndim; k++) {",
+     lambda: S.test_coordinates_index_vectors(_vectors())),
+    ("select_rounds_the_count_down", "o_slice_select", "(end - begin + step - 1) / step", "(end - begin) / step",
+     lambda: S.test_select_at_view_embedding_vectors(_vectors())),
+    ("select_keeps_the_stride", "o_slice_select", "out_strides[dim] *= step;", "",
+     lambda: S.test_select_at_view_embedding_vectors(_vectors())),
+    ("at_keeps_the_offset", "o_slice_at", "*out_offset = s->offset + index * s->strides[dim];", "*out_offset = s->offset;",
+     lambda: S.test_select_at_view_embedding_vectors(_vectors())),
+    ("subview_checks_starts_only", "o_slice_subview", "starts[d] + lens[d] > s->sizes[d]", "starts[d] >= s->sizes[d]",
+     lambda: S.test_subview_inclusion()),
+    ("view_accepts_an_offset", "o_slice_view", "if (s->offset != 0) return O_ERR_INCOMPATIBLE_VIEW;", "",
+     lambda: S.test_select_at_view_embedding_vectors(_vectors())),
+    ("unpack_writes_packed_order", "o_slice_unpack", "(char*)dst_base + loc * elem_size", "(char*)dst_base + i * elem_size",
+     lambda: S.test_pack_unpack_against_as_strided()),
+    ("pack_runs_all_cores_starts_rows_at_the_offset", "o_pack_runs_mt", "o_slice_get(s, r * run, &loc);", "loc = s->offset + r * run;",
+     lambda: S.test_pack_unpack_against_as_strided()),
+    ("mesh_members_start_at_the_rank", "o_mesh_dim_members", "uint64_t start = rank - stride * coords[dim];", "uint64_t start = rank;",
+     lambda: S.test_device_mesh_vectors(_vectors())),
+    ("stack_interleaves_members", "o_stack", "[(uint64_t)g * numel * elem_size + b]", "[(uint64_t)b * n + g]",
+     lambda: K.test_stack_matches_reference_all_gather_vector()),
+    ("flat_unpack_reads_from_the_start", "o_flat_unpack", "(const char*)flat + offsets[t] * elem_size", "(const char*)flat",
+     lambda: T.test_fp8_dequant_accumulate_and_flat()),
+    ("f16_subnormals_flush_to_zero", "f32_to_f16_rne", "uint32_t m = (uint32_t)rintf(ldexpf(av, 24));", "uint32_t m = 0;",
+     lambda: T.test_f16_round_matches_torch()),
+    ("f16_overflow_saturates_instead_of_infinity", "f32_to_f16_rne", "if (e >= 31) return (uint16_t)(sign | 0x7c00u);", "if (e >= 31) return (uint16_t)(sign | 0x7bffu);",
+     lambda: T.test_f16_round_matches_torch()),
+    ("u8_sum_saturates", "o_reduce_u8", "acc = (uint8_t)(acc + in[r][i]);", "acc = (uint8_t)(acc + in[r][i] > 255 ? 255 : acc + in[r][i]);",
+     lambda: T.test_reduce_integer_wraps()),
     # bf16 rounding and the plain reduces
     ("bf16_ties_round_away_from_zero", "f32_to_bf16_rne", "u += 0x7fffu + lsb;", "u += 0x8000u;",
      lambda: T.test_bf16_round_matches_torch()),

@@ -78,6 +78,11 @@ def test_select_at_view_embedding_vectors(vec):
         else:
             v = s.view(case["new_sizes"])
             assert v.strides == case["strides"] and v.offset == 0, case["src"]
+    # slice.rs:601-606: a base that does not start at 0 is refused even when it is empty (every other such base already
+    # fails the membership test of offset 0)
+    with pytest.raises(OracleError) as e:
+        OSlice(3, [0], [1]).view([0])
+    assert e.value.name == "IncompatibleView"
     for case in vec["embedding"]:
         base, view = mk(case["base"]), mk(case["view"])
         if case["ok"]:
