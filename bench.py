@@ -1137,6 +1137,67 @@ def sweep_platform(launches=30):
         torch.cuda.empty_cache()
 
 
+REDUCE_OPS_HEADER = """\
+# mhip_reduce over element types, member counts and ops (MI355X)
+
+Command (repository root, one GPU; about a minute):
+
+    python bench.py --sweep reduce_ops > profiles/reduce_ops_dtypes.md
+
+Every cell is the fraction of the 8 TB/s HBM peak that `mhip_reduce` reaches on n members of 48 MiB each into a separate
+48 MiB output (algorithmic bytes = (n + 1) x 48 MiB), members and outputs in separate allocations, median of 3 runs of
+{launches} launches, 2 to 4 rotating buffer sets (at most 3 GiB of them).  Sum and Avg are the ops of the path; Prod, Max and Min
+share one kernel per type that tests the op once per 16-byte vector.
+"""
+
+
+def sweep_reduce_ops(launches=20):
+    """Fraction of HBM peak of mhip_reduce over dtype x member count x op (--sweep reduce_ops)."""
+    torch, lib, _ = _load()
+    from monarch_amd import _torch
+    from monarch_amd import reduce as R
+    torch.cuda.set_device(0)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ops = [R.ReduceOp.Sum, R.ReduceOp.Avg, R.ReduceOp.Prod, R.ReduceOp.Max, R.ReduceOp.Min]
+    print(REDUCE_OPS_HEADER.format(launches=launches))
+    print("| element type | members | " + " | ".join(o.name for o in ops) + " |")
+    print("|---|---:|" + "---:|" * len(ops))
+    for dt in (torch.bfloat16, torch.float16, torch.float32, torch.float64, torch.int32, torch.int64, torch.uint8, torch.int8):
+        es = torch.empty(0, dtype=dt).element_size()
+        numel = (48 << 20) // es
+        for n in (2, 3, 4, 8, 16, 33):
+            sets = max(2, min(4, (3 << 30) // ((n + 1) * (48 << 20))))
+            bufs = []
+            for _ in range(sets):
+                xs = [torch.empty(numel, dtype=dt, device="cuda:0") for _ in range(n)]
+                for x in xs:
+                    x.view(torch.uint8).random_(0, 100)   # small positive values in every type: no NaN, no Inf
+                bufs.append((xs, torch.empty(numel, dtype=dt, device="cuda:0")))
+            cells = []
+            for op in ops:
+                if op == R.ReduceOp.Avg and not dt.is_floating_point:
+                    cells.append("—")
+                    continue
+                calls = []
+                for xs, o in bufs:
+                    ptrs = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+                    calls.append(prepared("mhip_reduce", o.data_ptr(), ptrs, n, numel, _torch.dtype_code(dt), int(op), STREAM()))
+                res = []
+                for _ in range(3):
+                    for i in range(sets):
+                        assert calls[i]() == 0
+                    torch.cuda.synchronize()
+                    ev = Events(lib, stream)
+                    ev.start()
+                    for i in range(launches):
+                        calls[i % sets]()
+                    res.append((n + 1) * numel * es / (ev.stop_ms() / launches) / 1e6 / HBM_PEAK_GBS)
+                cells.append(f"{sorted(res)[1]:.3f}")
+            print(f"| {str(dt)[6:]} | {n} | " + " | ".join(cells) + " |", flush=True)
+            del bufs, calls
+            torch.cuda.empty_cache()
+
+
 STRIDED_VIEWS_HEADER = """\
 # Strided pack / unpack of one column range: row length x alignment (MI355X)
 
@@ -1443,11 +1504,14 @@ def main():
     ap.add_argument("--all", action="store_true", help="also run every other workload with its own CPU leg; their lines go to stderr")
     ap.add_argument("--no-summary", action="store_true", help="leave out the `workloads` object of the default run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views", "bucket_sizes", "platform"], help="print a table instead of the bench line")
+    ap.add_argument("--sweep", choices=sorted(SWEEPS) + ["strided_views", "bucket_sizes", "platform", "reduce_ops"], help="print a table instead of the bench line")
     ap.add_argument("--dtypes", default="u8,bf16,f32,f64", help="element types of --sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.sweep == "reduce_ops":
+        sweep_reduce_ops()
+        return
     if args.sweep == "platform":
         sweep_platform()
         return
