@@ -4,6 +4,7 @@ switches kernels (tile, chunk, block and vector widths and their neighbours), bu
 zones either side of every buffer catch stray writes.  Each `*_case` function runs one case and raises AssertionError
 naming it; run as a program it repeats them for a number of seconds: python tests/fuzz_cases.py SECONDS SEED [pack|many|reduce|scatter|fp8 ...]."""
 import ctypes as C
+import math
 import os
 import random
 import sys
@@ -27,6 +28,7 @@ LENGTHS = [1, 2, 7, 8, 9, 15, 16, 17, 63, 64, 65, 255, 256, 257, 1000, 1023, 102
            8192, 8193, 16384, 65535, 65536, 65537, 262144 + 3, 1048576, 1048577]
 OPS = [(R.ReduceOp.Sum, oracle.SUM), (R.ReduceOp.Avg, oracle.AVG), (R.ReduceOp.Prod, oracle.PROD), (R.ReduceOp.Max, oracle.MAX),
        (R.ReduceOp.Min, oracle.MIN)]
+GROW = 0.0   # log2 of FUZZ_SCALE: stretches the log-uniform size draws of a long run
 FLOATS = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
 INTS = [torch.uint8, torch.int8, torch.int32, torch.int64]
 
@@ -51,7 +53,7 @@ def random_slice(gen, max_elems, max_span):
         ndim = gen.choice([1, 2, 2, 2, 3, 3, 4])
         sizes, total = [], 1
         for _ in range(ndim):
-            z = gen.choice(EXTENTS) if gen.random() < 0.5 else int(2 ** gen.uniform(0, 12.5))
+            z = gen.choice(EXTENTS) if gen.random() < 0.5 else int(2 ** gen.uniform(0, 12.5 + GROW / 2))
             z = max(1, min(z, max(1, max_elems // total)))
             sizes.append(z)
             total *= z
@@ -198,7 +200,7 @@ def _same(got, want, dtype):
 def reduce_case(gen, tag, max_numel=1 << 21):
     dtype = gen.choice(FLOATS + FLOATS + INTS)
     n = gen.choice([1, 2, 2, 3, 4, 5, 7, 8, 8, 8, 9, 12, 16, 17, 24])
-    numel = min(max_numel, gen.choice(LENGTHS) if gen.random() < 0.6 else int(2 ** gen.uniform(0, 21)))
+    numel = min(max_numel, gen.choice(LENGTHS) if gen.random() < 0.6 else int(2 ** gen.uniform(0, 21 + GROW)))
     op, code = gen.choice(OPS)
     if dtype in INTS and op == R.ReduceOp.Avg:
         op, code = OPS[0]
@@ -244,7 +246,7 @@ def scatter_case(gen, tag, max_len=1 << 18):
         op, code = OPS[0]
     es = torch.empty(0, dtype=dtype).element_size()
     if gen.random() < 0.5:
-        in_view, L = None, min(max_len, gen.choice(LENGTHS) if gen.random() < 0.5 else int(2 ** gen.uniform(3, 18)))
+        in_view, L = None, min(max_len, gen.choice(LENGTHS) if gen.random() < 0.5 else int(2 ** gen.uniform(3, 18 + GROW)))
         span, loc_in = L, None
     else:
         in_view, span, L = random_slice(gen, max_len, (16 << 20) // es)
@@ -382,11 +384,18 @@ CASES = {"pack": pack_case, "many": many_case, "reduce": reduce_case, "scatter":
 def long_run(seconds, seed, kinds):
     gen = random.Random(seed)
     t0, n = time.time(), {k: 0 for k in kinds}
+    global GROW
+    scale = int(os.environ.get("FUZZ_SCALE", "1"))   # FUZZ_SCALE=8: cases up to eight times as large (fewer of them per second)
+    GROW = math.log2(scale)
+    bounds = {"pack": dict(max_bytes=(6 << 20) * scale, max_span_bytes=(96 << 20) * scale),
+              "many": dict(max_bytes=(2 << 20) * scale, max_span_bytes=(24 << 20) * scale),
+              "reduce": dict(max_numel=(1 << 21) * scale), "scatter": dict(max_len=(1 << 18) * scale),
+              "fp8": dict(max_tensor=300000 * scale)}
     while time.time() - t0 < seconds:
         k = gen.choice(kinds)
         tag = f"seed {seed} case {sum(n.values())}"
         print(tag, k, flush=True)  # names the case before anything of it runs on the GPU
-        CASES[k](gen, tag)
+        CASES[k](gen, tag, **bounds[k])
         n[k] += 1
     print("ok:", ", ".join(f"{v} {k}" for k, v in n.items()), f"in {time.time() - t0:.0f} s, seed {seed}", flush=True)
 
